@@ -1,0 +1,123 @@
+"""Float64 brute-force statement of the pair-stack math.  TEST INFRASTRUCTURE ONLY.
+
+Written from the index formulas of the path (one Python loop per free index,
+numpy float64 dot products over the contracted one), deliberately sharing no
+code and no library routine (no layer_norm, no einsum, no softmax) with
+oracle/pairstack_oracle.py, so that a dropped term, a swapped index or a
+transposed operand in the oracle shows up as a mismatch.  Usable only for
+tiny N.
+
+Index formulas and where the reference states them:
+  LayerNorm              normalization.py:70-84   y = (x-mean)/sqrt(var_biased+eps)*w+b
+  a, b projections       tmu.py:487-493           a = mask * sigmoid(zn Wag^T) * (zn Wap^T)
+  outgoing contraction   tmu.py:77-79,95          x[i,j,c] = sum_k a[i,k,c] b[j,k,c]
+  incoming contraction   tmu.py:81-82,95          x[i,j,c] = sum_k a[k,i,c] b[k,j,c]
+  trimul output          tmu.py:498-501           (LN_out(x) Wz^T) * sigmoid(zn Wg^T)
+  attention logits       attention.py:123-127     s = q.k/sqrt(c) + inf*(mask-1) + tb
+  triangle bias          tri_att.py:137-140       tb[h,q,k] = (xn[q,k,:] Wz^T)[h]
+  gating / output        attention.py:288-302     (o*sigmoid(xn Wg^T)) Wo^T, channel = h*c+d
+"""
+
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+
+def _f64(t):
+    return np.asarray(t.detach().cpu().double().numpy() if hasattr(t, "detach") else t, dtype=np.float64)
+
+
+def _ln(v, w, b, eps=1e-5):
+    mu = v.sum() / v.size
+    var = ((v - mu) ** 2).sum() / v.size
+    return (v - mu) / math.sqrt(var + eps) * w + b
+
+
+def _sig(v):
+    return 1.0 / (1.0 + np.exp(-v))
+
+
+def trimul_update(z, mask, p, outgoing):
+    """z: [N, N, C], mask: [N, N] -> [N, N, C] float64."""
+    z = _f64(z)
+    mask = _f64(mask)
+    P = {k: _f64(v) for k, v in p.items()}
+    N, _, C = z.shape
+    Ch = P["linear_a_p.weight"].shape[0]
+    zn = np.zeros_like(z)
+    a = np.zeros((N, N, Ch))
+    b = np.zeros((N, N, Ch))
+    for i in range(N):
+        for j in range(N):
+            zn[i, j] = _ln(z[i, j], P["layer_norm_in.weight"], P["layer_norm_in.bias"])
+            a[i, j] = mask[i, j] * _sig(P["linear_a_g.weight"] @ zn[i, j]) * (P["linear_a_p.weight"] @ zn[i, j])
+            b[i, j] = mask[i, j] * _sig(P["linear_b_g.weight"] @ zn[i, j]) * (P["linear_b_p.weight"] @ zn[i, j])
+    out = np.zeros((N, N, C))
+    for i in range(N):
+        for j in range(N):
+            x = np.zeros(Ch)
+            for k in range(N):
+                if outgoing:
+                    x += a[i, k] * b[j, k]
+                else:
+                    x += a[k, i] * b[k, j]
+            xn = _ln(x, P["layer_norm_out.weight"], P["layer_norm_out.bias"])
+            out[i, j] = (P["linear_z.weight"] @ xn) * _sig(P["linear_g.weight"] @ zn[i, j])
+    return out
+
+
+def triattn_update(x, mask, p, no_heads, starting=True, inf=1e9):
+    """x: [I, J, C] (I == J), mask: [I, J] -> [I, J, C] float64.
+
+    The ending node is stated directly on the un-transposed tensor:
+    out[i,j] attends over k with q from x[i,j], k/v from x[k,j], key mask
+    mask[k,j] and triangle bias from x[k,i]  (tri_att.py:126-128,164-165).
+    """
+    x = _f64(x)
+    mask = _f64(mask)
+    P = {k: _f64(v) for k, v in p.items()}
+    N, _, C = x.shape
+    H = no_heads
+    Wq, Wk, Wv, Wg = (P["mha.linear_%s.weight" % n] for n in "qkvg")
+    Wo, Wb = P["mha.linear_o.weight"], P["linear_z.weight"]
+    c = Wq.shape[0] // H
+    xn = np.zeros_like(x)
+    for i in range(N):
+        for j in range(N):
+            xn[i, j] = _ln(x[i, j], P["layer_norm.weight"], P["layer_norm.bias"])
+    out = np.zeros((N, N, C))
+    for i in range(N):
+        for j in range(N):
+            qv = (Wq @ xn[i, j]) / math.sqrt(c)
+            gv = _sig(Wg @ xn[i, j])
+            o = np.zeros(H * c)
+            for h in range(H):
+                s = np.zeros(N)
+                vals = np.zeros((N, c))
+                for k in range(N):
+                    if starting:
+                        src, mk, bsrc = xn[i, k], mask[i, k], xn[j, k]
+                    else:
+                        src, mk, bsrc = xn[k, j], mask[k, j], xn[k, i]
+                    kv = (Wk @ src)[h * c:(h + 1) * c]
+                    vals[k] = (Wv @ src)[h * c:(h + 1) * c]
+                    qk = qv[h * c:(h + 1) * c] @ kv
+                    tb = (Wb @ bsrc)[h]
+                    if mk == 1.0:
+                        s[k] = qk + tb
+                    else:
+                        # The reference adds the mask bias to the logit first, then the
+                        # triangle bias (attention.py:126-127), in float32: -1e9 absorbs
+                        # any |logit| < 32 (ulp(1e9) = 64), which is what makes a fully
+                        # masked row a uniform average.  float64 would not absorb, so
+                        # these two adds are rounded to float32 here.
+                        t = np.float32(np.float32(qk) + np.float32(inf * (mk - 1.0)))
+                        s[k] = float(np.float32(t + np.float32(tb)))
+                s = s - s.max()
+                w = np.exp(s)
+                w = w / w.sum()
+                o[h * c:(h + 1) * c] = w @ vals
+            out[i, j] = Wo @ (o * gv)
+    return out

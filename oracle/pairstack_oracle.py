@@ -1,0 +1,274 @@
+"""CPU oracle for the OpenFold3 pair-stack hot path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, in plain fp32 PyTorch on the CPU, the arithmetic of the
+reference's stock (no alternative kernel) path through
+
+  * TriangleMultiplicativeUpdate.forward
+      openfold3/core/model/layers/triangular_multiplicative_update.py:482-503
+    with _combine_projections (same file, :71-97),
+  * TriangleAttention.forward
+      openfold3/core/model/layers/triangular_attention.py:102-167
+    with Attention._prep_qkv / _attention / _wrap_up
+      openfold3/core/model/primitives/attention.py:265-302, :94-135,
+  * PairBlock.tri_mul_out_in / tri_att_start_end
+      openfold3/core/model/latent/base_blocks.py:307-406,
+  * TemplatePairBlock.forward (per-template loop, tri_mul_first=True)
+      openfold3/core/model/latent/template_module.py:148-166.
+
+It may be imported by tests/, by __graft_entry__.smoke() and by the
+cpu_baseline leg of bench.py, as the checker or the timed CPU baseline.
+The shipped package never imports it.
+
+The library routines it calls (F.layer_norm, F.linear, torch.einsum,
+torch.softmax, torch.sigmoid) are the very routines the reference calls at
+normalization.py:70-84, linear.py:127-138, tmu.py:95, attention.py:86-133 and
+tmu.py:69.  The reference holds no golden vectors for this path; every
+function here is pinned by tests/test_oracle_pinning.py against
+oracle/brute_force.py (float64 explicit loops written from the index
+formulas), against torch's scaled_dot_product_attention, and against the
+algebraic invariants of the path.
+
+Parameters travel as a flat ``dict[str, Tensor]`` keyed exactly like the
+reference modules' state dicts (``layer_norm_in.weight``, ``linear_a_p.weight``,
+``mha.linear_q.weight`` ...), so a drop-in module's ``state_dict()`` can be
+handed to the oracle unchanged.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+LN_EPS = 1e-5  # normalization.py:36 (eps default)
+INF = 1e9  # triangular_attention.py:38
+
+
+# --------------------------------------------------------------------------
+# primitives
+# --------------------------------------------------------------------------
+def layer_norm(x, weight, bias, eps: float = LN_EPS):
+    """normalization.py:59-86: F.layer_norm over the last dim, affine."""
+    return F.layer_norm(x, (x.shape[-1],), weight.to(x.dtype), bias.to(x.dtype), eps)
+
+
+def linear(x, weight):
+    """linear.py:115-138 for a bias-free Linear: x @ W^T, W is [out, in]."""
+    return F.linear(x, weight.to(x.dtype))
+
+
+# --------------------------------------------------------------------------
+# triangle multiplicative update
+# --------------------------------------------------------------------------
+def trimul_contract(a, b, outgoing: bool):
+    """tmu.py:71-97.  a, b: [*, N, N, C] -> [*, N, N, C].
+
+    Follows the reference literally: permute to channel-major, one matrix
+    product per channel, permute back.
+    """
+    nd = a.dim()
+    lead = list(range(nd - 3))
+
+    def perm(t, inds):
+        return t.permute(lead + [nd - 3 + i for i in inds])
+
+    if outgoing:
+        a = perm(a, (2, 0, 1))
+        b = perm(b, (2, 1, 0))
+    else:
+        a = perm(a, (2, 1, 0))
+        b = perm(b, (2, 0, 1))
+    p = torch.einsum("...ij,...jk->...ik", a, b)
+    return perm(p, (1, 2, 0))
+
+
+def trimul_update(z, mask, p, outgoing: bool):
+    """tmu.py:482-503.  Returns the update only (the caller adds it to z)."""
+    if mask is None:
+        mask = z.new_ones(z.shape[:-1])
+    m = mask.to(z.dtype).unsqueeze(-1)
+    zn = layer_norm(z, p["layer_norm_in.weight"], p["layer_norm_in.bias"])
+    a = m
+    a = a * torch.sigmoid(linear(zn, p["linear_a_g.weight"]))
+    a = a * linear(zn, p["linear_a_p.weight"])
+    b = m
+    b = b * torch.sigmoid(linear(zn, p["linear_b_g.weight"]))
+    b = b * linear(zn, p["linear_b_p.weight"])
+    x = trimul_contract(a, b, outgoing)
+    del a, b
+    x = layer_norm(x, p["layer_norm_out.weight"], p["layer_norm_out.bias"])
+    x = linear(x, p["linear_z.weight"])
+    g = torch.sigmoid(linear(zn, p["linear_g.weight"]))
+    return x * g
+
+
+# --------------------------------------------------------------------------
+# triangle attention
+# --------------------------------------------------------------------------
+def attention_core(q, k, v, biases):
+    """attention.py:94-135.  q,k,v: [*, H, Q/K, c]; q already scaled."""
+    s = torch.einsum("...qc,...kc->...qk", q, k)
+    for bias in biases:
+        s = s + bias
+    s = torch.softmax(s, dim=-1)
+    return torch.einsum("...qk,...kc->...qc", s.to(v.dtype), v)
+
+
+def triattn_update(x, mask, p, no_heads: int, starting: bool = True, inf: float = INF,
+                   row_chunk: int | None = None):
+    """tri_att.py:102-167 + Attention.forward default branch (attention.py:366-413).
+
+    x: [*, I, J, C]; mask: [*, I, J].  Returns the update only.
+    ``row_chunk`` bounds the materialised logits by processing that many rows
+    of I at a time; it changes no value (rows are independent).
+    """
+    if mask is None:
+        mask = x.new_ones(x.shape[:-1])
+    if not starting:
+        x = x.transpose(-2, -3)
+        mask = mask.transpose(-1, -2)
+    xn = layer_norm(x, p["layer_norm.weight"], p["layer_norm.bias"])
+    mask_bias = (inf * (mask.to(x.dtype) - 1))[..., :, None, None, :]  # [*, I, 1, 1, J]
+    tb = linear(xn, p["linear_z.weight"])  # [*, I, J, H]
+    nd = tb.dim()
+    tb = tb.permute(list(range(nd - 3)) + [nd - 1, nd - 3, nd - 2])  # [*, H, I, J]
+    tb = tb.unsqueeze(-4)  # [*, 1, H, I, J]
+
+    H = no_heads
+    n_rows = xn.shape[-3]
+    step = n_rows if row_chunk is None else row_chunk
+    outs = []
+    for r0 in range(0, n_rows, step):
+        xr = xn[..., r0:r0 + step, :, :]
+        q = linear(xr, p["mha.linear_q.weight"])
+        k = linear(xr, p["mha.linear_k.weight"])
+        v = linear(xr, p["mha.linear_v.weight"])
+        c = q.shape[-1] // H
+        q = q.view(q.shape[:-1] + (H, c)).transpose(-2, -3)  # [*, I, H, J, c]
+        k = k.view(k.shape[:-1] + (H, c)).transpose(-2, -3)
+        v = v.view(v.shape[:-1] + (H, c)).transpose(-2, -3)
+        q = q / math.sqrt(c)  # attention.py:283-284
+        o = attention_core(q, k, v, [mask_bias[..., r0:r0 + step, :, :, :], tb])
+        o = o.transpose(-2, -3)  # [*, I, J, H, c]
+        g = torch.sigmoid(linear(xr, p["mha.linear_g.weight"]))
+        g = g.view(g.shape[:-1] + (H, c))
+        o = (o * g).reshape(o.shape[:-2] + (H * c,))
+        outs.append(linear(o, p["mha.linear_o.weight"]))
+    out = outs[0] if len(outs) == 1 else torch.cat(outs, dim=-3)
+    if not starting:
+        out = out.transpose(-2, -3)
+    return out
+
+
+# --------------------------------------------------------------------------
+# block sequencing
+# --------------------------------------------------------------------------
+def _sub(p, prefix):
+    n = len(prefix)
+    return {k[n:]: v for k, v in p.items() if k.startswith(prefix)}
+
+
+def pair_stack_block(z, pair_mask, p, no_heads: int, row_chunk: int | None = None):
+    """base_blocks.py:322-351 then :364-406 in eval mode (dropout = identity,
+    dropout.py:57-58), out of place.  The pair transition (:470-478) is not
+    part of this path.  ``p`` holds the four sub-modules under the reference's
+    prefixes tri_mul_out. / tri_mul_in. / tri_att_start. / tri_att_end.
+    """
+    z = z + trimul_update(z, pair_mask, _sub(p, "tri_mul_out."), outgoing=True)
+    z = z + trimul_update(z, pair_mask, _sub(p, "tri_mul_in."), outgoing=False)
+    z = z + triattn_update(z, pair_mask, _sub(p, "tri_att_start."), no_heads,
+                           starting=True, row_chunk=row_chunk)
+    # the reference builds tri_att_end as a *starting* module and transposes
+    # around the call (base_blocks.py:282-288, :380-404)
+    zt = z.transpose(-2, -3)
+    zt = zt + triattn_update(zt, pair_mask.transpose(-1, -2), _sub(p, "tri_att_end."),
+                             no_heads, starting=True, row_chunk=row_chunk)
+    return zt.transpose(-2, -3)
+
+
+def template_pair_stack(t, mask, blocks, no_heads: int, row_chunk: int | None = None):
+    """template_module.py:148-166 with tri_mul_first=True, for every block of
+    ``blocks`` in turn: each template is an independent pair representation.
+    t: [*, T, N, N, C]; mask: [*, T, N, N].  Pair transition and the final
+    LayerNorm of the stack are outside this path.
+    """
+    outs = []
+    for ti in range(t.shape[-4]):
+        zt = t[..., ti, :, :, :]
+        mt = mask[..., ti, :, :]
+        for p in blocks:
+            zt = pair_stack_block(zt, mt, p, no_heads, row_chunk=row_chunk)
+        outs.append(zt.unsqueeze(-4))
+    return torch.cat(outs, dim=-4)
+
+
+# --------------------------------------------------------------------------
+# seeded synthetic parameters / inputs (shared by tests, smoke and bench)
+# --------------------------------------------------------------------------
+def make_trimul_params(gen, c_z: int, c_hidden: int):
+    def lin(o, i):
+        return torch.randn(o, i, generator=gen) / math.sqrt(i)
+
+    return {
+        "layer_norm_in.weight": 1 + 0.1 * torch.randn(c_z, generator=gen),
+        "layer_norm_in.bias": 0.1 * torch.randn(c_z, generator=gen),
+        "layer_norm_out.weight": 1 + 0.1 * torch.randn(c_hidden, generator=gen),
+        "layer_norm_out.bias": 0.1 * torch.randn(c_hidden, generator=gen),
+        "linear_a_p.weight": lin(c_hidden, c_z),
+        "linear_a_g.weight": lin(c_hidden, c_z),
+        "linear_b_p.weight": lin(c_hidden, c_z),
+        "linear_b_g.weight": lin(c_hidden, c_z),
+        "linear_g.weight": lin(c_z, c_z),
+        "linear_z.weight": lin(c_z, c_hidden),
+    }
+
+
+def make_triattn_params(gen, c_in: int, c_head: int, no_heads: int):
+    def lin(o, i):
+        return torch.randn(o, i, generator=gen) / math.sqrt(i)
+
+    hc = c_head * no_heads
+    return {
+        "layer_norm.weight": 1 + 0.1 * torch.randn(c_in, generator=gen),
+        "layer_norm.bias": 0.1 * torch.randn(c_in, generator=gen),
+        "linear_z.weight": lin(no_heads, c_in),
+        "mha.linear_q.weight": lin(hc, c_in),
+        "mha.linear_k.weight": lin(hc, c_in),
+        "mha.linear_v.weight": lin(hc, c_in),
+        "mha.linear_g.weight": lin(hc, c_in),
+        "mha.linear_o.weight": lin(c_in, hc),
+    }
+
+
+def make_block_params(seed: int, c_z: int, c_hidden_mul: int, c_head: int, no_heads: int):
+    """Every hot-path Linear ~ N(0, 1/fan_in) (the reference's tests override
+    the zero 'final'/'gating' inits the same way, tests/test_kernels.py:381-385);
+    LayerNorm weight 1+0.1N, bias 0.1N so the affine terms are exercised."""
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    p = {}
+    for name, outgoing in (("tri_mul_out.", True), ("tri_mul_in.", False)):
+        for k, v in make_trimul_params(gen, c_z, c_hidden_mul).items():
+            p[name + k] = v
+    for name in ("tri_att_start.", "tri_att_end."):
+        for k, v in make_triattn_params(gen, c_z, c_head, no_heads).items():
+            p[name + k] = v
+    return p
+
+
+def make_pair_input(seed: int, batch_shape, n: int, c_z: int):
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    return torch.randn(*batch_shape, n, n, c_z, generator=gen)
+
+
+def tail_padding_mask(batch_shape, n: int, n_pad):
+    """pair_mask = outer(token_mask, token_mask) with the last n_pad tokens
+    zeroed.  n_pad may be an int or a tensor shaped like batch_shape."""
+    pad = torch.as_tensor(n_pad).expand(tuple(batch_shape)) if len(batch_shape) else torch.as_tensor(n_pad)
+    idx = torch.arange(n)
+    tok = (idx < (n - pad)[..., None]).to(torch.float32)
+    return tok[..., :, None] * tok[..., None, :]
+
+
+def round_bf16(t):
+    return t.to(torch.bfloat16).to(torch.float32)
