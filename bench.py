@@ -1,0 +1,208 @@
+"""Benchmark of the pair-stack block (triangle multiplication out + in, triangle attention
+start + end, residual adds fused) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--n 768] [--no-cpu]
+
+A step is one block forward, in place, on a z that already lives in HBM.  The workload is
+BASELINE config 3: N_token = 768, c_z = 128, c_hidden_mul = 128, 4 heads x 32, batch 1,
+all-ones mask, bf16, synthetic N(0,1) input and seeded random weights.  Prints one JSON line.
+
+Besides the whole-block time the line carries
+  roofline      the triangle-multiplication contraction (the MFMA-bound kernel the target
+                of >= 50 % of bf16 peak is set on): algorithmic 2*B*N^3*C_h flops over its
+                average launch duration, measured here with events on the launch stream;
+  kernels       the same figure for every kernel of the block, each against the roof that
+                bounds it (MFMA for the contraction and the attention core, HBM for the
+                LayerNorm/projection passes; algorithmic bytes per launch are listed in
+                KERNEL_MODEL below);
+  cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path)
+                timed once on the host cores for the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "openfold-3_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+METRIC = "ms per Pairformer pair-stack block at N=768 bf16; % of MFMA peak & HBM GB/s"
+
+
+def kernel_model(B, N, C, CH, H, D):
+    """Algorithmic work per launch.  U = one bf16 pass over z."""
+    U = B * N * N * C * 2
+    hd = H * D
+    return {
+        # reads z, writes a and b
+        "trimul_proj": {"bound": "hbm", "bytes": U + 2 * B * N * N * CH * 2 + B * N * N * 4},
+        # 2*B*N^3*C_h multiply-adds counted as 2 flops
+        "trimul_contract": {"bound": "mfma", "flops": 2 * B * N ** 3 * CH},
+        # reads x and z, writes out
+        "trimul_out": {"bound": "hbm", "bytes": B * N * N * CH * 2 + 2 * U},
+        # reads x, writes q, k, v (+ fp32 triangle bias and mask bias)
+        "triattn_proj": {"bound": "hbm", "bytes": U + 3 * B * N * N * hd * 2 + B * H * N * N * 4 + B * N * N * 4},
+        # QK^T and PV
+        "triattn_flash": {"bound": "mfma", "flops": 4 * B * N ** 3 * H * D},
+        # reads o and x, writes out
+        "triattn_out": {"bound": "hbm", "bytes": B * N * N * hd * 2 + 2 * U},
+    }
+
+
+def time_events(fn, steps, warmup, torch):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps  # ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--n", type=int, default=768, help="N_token (768 = the headline configuration)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--contract-variant", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build is single-GPU (one pair-stack block on one MI355X); run with --gpus 1")
+
+    import torch
+
+    from of3pair import _lib
+    from of3pair import build as of3_build
+
+    if not of3_build.is_built():
+        of3_build.build()
+    import of3pair
+    from oracle import pairstack_oracle as orc
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, N, C, CH, H, D = 1, args.n, 128, 128, 4, 32
+
+    params = {k: orc.round_bf16(v) for k, v in orc.make_block_params(0, C, CH, D, H).items()}
+    block = of3pair.PairStack(C, CH, D, H)
+    block.load_state_dict(params)
+    block = block.to(dev).to(torch.bfloat16).eval()
+    z_host = orc.round_bf16(orc.make_pair_input(1, (B,), N, C))
+    z = z_host.to(dev).to(torch.bfloat16)
+    mask = torch.ones(B, N, N, device=dev)
+
+    # ---- whole block, in place, inputs resident
+    def step():
+        block(z, mask, inplace_safe=True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- per-kernel durations through the stage entry points of the C ABI
+    lib = _lib.load()
+    s = torch.cuda.current_stream().cuda_stream
+    Np = lib.of3_padded_n(N)
+    bf = torch.bfloat16
+    zz = z_host.to(dev).to(bf)
+    zs = _lib.strides3(zz.stride()[:3])
+    ms_ = _lib.strides3(mask.stride())
+    tm = {k[len("tri_mul_out."):]: v.to(dev).to(bf).contiguous() for k, v in params.items() if k.startswith("tri_mul_out.")}
+    ta = {k[len("tri_att_start."):]: v.to(dev).to(bf).contiguous() for k, v in params.items() if k.startswith("tri_att_start.")}
+    a = torch.zeros(B, CH, Np, Np, dtype=bf, device=dev)
+    b = torch.zeros_like(a)
+    x = torch.zeros_like(a)
+    out = torch.empty_like(zz)
+    q = torch.zeros(B, N, H, Np, D, dtype=bf, device=dev)
+    k = torch.zeros_like(q)
+    vt = torch.zeros(B, N, H, D, Np, dtype=bf, device=dev)
+    tb = torch.zeros(B, H, N, Np, device=dev)
+    mb = torch.zeros(B, N, Np, device=dev)
+    o = torch.zeros(B, N, N, H * D, dtype=bf, device=dev)
+    P = lambda t: t.data_ptr()  # noqa: E731
+
+    def ck(st):
+        _lib.check(st, "bench stage")
+
+    stages = {
+        "trimul_proj": lambda: ck(lib.of3_trimul_proj(P(zz), zs, P(mask), ms_, P(tm["layer_norm_in.weight"]),
+                                                      P(tm["layer_norm_in.bias"]), P(tm["linear_a_p.weight"]),
+                                                      P(tm["linear_a_g.weight"]), P(tm["linear_b_p.weight"]),
+                                                      P(tm["linear_b_g.weight"]), P(a), P(b), B, N, C, CH, 1, s)),
+        "trimul_contract": lambda: ck(lib.of3_trimul_contract(P(a), P(b), P(x), B, N, CH, args.contract_variant, s)),
+        "trimul_out": lambda: ck(lib.of3_trimul_out(P(x), P(zz), zs, P(out), P(tm["layer_norm_in.weight"]),
+                                                    P(tm["layer_norm_in.bias"]), P(tm["layer_norm_out.weight"]),
+                                                    P(tm["layer_norm_out.bias"]), P(tm["linear_g.weight"]),
+                                                    P(tm["linear_z.weight"]), B, N, C, CH, 1, s)),
+        "triattn_proj": lambda: ck(lib.of3_triattn_proj(P(zz), zs, P(mask), ms_, P(ta["layer_norm.weight"]),
+                                                        P(ta["layer_norm.bias"]), P(ta["mha.linear_q.weight"]),
+                                                        P(ta["mha.linear_k.weight"]), P(ta["mha.linear_v.weight"]),
+                                                        P(ta["linear_z.weight"]), P(q), P(k), P(vt), P(tb), P(mb),
+                                                        B, N, C, H, D, 1e9, s)),
+        "triattn_flash": lambda: ck(lib.of3_triattn_flash(P(q), P(k), P(vt), P(tb), P(mb), P(o), B, N, H, D, s)),
+        "triattn_out": lambda: ck(lib.of3_triattn_out(P(o), P(zz), zs, P(out), P(ta["layer_norm.weight"]),
+                                                      P(ta["layer_norm.bias"]), P(ta["mha.linear_g.weight"]),
+                                                      P(ta["mha.linear_o.weight"]), B, N, C, H, D, 1, s)),
+    }
+    model = kernel_model(B, N, C, CH, H, D)
+    kernels = {}
+    for name, fn in stages.items():
+        ms = time_events(fn, max(args.steps, 10), max(args.warmup, 3), torch)
+        m = model[name]
+        if m["bound"] == "mfma":
+            ach = m["flops"] / (ms * 1e-3) / 1e12
+            kernels[name] = {"bound": "mfma", "ms": round(ms, 4), "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
+                             "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4)}
+        else:
+            ach = m["bytes"] / (ms * 1e-3) / 1e9
+            kernels[name] = {"bound": "hbm", "ms": round(ms, 4), "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
+                             "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4)}
+    dom = kernels["trimul_contract"]
+    roofline = {"kernel": "trimul_contract", "bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": dom["frac"], "traffic": None}
+
+    # ---- CPU baseline: the oracle on the host cores, one block of the same workload
+    cpu = None
+    if not args.no_cpu:
+        torch.set_num_threads(os.cpu_count() or 1)
+        mask_h = torch.ones(B, N, N)
+        t0 = time.perf_counter()
+        with torch.no_grad():
+            orc.pair_stack_block(z_host, mask_h, params, H, row_chunk=32)
+        cpu_ms = (time.perf_counter() - t0) * 1e3
+        cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": "1 block forward, fp32, N=%d, same weights and input (tri-attn in 32-row chunks)" % N}
+
+    line = {
+        "metric": METRIC, "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "pair-stack block (trimul out+in, tri-attn start+end, residuals), B=1, N_token=%d, "
+                               "c_z=128, c_hidden_mul=128, 4 heads x 32, all-ones mask" % N},
+        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

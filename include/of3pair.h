@@ -1,0 +1,130 @@
+/* libof3pair: MI355X (gfx950) kernels for the OpenFold3 Pairformer pair stack.
+ *
+ * C ABI.  Every pointer is a DEVICE pointer owned by the caller (16-byte aligned), every
+ * tensor is bf16 unless stated otherwise, `stream` is a hipStream_t passed as void*.
+ * Calls only enqueue work on `stream`; they never allocate, free or synchronise, and keep
+ * no state between calls (apart from a per-thread "last HIP error" code and launch
+ * geometry cached per process).  Return value: OF3_OK or a negative of3_status.
+ *
+ * Reference interfaces these entry points stand in for (paths under the reference tree):
+ *   openfold3/core/model/layers/triangular_multiplicative_update.py
+ *       :421-503  TriangleMultiplicativeUpdate.forward          -> of3_trimul_fwd
+ *       :689-741  _cueq_triangle_mult (the existing fused-kernel operator boundary:
+ *                 z, mask, norm_in/out weight+bias, the gate/projection weights,
+ *                 direction, returns the update)                -> of3_trimul_fwd
+ *       :485-493  LayerNorm + gated a/b projections             -> of3_trimul_proj
+ *       :71-97    _combine_projections                          -> of3_trimul_contract
+ *       :498-501  LayerNorm_out, linear_z, gate                 -> of3_trimul_out
+ *   openfold3/core/model/layers/triangular_attention.py
+ *       :102-167  TriangleAttention.forward                     -> of3_triattn_fwd
+ *       :131-140  LayerNorm, mask bias, triangle bias           -> of3_triattn_proj
+ *   openfold3/core/model/primitives/attention.py
+ *       :265-286  Attention._prep_qkv                           -> of3_triattn_proj
+ *       :625-672  _cueq_triangle_attn (q,k,v [B,I,H,J,c], triangle bias, boolean mask,
+ *                 scale) / :94-135 _attention                   -> of3_triattn_flash
+ *       :288-302  Attention._wrap_up (gate, linear_o)           -> of3_triattn_out
+ *   openfold3/core/model/latent/base_blocks.py
+ *       :329-335  "z = z + update" after each module            -> add_residual = 1
+ *
+ * Shapes: B batch (templates are folded into B), N tokens, C = c_z, CH = c_hidden of the
+ * triangle multiplication, H heads of per-head width D.  Supported: (C, CH) in
+ * {(128,128), (64,64)}; H = 4 with (C, D) in {(128,32), (64,16)}; any N >= 1.
+ * NP = of3_padded_n(N) = N rounded up to a multiple of 128 is the leading dimension of
+ * the intermediate buffers.
+ *
+ * Pair tensors are addressed by element strides {stride_b, stride_i, stride_j} with a
+ * channel stride of 1; strides must be multiples of 8.  A transposed view (the
+ * ending-node attention of base_blocks.py:380-404, tri_att.py:126-128) is expressed by
+ * swapping stride_i and stride_j, no copy is needed.  Masks are fp32 [B,N,N] with their
+ * own element strides; a null mask means all ones (tmu.py:482-483, tri_att.py:120-124).
+ */
+#ifndef OF3PAIR_H
+#define OF3PAIR_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  OF3_OK = 0,
+  OF3_EINVAL = -1, /* bad shape, stride, alignment, dtype or null pointer */
+  OF3_ENOSPC = -2, /* workspace too small */
+  OF3_EHIP = -3    /* HIP launch error; code via of3_last_hip_error() */
+} of3_status;
+
+typedef enum { OF3_DTYPE_F32 = 0, OF3_DTYPE_BF16 = 1 } of3_dtype;
+
+int of3_version(void);
+/* HIP error code of the last OF3_EHIP on the calling thread (0 if none). */
+int of3_last_hip_error(void);
+const char* of3_status_string(int status);
+int64_t of3_padded_n(int64_t n);
+
+/* ---- triangle multiplicative update ------------------------------------------------ */
+
+/* Bytes of scratch of3_trimul_fwd needs: a, b, x = 3 * B*CH*NP*NP bf16. */
+int64_t of3_trimul_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t CH);
+
+/* a, b [B][CH][NP][NP]: gated, masked projections, channel-major and contiguous along
+ * the contracted index: a[b][c][i][k] = a_ref[b,i,k,c] (outgoing) or a_ref[b,k,i,c]
+ * (incoming); entries with k >= N are zero, rows i >= N are left untouched. */
+int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
+                    const void* ln_in_w, const void* ln_in_b, const void* w_a_p, const void* w_a_g,
+                    const void* w_b_p, const void* w_b_g, void* a, void* b, int64_t B, int64_t N, int64_t C,
+                    int64_t CH, int outgoing, void* stream);
+
+/* x[b][c][i][j] = sum_k a[b][c][i][k] * b[b][c][j][k]  over the padded planes.
+ * variant: 0 = automatic, 1/2/3 = 128x128 / 256x128 / 256x256 work-group tile. */
+int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
+                        void* stream);
+
+/* out = [z +] (LN_out(x) Wz^T) * sigmoid(LN_in(z) Wg^T); out uses z's strides. */
+int of3_trimul_out(const void* x, const void* z, const int64_t z_strides[3], void* out, const void* ln_in_w,
+                   const void* ln_in_b, const void* ln_out_w, const void* ln_out_b, const void* w_g,
+                   const void* w_z, int64_t B, int64_t N, int64_t C, int64_t CH, int add_residual, void* stream);
+
+/* The whole module: the three kernels above on `workspace`.  out may alias z only when
+ * add_residual is set or the caller no longer needs z (each position is read before it is
+ * written, by the same work-group). */
+int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
+                   const void* ln_in_w, const void* ln_in_b, const void* ln_out_w, const void* ln_out_b,
+                   const void* w_a_p, const void* w_a_g, const void* w_b_p, const void* w_b_g, const void* w_g,
+                   const void* w_z, void* out, int64_t B, int64_t N, int64_t C, int64_t CH, int outgoing,
+                   int add_residual, void* workspace, int64_t workspace_bytes, int dtype, void* stream);
+
+/* ---- triangle attention ------------------------------------------------------------- */
+
+/* Scratch of of3_triattn_fwd, in this order, each part 256-byte aligned:
+ *   q, k  [B][N][H][NP][D] bf16      vt [B][N][H][D][NP] bf16
+ *   tbias [B][H][N][NP] fp32         mbias [B][N][NP] fp32       o [B][N][N][H*D] bf16 */
+int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D);
+
+/* q is pre-multiplied by log2(e)/sqrt(D); tbias and mbias by log2(e); mbias is -inf for
+ * j >= N.  (i, j) are the module's frame as given by x_strides / mask_strides. */
+int of3_triattn_proj(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
+                     const void* ln_w, const void* ln_b, const void* w_q, const void* w_k, const void* w_v,
+                     const void* w_bias, void* q, void* k, void* vt, float* tbias, float* mbias, int64_t B,
+                     int64_t N, int64_t C, int64_t H, int64_t D, float inf, void* stream);
+
+/* o[b][i][q][h*D+d] = softmax_k(q.k + mbias[i][k] + tbias[h][q][k]) v, base-2 logits. */
+int of3_triattn_flash(const void* q, const void* k, const void* vt, const float* tbias, const float* mbias, void* o,
+                      int64_t B, int64_t N, int64_t H, int64_t D, void* stream);
+
+/* out = [x +] (o * sigmoid(LN(x) Wg^T)) Wo^T; out uses x's strides. */
+int of3_triattn_out(const void* o, const void* x, const int64_t x_strides[3], void* out, const void* ln_w,
+                    const void* ln_b, const void* w_g, const void* w_o, int64_t B, int64_t N, int64_t C, int64_t H,
+                    int64_t D, int add_residual, void* stream);
+
+int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
+                    const void* ln_w, const void* ln_b, const void* w_bias, const void* w_q, const void* w_k,
+                    const void* w_v, const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C,
+                    int64_t H, int64_t D, float inf, int add_residual, void* workspace, int64_t workspace_bytes,
+                    int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* OF3PAIR_H */

@@ -1,0 +1,87 @@
+// Internal launch interface between the C-ABI layer (of3pair_api.hip) and the kernels.
+// Every launcher validates nothing: the ABI layer has already checked shapes, and each
+// launcher only enqueues work on `stream` and returns hipGetLastError().
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace of3 {
+
+typedef uint16_t bf16_t;
+
+// Pair tensor addressing shared by the position-wise kernels.  A "row" r and a position
+// k along the tile axis address z[b][r][k] at  b*stride_b + r*stride_r + k*stride_k
+// (elements).  Swapping stride_r/stride_k walks the transposed tensor, which is how the
+// incoming update and the ending-node attention run without a physical transpose.
+struct PairView {
+  int64_t stride_b, stride_r, stride_k;
+};
+
+struct TrimulProjArgs {
+  const bf16_t* z;
+  const float* mask;  // may be null (all ones); addressed with mask_view (channel-less)
+  PairView z_view, mask_view;
+  const bf16_t *ln_w, *ln_b;                  // [C]
+  const bf16_t *w_ap, *w_ag, *w_bp, *w_bg;    // [CH][C]
+  bf16_t *a, *b;                              // [B][CH][Np][Np]
+  int B, N, Np;
+};
+hipError_t trimul_proj_launch(const TrimulProjArgs& args, int C, int CH, hipStream_t stream);
+
+// variant: 1 = 128x128, 2 = 256x128, 3 = 256x256 work-group tile
+hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
+                                  hipStream_t stream);
+
+struct TrimulOutArgs {
+  const bf16_t* x;  // [B][CH][Np][Np]
+  const bf16_t* z;  // gate input (and residual)
+  bf16_t* out;      // same addressing as z
+  PairView z_view;  // canonical orientation (i, j): x is direction-agnostic
+  const bf16_t *ln_in_w, *ln_in_b;    // [C]
+  const bf16_t *ln_out_w, *ln_out_b;  // [CH]
+  const bf16_t *w_g;                  // [C][C]
+  const bf16_t *w_z;                  // [C][CH]
+  int B, N, Np;
+  int add_residual;
+};
+hipError_t trimul_out_launch(const TrimulOutArgs& args, int C, int CH, hipStream_t stream);
+
+struct TriattnProjArgs {
+  const bf16_t* x;    // pair tensor, addressed with x_view in the module's (I, J) frame
+  const float* mask;  // may be null
+  PairView x_view, mask_view;
+  const bf16_t *ln_w, *ln_b;          // [C]
+  const bf16_t *w_q, *w_k, *w_v;      // [H*D][C]
+  const bf16_t *w_b;                  // [H][C]   (linear_z: triangle bias)
+  bf16_t *q, *k;                      // [B][N][H][Jp][D]
+  bf16_t *vt;                         // [B][N][H][D][Jp]
+  float *tbias;                       // [B][H][N][Jp]   (pre-multiplied by log2 e)
+  float *mbias;                       // [B][N][Jp]      (log2 e * inf * (mask-1); -inf for j >= N)
+  int B, N, Jp, H;
+  float inf;
+};
+hipError_t triattn_proj_launch(const TriattnProjArgs& args, int C, int D, hipStream_t stream);
+
+struct TriattnFlashArgs {
+  const bf16_t *q, *k, *vt;
+  const float *tbias, *mbias;
+  bf16_t* o;  // [B][N][N][H*D]  (module frame, channel = h*D + d)
+  int B, N, Jp, H;
+};
+hipError_t triattn_flash_launch(const TriattnFlashArgs& args, int D, hipStream_t stream);
+
+struct TriattnOutArgs {
+  const bf16_t* o;   // [B][N][N][H*D]
+  const bf16_t* x;   // module input (gate input and residual), x_view addressing
+  bf16_t* out;       // x_view addressing
+  PairView x_view;
+  const bf16_t *ln_w, *ln_b;  // [C]
+  const bf16_t *w_g;          // [H*D][C]
+  const bf16_t *w_o;          // [C][H*D]
+  int B, N;
+  int add_residual;
+};
+hipError_t triattn_out_launch(const TriattnOutArgs& args, int C, int HD, hipStream_t stream);
+
+}  // namespace of3

@@ -1,0 +1,291 @@
+// C-ABI layer of libof3pair: argument validation, workspace carving, kernel sequencing.
+// The contract of every entry point is stated in include/of3pair.h.
+#include "../../include/of3pair.h"
+
+#include <hip/hip_runtime.h>
+
+#include "of3_kernels.h"
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+inline int fail_hip(hipError_t e) {
+  g_last_hip_error = (int)e;
+  return OF3_EHIP;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int64_t align256(int64_t n) { return (n + 255) & ~(int64_t)255; }
+inline int64_t padded(int64_t n) { return (n + 127) / 128 * 128; }
+
+inline bool trimul_dims_ok(int64_t B, int64_t N, int64_t C, int64_t CH) {
+  if (B < 1 || N < 1 || N > (1 << 20)) return false;
+  return (C == 128 && CH == 128) || (C == 64 && CH == 64);
+}
+inline bool triattn_dims_ok(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
+  if (B < 1 || N < 1 || N > (1 << 20)) return false;
+  if (B * H > 65535 || (N + 3) / 4 > 65535) return false;
+  return H == 4 && ((C == 128 && D == 32) || (C == 64 && D == 16));
+}
+inline bool strides_ok(const int64_t s[3]) {
+  return s && s[0] >= 0 && s[1] > 0 && s[2] > 0 && (s[0] % 8 == 0) && (s[1] % 8 == 0) && (s[2] % 8 == 0);
+}
+inline bool mask_ok(const float* mask, const int64_t s[3]) {
+  if (!mask) return true;
+  return s && s[0] >= 0 && s[1] >= 0 && s[2] >= 0;
+}
+
+inline of3::PairView view(const int64_t s[3], bool swap) {
+  of3::PairView v;
+  v.stride_b = s[0];
+  v.stride_r = swap ? s[2] : s[1];
+  v.stride_k = swap ? s[1] : s[2];
+  return v;
+}
+inline of3::PairView mask_view(const float* mask, const int64_t s[3], bool swap) {
+  of3::PairView v = {0, 0, 0};
+  if (mask) v = view(s, swap);
+  return v;
+}
+
+inline const of3::bf16_t* bf(const void* p) { return static_cast<const of3::bf16_t*>(p); }
+inline of3::bf16_t* bf(void* p) { return static_cast<of3::bf16_t*>(p); }
+
+inline int contract_variant_auto(int64_t Np) {
+  // 256x128 tiles divide N = 768 into 9 full waves over 256 CUs; small problems keep the
+  // 128x128 tile so that every CU still gets work.
+  return Np >= 512 ? 2 : 1;
+}
+
+}  // namespace
+
+extern "C" {
+
+int of3_version(void) { return 1; }
+int of3_last_hip_error(void) { return g_last_hip_error; }
+
+const char* of3_status_string(int status) {
+  switch (status) {
+    case OF3_OK:
+      return "ok";
+    case OF3_EINVAL:
+      return "invalid argument (shape, stride, alignment, dtype or null pointer)";
+    case OF3_ENOSPC:
+      return "workspace too small";
+    case OF3_EHIP:
+      return "HIP error (see of3_last_hip_error)";
+    default:
+      return "unknown status";
+  }
+}
+
+int64_t of3_padded_n(int64_t n) { return n < 1 ? 0 : padded(n); }
+
+int64_t of3_trimul_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t CH) {
+  if (!trimul_dims_ok(B, N, C, CH)) return OF3_EINVAL;
+  const int64_t Np = padded(N);
+  return 3 * align256(B * CH * Np * Np * 2);
+}
+
+int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
+                    const void* ln_in_w, const void* ln_in_b, const void* w_a_p, const void* w_a_g,
+                    const void* w_b_p, const void* w_b_g, void* a, void* b, int64_t B, int64_t N, int64_t C,
+                    int64_t CH, int outgoing, void* stream) {
+  if (!trimul_dims_ok(B, N, C, CH) || !strides_ok(z_strides) || !mask_ok(mask, mask_strides)) return OF3_EINVAL;
+  const void* ptrs[] = {z, ln_in_w, ln_in_b, w_a_p, w_a_g, w_b_p, w_b_g, a, b};
+  for (const void* p : ptrs)
+    if (!p || !aligned16(p)) return OF3_EINVAL;
+  of3::TrimulProjArgs args;
+  args.z = bf(z);
+  args.mask = mask;
+  args.z_view = view(z_strides, !outgoing);
+  args.mask_view = mask_view(mask, mask_strides, !outgoing);
+  args.ln_w = bf(ln_in_w);
+  args.ln_b = bf(ln_in_b);
+  args.w_ap = bf(w_a_p);
+  args.w_ag = bf(w_a_g);
+  args.w_bp = bf(w_b_p);
+  args.w_bg = bf(w_b_g);
+  args.a = bf(a);
+  args.b = bf(b);
+  args.B = (int)B;
+  args.N = (int)N;
+  args.Np = (int)padded(N);
+  hipError_t e = of3::trimul_proj_launch(args, (int)C, (int)CH, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
+int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
+                        void* stream) {
+  if (B < 1 || N < 1 || (CH != 128 && CH != 64) || variant < 0 || variant > 3) return OF3_EINVAL;
+  if (!a || !b || !x || !aligned16(a) || !aligned16(b) || !aligned16(x)) return OF3_EINVAL;
+  const int64_t Np = padded(N);
+  if (variant == 0) variant = contract_variant_auto(Np);
+  hipError_t e = of3::trimul_contract_launch(bf(a), bf(b), bf(x), (int)(B * CH), (int)Np, variant,
+                                             static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
+int of3_trimul_out(const void* x, const void* z, const int64_t z_strides[3], void* out, const void* ln_in_w,
+                   const void* ln_in_b, const void* ln_out_w, const void* ln_out_b, const void* w_g,
+                   const void* w_z, int64_t B, int64_t N, int64_t C, int64_t CH, int add_residual, void* stream) {
+  if (!trimul_dims_ok(B, N, C, CH) || !strides_ok(z_strides)) return OF3_EINVAL;
+  const void* ptrs[] = {x, z, out, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_g, w_z};
+  for (const void* p : ptrs)
+    if (!p || !aligned16(p)) return OF3_EINVAL;
+  of3::TrimulOutArgs args;
+  args.x = bf(x);
+  args.z = bf(z);
+  args.out = bf(out);
+  args.z_view = view(z_strides, false);
+  args.ln_in_w = bf(ln_in_w);
+  args.ln_in_b = bf(ln_in_b);
+  args.ln_out_w = bf(ln_out_w);
+  args.ln_out_b = bf(ln_out_b);
+  args.w_g = bf(w_g);
+  args.w_z = bf(w_z);
+  args.B = (int)B;
+  args.N = (int)N;
+  args.Np = (int)padded(N);
+  args.add_residual = add_residual ? 1 : 0;
+  hipError_t e = of3::trimul_out_launch(args, (int)C, (int)CH, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
+int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
+                   const void* ln_in_w, const void* ln_in_b, const void* ln_out_w, const void* ln_out_b,
+                   const void* w_a_p, const void* w_a_g, const void* w_b_p, const void* w_b_g, const void* w_g,
+                   const void* w_z, void* out, int64_t B, int64_t N, int64_t C, int64_t CH, int outgoing,
+                   int add_residual, void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
+  if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
+  if (!trimul_dims_ok(B, N, C, CH)) return OF3_EINVAL;
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OF3_EINVAL;
+  if (workspace_bytes < of3_trimul_workspace_bytes(B, N, C, CH)) return OF3_ENOSPC;
+  const int64_t Np = padded(N);
+  const int64_t part = align256(B * CH * Np * Np * 2);
+  char* ws = static_cast<char*>(workspace);
+  void* a = ws;
+  void* b = ws + part;
+  void* x = ws + 2 * part;
+  int st = of3_trimul_proj(z, z_strides, mask, mask_strides, ln_in_w, ln_in_b, w_a_p, w_a_g, w_b_p, w_b_g, a, b, B, N,
+                           C, CH, outgoing, stream);
+  if (st != OF3_OK) return st;
+  st = of3_trimul_contract(a, b, x, B, N, CH, 0, stream);
+  if (st != OF3_OK) return st;
+  return of3_trimul_out(x, z, z_strides, out, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_g, w_z, B, N, C, CH,
+                        add_residual, stream);
+}
+
+int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
+  if (!triattn_dims_ok(B, N, C, H, D)) return OF3_EINVAL;
+  const int64_t Np = padded(N);
+  const int64_t qkv = align256(B * N * H * Np * D * 2);
+  return 3 * qkv + align256(B * H * N * Np * 4) + align256(B * N * Np * 4) + align256(B * N * N * H * D * 2);
+}
+
+int of3_triattn_proj(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
+                     const void* ln_w, const void* ln_b, const void* w_q, const void* w_k, const void* w_v,
+                     const void* w_bias, void* q, void* k, void* vt, float* tbias, float* mbias, int64_t B,
+                     int64_t N, int64_t C, int64_t H, int64_t D, float inf, void* stream) {
+  if (!triattn_dims_ok(B, N, C, H, D) || !strides_ok(x_strides) || !mask_ok(mask, mask_strides)) return OF3_EINVAL;
+  const void* ptrs[] = {x, ln_w, ln_b, w_q, w_k, w_v, w_bias, q, k, vt, tbias, mbias};
+  for (const void* p : ptrs)
+    if (!p || !aligned16(p)) return OF3_EINVAL;
+  of3::TriattnProjArgs args;
+  args.x = bf(x);
+  args.mask = mask;
+  args.x_view = view(x_strides, false);
+  args.mask_view = mask_view(mask, mask_strides, false);
+  args.ln_w = bf(ln_w);
+  args.ln_b = bf(ln_b);
+  args.w_q = bf(w_q);
+  args.w_k = bf(w_k);
+  args.w_v = bf(w_v);
+  args.w_b = bf(w_bias);
+  args.q = bf(q);
+  args.k = bf(k);
+  args.vt = bf(vt);
+  args.tbias = tbias;
+  args.mbias = mbias;
+  args.B = (int)B;
+  args.N = (int)N;
+  args.Jp = (int)padded(N);
+  args.H = (int)H;
+  args.inf = inf;
+  hipError_t e = of3::triattn_proj_launch(args, (int)C, (int)D, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
+int of3_triattn_flash(const void* q, const void* k, const void* vt, const float* tbias, const float* mbias, void* o,
+                      int64_t B, int64_t N, int64_t H, int64_t D, void* stream) {
+  const int64_t C = (D == 32) ? 128 : 64;
+  if (!triattn_dims_ok(B, N, C, H, D)) return OF3_EINVAL;
+  const void* ptrs[] = {q, k, vt, tbias, mbias, o};
+  for (const void* p : ptrs)
+    if (!p || !aligned16(p)) return OF3_EINVAL;
+  of3::TriattnFlashArgs args;
+  args.q = bf(q);
+  args.k = bf(k);
+  args.vt = bf(vt);
+  args.tbias = tbias;
+  args.mbias = mbias;
+  args.o = bf(o);
+  args.B = (int)B;
+  args.N = (int)N;
+  args.Jp = (int)padded(N);
+  args.H = (int)H;
+  hipError_t e = of3::triattn_flash_launch(args, (int)D, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
+int of3_triattn_out(const void* o, const void* x, const int64_t x_strides[3], void* out, const void* ln_w,
+                    const void* ln_b, const void* w_g, const void* w_o, int64_t B, int64_t N, int64_t C, int64_t H,
+                    int64_t D, int add_residual, void* stream) {
+  if (!triattn_dims_ok(B, N, C, H, D) || !strides_ok(x_strides)) return OF3_EINVAL;
+  const void* ptrs[] = {o, x, out, ln_w, ln_b, w_g, w_o};
+  for (const void* p : ptrs)
+    if (!p || !aligned16(p)) return OF3_EINVAL;
+  of3::TriattnOutArgs args;
+  args.o = bf(o);
+  args.x = bf(x);
+  args.out = bf(out);
+  args.x_view = view(x_strides, false);
+  args.ln_w = bf(ln_w);
+  args.ln_b = bf(ln_b);
+  args.w_g = bf(w_g);
+  args.w_o = bf(w_o);
+  args.B = (int)B;
+  args.N = (int)N;
+  args.add_residual = add_residual ? 1 : 0;
+  hipError_t e = of3::triattn_out_launch(args, (int)C, (int)(H * D), static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
+int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
+                    const void* ln_w, const void* ln_b, const void* w_bias, const void* w_q, const void* w_k,
+                    const void* w_v, const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C,
+                    int64_t H, int64_t D, float inf, int add_residual, void* workspace, int64_t workspace_bytes,
+                    int dtype, void* stream) {
+  if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
+  if (!triattn_dims_ok(B, N, C, H, D)) return OF3_EINVAL;
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OF3_EINVAL;
+  if (workspace_bytes < of3_triattn_workspace_bytes(B, N, C, H, D)) return OF3_ENOSPC;
+  const int64_t Np = padded(N);
+  const int64_t qkv = align256(B * N * H * Np * D * 2);
+  char* ws = static_cast<char*>(workspace);
+  void* q = ws;
+  void* k = ws + qkv;
+  void* vt = ws + 2 * qkv;
+  float* tbias = reinterpret_cast<float*>(ws + 3 * qkv);
+  float* mbias = reinterpret_cast<float*>(ws + 3 * qkv + align256(B * H * N * Np * 4));
+  void* o = ws + 3 * qkv + align256(B * H * N * Np * 4) + align256(B * N * Np * 4);
+  int st = of3_triattn_proj(x, x_strides, mask, mask_strides, ln_w, ln_b, w_q, w_k, w_v, w_bias, q, k, vt, tbias,
+                            mbias, B, N, C, H, D, inf, stream);
+  if (st != OF3_OK) return st;
+  st = of3_triattn_flash(q, k, vt, tbias, mbias, o, B, N, H, D, stream);
+  if (st != OF3_OK) return st;
+  return of3_triattn_out(o, x, x_strides, out, ln_w, ln_b, w_g, w_o, B, N, C, H, D, add_residual, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,234 @@
+// Triangle-attention input pass: xn = LayerNorm(x), then
+//     q = (xn Wq^T) * log2(e)/sqrt(D),  k = xn Wk^T,  v = xn Wv^T     (attention.py:265-286)
+//     triangle bias tb[h][q][k] = log2(e) * (xn[q][k] . Wb[h])          (tri_att.py:137-140)
+//     mask bias     mb[i][k]    = log2(e) * inf * (mask[i][k] - 1)      (tri_att.py:134)
+// written in the layouts the flash kernel consumes: q, k as [b][i][h][j][d]; v transposed
+// as [b][i][h][d][j]; tb as [b][h][i][j] and mb as [b][i][j] in fp32.  log2(e) is folded
+// in so the softmax can use the hardware base-2 exponential.  The PairView makes (i, j)
+// walk either the tensor itself (starting node) or its transpose (ending node).
+//
+// HBM bound (reads x once, writes q, k, v once).  Same structure as the
+// triangle-multiplication input pass: weights resident in registers as MFMA A operands,
+// 128-position tiles normalised in registers and staged once in LDS.
+#include "of3_device.h"
+#include "of3_kernels.h"
+
+namespace of3 {
+
+namespace {
+
+template <int C, int D>
+__global__ __launch_bounds__(256) void triattn_proj_kernel(TriattnProjArgs p, int tiles_per_row, int total_tiles) {
+  constexpr int H = 4;
+  constexpr int HD = H * D;
+  constexpr int NCH = C / 8;
+  constexpr int LPP = NCH;
+  constexpr int PPI = 64 / LPP;
+  constexpr int TP = 128;
+  constexpr int LN_ITERS = 32 / PPI;
+  constexpr int KS = C / 16;
+  constexpr int NT = HD / 32;          // 32-row output tiles per matrix (4 or 2)
+  constexpr bool WIDE = (NT == 4);     // HD = 128: wave w owns tile w of q, k and v
+  constexpr int NJ = WIDE ? 3 : 2;     // HD = 64: wave m (< 3) owns both tiles of matrix m
+  static_assert(NT == 4 || NT == 2, "H*D must be 128 or 64");
+
+  __shared__ u32x4_t tile[TP * NCH];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int ln_chunk = lane % LPP, ln_pp = lane / LPP;
+
+  float lw[8], lb[8];
+  load_affine8(p.ln_w, ln_chunk, lw);
+  load_affine8(p.ln_b, ln_chunk, lb);
+
+  const bool has_jobs = WIDE || wave < 3;
+  // job jj of this wave: matrix (0 q, 1 k, 2 v) and output tile
+  auto job_matrix = [&](int jj) { return WIDE ? jj : wave; };
+  auto job_tile = [&](int jj) { return WIDE ? wave : jj; };
+
+  u32x4_t wj[NJ][KS];
+#pragma unroll
+  for (int jj = 0; jj < NJ; ++jj) {
+    const int m = job_matrix(jj), ot = job_tile(jj);
+    const bf16_t* W = (m == 0) ? p.w_q : (m == 1 ? p.w_k : p.w_v);
+    // q, k: lane owns 16 consecutive channels (rowperm16); v: natural rows
+    const int row = 32 * ot + ((m == 2) ? l32 : rowperm16(l32));
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      u32x4_t w = {0u, 0u, 0u, 0u};
+      if (has_jobs) w = *reinterpret_cast<const u32x4_t*>(W + row * C + 16 * s + 8 * lh);
+      wj[jj][s] = w;
+    }
+  }
+  // triangle-bias weights: A rows 0..H-1 hold Wb, the rest are zero
+  u32x4_t wb[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    u32x4_t w = {0u, 0u, 0u, 0u};
+    if (l32 < H) w = *reinterpret_cast<const u32x4_t*>(p.w_b + l32 * C + 16 * s + 8 * lh);
+    wb[s] = w;
+  }
+  const float qscale = kLog2e * __builtin_amdgcn_rsqf((float)D);
+
+  const int N = p.N, Jp = p.Jp;
+  const int tiles_per_batch = N * tiles_per_row;
+
+  u32x4_t raw[LN_ITERS];
+  auto load_tile = [&](int tile_id) {
+    const int b = tile_id / tiles_per_batch;
+    const int rem = tile_id - b * tiles_per_batch;
+    const int i = rem / tiles_per_row;
+    const int j0 = (rem - i * tiles_per_row) * TP;
+    const bf16_t* xrow = p.x + b * p.x_view.stride_b + i * p.x_view.stride_r;
+#pragma unroll
+    for (int it = 0; it < LN_ITERS; ++it) {
+      const int j = j0 + wave * 32 + it * PPI + ln_pp;
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (j < N) v = *reinterpret_cast<const u32x4_t*>(xrow + j * p.x_view.stride_k + 8 * ln_chunk);
+      raw[it] = v;
+    }
+  };
+
+  int tile_id = blockIdx.x;
+  if (tile_id < total_tiles) load_tile(tile_id);
+
+  for (; tile_id < total_tiles; tile_id += gridDim.x) {
+    const int b = tile_id / tiles_per_batch;
+    const int rem = tile_id - b * tiles_per_batch;
+    const int i = rem / tiles_per_row;
+    const int j0 = (rem - i * tiles_per_row) * TP;
+
+    // ---- LayerNorm phase (+ mask bias, one lane per position)
+#pragma unroll
+    for (int it = 0; it < LN_ITERS; ++it) {
+      const int pos = wave * 32 + it * PPI + ln_pp;
+      tile[tile_slot<NCH, 2>(pos, ln_chunk)] = layer_norm_chunk<C>(raw[it], lw, lb);
+      if (ln_chunk == 0) {
+        const int j = j0 + pos;
+        float mb = -__builtin_inff();
+        if (j < N) {
+          float m = 1.f;
+          if (p.mask) m = p.mask[b * p.mask_view.stride_b + i * p.mask_view.stride_r + j * p.mask_view.stride_k];
+          mb = kLog2e * (p.inf * (m - 1.f));
+        }
+        p.mbias[((size_t)b * N + i) * Jp + j] = mb;
+      }
+    }
+    __syncthreads();
+
+    if (tile_id + (int)gridDim.x < total_tiles) load_tile(tile_id + gridDim.x);
+
+    // ---- projection phase: position 4*l32 + t is column l32 of position-tile t
+    uint32_t vpk[2][2][16];   // v jobs only: [tile][position pair][register]
+    float vprev[2][16];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      u32x4_t bop[KS];
+      const int pos = 4 * l32 + t;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) bop[s] = tile[tile_slot<NCH, 2>(pos, 2 * s + lh)];
+
+      if (has_jobs) {
+#pragma unroll
+        for (int jj = 0; jj < NJ; ++jj) {
+          const int m = job_matrix(jj), ot = job_tile(jj);
+          f32x16_t acc = zero16();
+#pragma unroll
+          for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wj[jj][s], bop[s], acc);
+          if (m == 2) {
+            const int vi = WIDE ? 0 : jj;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              if (t & 1)
+                vpk[vi][t >> 1][v] = pack_bf16(vprev[vi][v], acc[v]);
+              else
+                vprev[vi][v] = acc[v];
+            }
+          } else {
+            // lane owns channels 32*ot + 16*lh + v  ->  head, d0 .. d0+15
+            const int ch0 = 32 * ot + 16 * lh;
+            const int head = ch0 / D, d0 = ch0 % D;
+            const float sc = (m == 0) ? qscale : 1.f;
+            u32x4_t o0, o1;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              o0[q] = pack_bf16(acc[2 * q] * sc, acc[2 * q + 1] * sc);
+              o1[q] = pack_bf16(acc[8 + 2 * q] * sc, acc[8 + 2 * q + 1] * sc);
+            }
+            bf16_t* base = (m == 0) ? p.q : p.k;
+            bf16_t* dst = base + ((((size_t)b * N + i) * H + head) * Jp + (j0 + pos)) * D + d0;
+            *reinterpret_cast<u32x4_t*>(dst) = o0;
+            *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
+          }
+        }
+      }
+
+      // triangle bias of this position tile: WIDE -> wave t, else wave 3
+      const bool bias_here = WIDE ? (wave == t) : (wave == 3);
+      if (bias_here) {
+        f32x16_t acc = zero16();
+#pragma unroll
+        for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wb[s], bop[s], acc);
+        // rows 0..3 of the result sit in registers 0..3 of lanes 0..31
+        const int j = j0 + pos;
+        if (lh == 0 && j < Jp) {
+#pragma unroll
+          for (int h = 0; h < H; ++h)
+            p.tbias[(((size_t)b * H + h) * N + i) * Jp + j] = (j < N) ? acc[h] * kLog2e : 0.f;
+        }
+      }
+    }
+
+    // ---- v stores: register v is channel 32*ot + 8*(v/4) + 4*lh + v%4 = head*D + d
+    if (has_jobs) {
+#pragma unroll
+      for (int jj = 0; jj < NJ; ++jj) {
+        if (job_matrix(jj) != 2) continue;
+        const int ot = job_tile(jj);
+        const int vi = WIDE ? 0 : jj;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int ch = 32 * ot + 8 * (v >> 2) + 4 * lh + (v & 3);
+          const int head = ch / D, d = ch % D;
+          bf16_t* dst = p.vt + ((((size_t)b * N + i) * H + head) * D + d) * Jp + j0 + 4 * l32;
+          u32x2_t w2 = {vpk[vi][0][v], vpk[vi][1][v]};
+          *reinterpret_cast<u32x2_t*>(dst) = w2;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <int C, int D>
+hipError_t launch(const TriattnProjArgs& a, hipStream_t stream) {
+  auto kern = triattn_proj_kernel<C, D>;
+  static int grid_cap = 0;
+  if (grid_cap == 0) {
+    int dev = 0, cus = 0, per_cu = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, 0);
+    if (e != hipSuccess) return e;
+    grid_cap = cus * (per_cu > 0 ? per_cu : 1);
+  }
+  const int tiles_per_row = a.Jp / 128;
+  const long total = (long)a.B * a.N * tiles_per_row;
+  const int grid = (int)(total < grid_cap ? total : grid_cap);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), 0, stream, a, tiles_per_row, (int)total);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t triattn_proj_launch(const TriattnProjArgs& args, int C, int D, hipStream_t stream) {
+  if (args.H != 4) return hipErrorInvalidValue;
+  if (C == 128 && D == 32) return launch<128, 32>(args, stream);
+  if (C == 64 && D == 16) return launch<64, 16>(args, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace of3

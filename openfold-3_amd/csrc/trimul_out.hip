@@ -1,0 +1,195 @@
+// Triangle-multiplication output pass
+//     out = [z +] (LayerNorm_out(x) Wz^T) * sigmoid(LayerNorm_in(z) Wg^T)
+// (triangular_multiplicative_update.py:498-501; the optional residual is the caller's
+// "z = z + update" of base_blocks.py:329-335 fused in).  x arrives channel-major
+// [b][c][i][j] from the contraction and is transposed to position-major on its way into
+// LDS; the gate is recomputed from z instead of being stored by the input pass, which
+// saves one full write and one full read of a z-sized tensor.
+//
+// HBM bound: reads x and z once, writes out once.
+#include "of3_device.h"
+#include "of3_kernels.h"
+
+namespace of3 {
+
+namespace {
+
+template <int C, int CH>
+__global__ __launch_bounds__(256) void trimul_out_kernel(TrimulOutArgs p, int tiles_per_row, int total_tiles) {
+  static_assert(C == CH, "position-major x tile shares the z tile geometry");
+  constexpr int NCH = C / 8;
+  constexpr int LPP = NCH;
+  constexpr int PPI = 64 / LPP;
+  constexpr int TP = 128;
+  constexpr int LN_ITERS = 32 / PPI;
+  constexpr int KS = C / 16;
+  constexpr int NOT = C / 32;            // output-channel tiles
+  constexpr int WPG = 4 / NOT;           // waves sharing one output tile (1 or 2)
+  constexpr int TPW = 4 / WPG;           // position tiles per wave
+  constexpr int XROUNDS = (CH / 2) * 16 / 256;  // (channel pair, 8-position group) items per thread
+
+  __shared__ u32x4_t ztile[TP * NCH];
+  __shared__ u32x4_t xtile[TP * NCH];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int ln_chunk = lane % LPP, ln_pp = lane / LPP;
+
+  float iw[8], ib[8], ow[8], ob[8];
+  load_affine8(p.ln_in_w, ln_chunk, iw);
+  load_affine8(p.ln_in_b, ln_chunk, ib);
+  load_affine8(p.ln_out_w, ln_chunk, ow);
+  load_affine8(p.ln_out_b, ln_chunk, ob);
+
+  // A operands: logical output channel of A-row r is 32*ot + rowperm16(r), so that a lane
+  // ends up with the 16 consecutive channels 32*ot + 16*lh + v
+  const int ot = wave % NOT;
+  const int t0 = (wave / NOT) * TPW;
+  u32x4_t wz[KS], wgt[KS];
+  {
+    const int row = 32 * ot + rowperm16(l32);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      wz[s] = *reinterpret_cast<const u32x4_t*>(p.w_z + row * CH + 16 * s + 8 * lh);
+      wgt[s] = *reinterpret_cast<const u32x4_t*>(p.w_g + row * C + 16 * s + 8 * lh);
+    }
+  }
+
+  const int N = p.N, Np = p.Np;
+  const int tiles_per_batch = N * tiles_per_row;
+  uint16_t* xt16 = reinterpret_cast<uint16_t*>(xtile);
+  uint32_t* xt32 = reinterpret_cast<uint32_t*>(xtile);
+  (void)xt16;
+
+  for (int tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+    const int b = tile_id / tiles_per_batch;
+    const int rem = tile_id - b * tiles_per_batch;
+    const int i = rem / tiles_per_row;
+    const int j0 = (rem - i * tiles_per_row) * TP;
+    const bf16_t* zrow = p.z + b * p.z_view.stride_b + i * p.z_view.stride_r;
+    bf16_t* orow = p.out + b * p.z_view.stride_b + i * p.z_view.stride_r;
+
+    // ---- loads: z (row-wise, for the gate) and x (channel-major, transposed below)
+    u32x4_t zraw[LN_ITERS];
+#pragma unroll
+    for (int it = 0; it < LN_ITERS; ++it) {
+      const int j = j0 + wave * 32 + it * PPI + ln_pp;
+      u32x4_t v = {0u, 0u, 0u, 0u};
+      if (j < N) v = *reinterpret_cast<const u32x4_t*>(zrow + j * p.z_view.stride_k + 8 * ln_chunk);
+      zraw[it] = v;
+    }
+    u32x4_t xa[XROUNDS], xb[XROUNDS];
+#pragma unroll
+    for (int rr = 0; rr < XROUNDS; ++rr) {
+      const int item = rr * 256 + tid;
+      const int cp = item >> 4, pg = item & 15;  // channels 2cp, 2cp+1; positions 8pg..8pg+7
+      const bf16_t* src = p.x + (((size_t)b * CH + 2 * cp) * Np + i) * Np + j0 + 8 * pg;
+      xa[rr] = *reinterpret_cast<const u32x4_t*>(src);
+      xb[rr] = *reinterpret_cast<const u32x4_t*>(src + (size_t)Np * Np);
+    }
+
+    // x: transpose into xtile[pos][c] with 4-byte (channel pair) writes
+#pragma unroll
+    for (int rr = 0; rr < XROUNDS; ++rr) {
+      const int item = rr * 256 + tid;
+      const int cp = item >> 4, pg = item & 15;
+      const int chunk = (2 * cp) >> 3, within = (2 * cp) & 7;  // `within` is even
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t ua = xa[rr][e >> 1], ub = xb[rr][e >> 1];
+        const uint32_t w = (e & 1) ? ((ua >> 16) | (ub & 0xffff0000u)) : ((ua & 0xffffu) | (ub << 16));
+        const int pos = 8 * pg + e;
+        xt32[tile_slot<NCH, 0>(pos, chunk) * 4 + (within >> 1)] = w;
+      }
+    }
+    // z: LayerNorm_in -> ztile
+#pragma unroll
+    for (int it = 0; it < LN_ITERS; ++it) {
+      const int pos = wave * 32 + it * PPI + ln_pp;
+      ztile[tile_slot<NCH, 0>(pos, ln_chunk)] = layer_norm_chunk<C>(zraw[it], iw, ib);
+    }
+    __syncthreads();
+
+    // x: LayerNorm_out in place (lane owns one 16-byte chunk of one position)
+#pragma unroll
+    for (int it = 0; it < LN_ITERS; ++it) {
+      const int pos = wave * 32 + it * PPI + ln_pp;
+      const int slot = tile_slot<NCH, 0>(pos, ln_chunk);
+      xtile[slot] = layer_norm_chunk<CH>(xtile[slot], ow, ob);
+    }
+    __syncthreads();
+
+    // ---- matrix phase
+#pragma unroll
+    for (int tt = 0; tt < TPW; ++tt) {
+      const int t = t0 + tt;
+      const int pos = 32 * t + l32;
+      f32x16_t accu = zero16(), accg = zero16();
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const u32x4_t bx = xtile[tile_slot<NCH, 0>(pos, 2 * s + lh)];
+        const u32x4_t bz = ztile[tile_slot<NCH, 0>(pos, 2 * s + lh)];
+        accu = mfma_32x32x16(wz[s], bx, accu);
+        accg = mfma_32x32x16(wgt[s], bz, accg);
+      }
+      const int j = j0 + pos;
+      if (j < N) {
+        const int64_t off = j * p.z_view.stride_k + 32 * ot + 16 * lh;
+        float res[16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) res[v] = accu[v] * sigmoidf_fast(accg[v]);
+        if (p.add_residual) {
+          const u32x4_t r0 = *reinterpret_cast<const u32x4_t*>(zrow + off);
+          const u32x4_t r1 = *reinterpret_cast<const u32x4_t*>(zrow + off + 8);
+          float zr[8];
+          unpack8(r0, zr);
+#pragma unroll
+          for (int v = 0; v < 8; ++v) res[v] += zr[v];
+          unpack8(r1, zr);
+#pragma unroll
+          for (int v = 0; v < 8; ++v) res[8 + v] += zr[v];
+        }
+        u32x4_t o0, o1;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          o0[q] = pack_bf16(res[2 * q], res[2 * q + 1]);
+          o1[q] = pack_bf16(res[8 + 2 * q], res[8 + 2 * q + 1]);
+        }
+        *reinterpret_cast<u32x4_t*>(orow + off) = o0;
+        *reinterpret_cast<u32x4_t*>(orow + off + 8) = o1;
+      }
+    }
+    __syncthreads();  // both tiles are rewritten by the next iteration
+  }
+}
+
+template <int C, int CH>
+hipError_t launch(const TrimulOutArgs& a, hipStream_t stream) {
+  auto kern = trimul_out_kernel<C, CH>;
+  static int grid_cap = 0;
+  if (grid_cap == 0) {
+    int dev = 0, cus = 0, per_cu = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, 0);
+    if (e != hipSuccess) return e;
+    grid_cap = cus * (per_cu > 0 ? per_cu : 1);
+  }
+  const int tiles_per_row = (a.N + 127) / 128;
+  const long total = (long)a.B * a.N * tiles_per_row;
+  const int grid = (int)(total < grid_cap ? total : grid_cap);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), 0, stream, a, tiles_per_row, (int)total);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t trimul_out_launch(const TrimulOutArgs& args, int C, int CH, hipStream_t stream) {
+  if (C == 128 && CH == 128) return launch<128, 128>(args, stream);
+  if (C == 64 && CH == 64) return launch<64, 64>(args, stream);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace of3

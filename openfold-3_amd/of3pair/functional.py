@@ -1,0 +1,155 @@
+"""Tensor-level wrappers over the C ABI: the functional boundary the reference already has
+for alternative kernels (_cueq_triangle_mult, tmu.py:689-741; Attention's kernel branch,
+attention.py:366-413), here with a single implementation and no dispatch.
+
+All functions run on the current CUDA(HIP) stream of the tensors' device, are forward-only
+and accept bf16 pair tensors shaped [*, N, N, C] (any number of leading batch dimensions, a
+transposed view in the two N dimensions is fine and is not copied).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_workspaces: dict = {}
+
+
+def _workspace(device, nbytes: int) -> torch.Tensor:
+    """Grow-only scratch per device, owned by this Python layer (the library allocates
+    nothing).  Kernels on one stream are ordered, so one buffer per device is shared by all
+    modules; callers using several streams on one device must pass their own workspace."""
+    buf = _workspaces.get(device)
+    if buf is None or buf.numel() < nbytes:
+        buf = None
+        _workspaces.pop(device, None)
+        buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+        _workspaces[device] = buf
+    return buf
+
+
+def release_workspaces():
+    _workspaces.clear()
+
+
+def _require_gpu_bf16(t: torch.Tensor, name: str):
+    if not t.is_cuda:
+        raise RuntimeError("%s must live on the GPU: the pair-stack kernels have no CPU path" % name)
+    if t.dtype != torch.bfloat16:
+        raise ValueError("%s must be bfloat16 (got %s): only the bf16 kernels are built" % (name, t.dtype))
+
+
+def _flatten_pair(z: torch.Tensor):
+    """[*, N, N, C] -> a 4-D view [B, N, N, C] with unit channel stride, no copy when the
+    leading dimensions can be merged."""
+    if z.dim() < 3:
+        raise ValueError("pair tensor must be [*, N, N, C]")
+    n1, n2, c = z.shape[-3:]
+    if n1 != n2:
+        raise ValueError("pair tensor must be square in its two token dimensions, got %s" % (tuple(z.shape),))
+    if z.stride(-1) != 1 and c != 1:
+        z = z.contiguous()
+    lead = z.shape[:-3]
+    if len(lead) == 0:
+        z4 = z.unsqueeze(0)
+    elif len(lead) == 1:
+        z4 = z
+    else:
+        try:
+            z4 = z.view(-1, n1, n2, c)
+        except RuntimeError:
+            z4 = z.reshape(-1, n1, n2, c)
+    if any(s % 8 for s in z4.stride()[:3]) or z4.data_ptr() % 16:
+        z4 = z4.contiguous()
+    return z4, lead
+
+
+def _mask_arg(mask, lead, B, N, device):
+    if mask is None:
+        return None, None, None
+    m = mask
+    if m.shape[-2:] != (N, N):
+        raise ValueError("mask must be [*, N, N]")
+    if m.dtype != torch.float32:
+        m = m.to(torch.float32)
+    m = m.expand(*lead, N, N) if len(lead) else m
+    m3 = m.reshape(B, N, N) if m.dim() != 3 else m
+    return m3, m3.data_ptr(), _lib.strides3(m3.stride())
+
+
+def _w(t: torch.Tensor) -> torch.Tensor:
+    """Parameter as a contiguous bf16 device tensor (what a module cast with
+    .to(torch.bfloat16) holds; fp32 parameters are rounded once per call)."""
+    if t.dtype != torch.bfloat16 or not t.is_contiguous():
+        t = t.detach().to(torch.bfloat16).contiguous()
+    return t
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _out_like(z4: torch.Tensor) -> torch.Tensor:
+    return torch.empty_strided(z4.shape, z4.stride(), dtype=z4.dtype, device=z4.device)
+
+
+def _finish(z, z4, out4, lead, inplace):
+    out = out4.view(z.shape)
+    if not inplace:
+        return out
+    if z4.data_ptr() != z.data_ptr():  # the kernels ran on a re-laid-out copy
+        z.copy_(out)
+    return z
+
+
+def triangle_multiplicative_update(z, mask, norm_in_weight, norm_in_bias, norm_out_weight, norm_out_bias,
+                                   a_p_weight, a_g_weight, b_p_weight, b_g_weight, g_out_weight, p_out_weight,
+                                   outgoing: bool, add_residual: bool = False, inplace: bool = False):
+    """Update of tmu.py:482-503, or z + update when add_residual.  With inplace the result
+    overwrites z (the reference's inplace_safe contract, tmu.py:154-173)."""
+    _require_gpu_bf16(z, "z")
+    lib = _lib.load()
+    z4, lead = _flatten_pair(z)
+    B, N, _, C = z4.shape
+    CH = a_p_weight.shape[0]
+    nbytes = lib.of3_trimul_workspace_bytes(B, N, C, CH)
+    if nbytes < 0:
+        raise ValueError("triangle multiplication supports (c_z, c_hidden) = (128,128) or (64,64); got (%d,%d)" % (C, CH))
+    keep = [_w(t) for t in (norm_in_weight, norm_in_bias, norm_out_weight, norm_out_bias, a_p_weight, a_g_weight,
+                            b_p_weight, b_g_weight, g_out_weight, p_out_weight)]
+    m3, mptr, mstr = _mask_arg(mask, lead, B, N, z.device)
+    out4 = z4 if inplace else _out_like(z4)
+    ws = _workspace(z.device, nbytes)
+    with torch.cuda.device(z.device):
+        st = lib.of3_trimul_fwd(z4.data_ptr(), _lib.strides3(z4.stride()[:3]), mptr, mstr, *[k.data_ptr() for k in keep],
+                                out4.data_ptr(), B, N, C, CH, int(bool(outgoing)), int(bool(add_residual)),
+                                ws.data_ptr(), ws.numel(), _lib.OF3_DTYPE_BF16, _stream(z))
+    _lib.check(st, "of3_trimul_fwd")
+    return _finish(z, z4, out4, lead, inplace)
+
+
+def triangle_attention(x, mask, norm_weight, norm_bias, bias_weight, q_weight, k_weight, v_weight, g_weight,
+                       o_weight, no_heads: int, inf: float = 1e9, add_residual: bool = False,
+                       inplace: bool = False):
+    """Update of tri_att.py:102-167 for a starting-node module; hand in the transposed view
+    for the ending node (base_blocks.py:380-404 does exactly that)."""
+    _require_gpu_bf16(x, "x")
+    lib = _lib.load()
+    x4, lead = _flatten_pair(x)
+    B, N, _, C = x4.shape
+    H = int(no_heads)
+    D = q_weight.shape[0] // H
+    nbytes = lib.of3_triattn_workspace_bytes(B, N, C, H, D)
+    if nbytes < 0:
+        raise ValueError("triangle attention supports 4 heads with (c_in, c_head) = (128,32) or (64,16); "
+                         "got c_in=%d heads=%d c_head=%d" % (C, H, D))
+    keep = [_w(t) for t in (norm_weight, norm_bias, bias_weight, q_weight, k_weight, v_weight, g_weight, o_weight)]
+    m3, mptr, mstr = _mask_arg(mask, lead, B, N, x.device)
+    out4 = x4 if inplace else _out_like(x4)
+    ws = _workspace(x.device, nbytes)
+    with torch.cuda.device(x.device):
+        st = lib.of3_triattn_fwd(x4.data_ptr(), _lib.strides3(x4.stride()[:3]), mptr, mstr,
+                                 *[k.data_ptr() for k in keep], out4.data_ptr(), B, N, C, H, D, float(inf),
+                                 int(bool(add_residual)), ws.data_ptr(), ws.numel(), _lib.OF3_DTYPE_BF16, _stream(x))
+    _lib.check(st, "of3_triattn_fwd")
+    return _finish(x, x4, out4, lead, inplace)

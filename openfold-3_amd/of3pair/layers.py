@@ -1,0 +1,189 @@
+"""Drop-in counterparts of the reference's pair-stack layer modules.
+
+Constructor arguments, parameter names (state-dict keys) and forward signatures follow
+  openfold3/core/model/layers/triangular_multiplicative_update.py:119-152, :421-429, :506-519
+  openfold3/core/model/layers/triangular_attention.py:31-69, :102-111, :171-179
+so that a PairBlock (openfold3/core/model/latent/base_blocks.py:268-288) can hold these
+modules instead and load the same checkpoints.  The arithmetic runs in libof3pair (HIP);
+there is one implementation, so the reference's kernel-selection and chunking keyword
+arguments are accepted and ignored.  Forward only: gradients are not recorded.
+"""
+from __future__ import annotations
+
+import math
+from functools import partialmethod
+
+import torch
+import torch.nn as nn
+
+from . import functional as F3
+
+
+def _truncated_normal_(weight: torch.Tensor, scale: float = 1.0):
+    """LeCun fan-in truncated normal (cut at two standard deviations), the reference's
+    "default" Linear initialiser (initialization.py:48-63).  Drawn with torch's generator;
+    the reference draws the same distribution from scipy on numpy's global generator, so the
+    sample streams differ while the distribution does not."""
+    fan_in = weight.shape[1]
+    # standard deviation of a unit normal truncated to [-2, 2]
+    trunc_std = 0.87962566103423978
+    std = math.sqrt(scale / max(1, fan_in)) / trunc_std
+    with torch.no_grad():
+        nn.init.trunc_normal_(weight, mean=0.0, std=std, a=-2.0 * std, b=2.0 * std)
+
+
+def _init_linear(lin: nn.Linear, how: str):
+    if how == "default":
+        _truncated_normal_(lin.weight)
+    elif how in ("final", "gating"):
+        with torch.no_grad():
+            lin.weight.zero_()
+    else:
+        raise ValueError("Invalid init string.")
+
+
+# Initialiser table of the AF3 pair stack (default_linear_init_config.py:110-119, :45-53,
+# :78-83): every Linear is bias-free; gates and output projections start at zero.
+TRI_MUL_INIT = {
+    "linear_a_p": "default", "linear_a_g": "final", "linear_b_p": "default", "linear_b_g": "final",
+    "linear_g": "final", "linear_z": "final",
+}
+TRI_ATT_INIT = {
+    "linear_z": "default",
+    "mha": {"linear_q": "default", "linear_k": "default", "linear_v": "default", "linear_g": "gating",
+            "linear_o": "final"},
+}
+
+
+def _init_name(spec, key, default):
+    """Accepts the table above or a reference-style mapping {"bias": False, "init": "..."}."""
+    if spec is None:
+        return default
+    v = spec[key] if not hasattr(spec, "get") else spec.get(key, default)
+    if isinstance(v, str):
+        return v
+    if v.get("bias", False):
+        raise ValueError("the pair-stack kernels implement the bias-free Linears of the AF3 tables")
+    return v.get("init", default)
+
+
+class TriangleMultiplicativeUpdate(nn.Module):
+    """AF3 Algorithms 12 and 13 (tmu.py:119-503)."""
+
+    def __init__(self, c_z, c_hidden, _outgoing=True, linear_init_params=None):
+        super().__init__()
+        self.c_z = c_z
+        self.c_hidden = c_hidden
+        self._outgoing = _outgoing
+        self.linear_g = nn.Linear(c_z, c_z, bias=False)
+        self.linear_z = nn.Linear(c_hidden, c_z, bias=False)
+        self.layer_norm_in = nn.LayerNorm(c_z, eps=1e-5)
+        self.layer_norm_out = nn.LayerNorm(c_hidden, eps=1e-5)
+        self.linear_a_p = nn.Linear(c_z, c_hidden, bias=False)
+        self.linear_a_g = nn.Linear(c_z, c_hidden, bias=False)
+        self.linear_b_p = nn.Linear(c_z, c_hidden, bias=False)
+        self.linear_b_g = nn.Linear(c_z, c_hidden, bias=False)
+        for name, default in TRI_MUL_INIT.items():
+            _init_linear(getattr(self, name), _init_name(linear_init_params, name, default))
+
+    @torch.no_grad()
+    def forward(self, z, mask=None, inplace_safe=False, use_cueq_triangle_kernels=False,
+                _add_with_inplace=False, _inplace_chunk_size=256):
+        """z [*, N, N, C_z], mask [*, N, N] -> [*, N, N, C_z].
+
+        Returns the update; with inplace_safe the result overwrites z and, if
+        _add_with_inplace is also set, is z + update (tmu.py:473-480, :399-405).  The
+        kernel-selection flag and the chunk size are accepted for signature compatibility."""
+        return F3.triangle_multiplicative_update(
+            z, mask,
+            self.layer_norm_in.weight, self.layer_norm_in.bias,
+            self.layer_norm_out.weight, self.layer_norm_out.bias,
+            self.linear_a_p.weight, self.linear_a_g.weight, self.linear_b_p.weight, self.linear_b_g.weight,
+            self.linear_g.weight, self.linear_z.weight,
+            outgoing=self._outgoing,
+            add_residual=bool(inplace_safe and _add_with_inplace),
+            inplace=bool(inplace_safe),
+        )
+
+
+class TriangleMultiplicationOutgoing(TriangleMultiplicativeUpdate):
+    """AF3 Algorithm 12."""
+
+    __init__ = partialmethod(TriangleMultiplicativeUpdate.__init__, _outgoing=True)
+
+
+class TriangleMultiplicationIncoming(TriangleMultiplicativeUpdate):
+    """AF3 Algorithm 13."""
+
+    __init__ = partialmethod(TriangleMultiplicativeUpdate.__init__, _outgoing=False)
+
+
+class _GatedAttentionParams(nn.Module):
+    """Holds the parameters of the reference's Attention module (attention.py:206-263) under
+    the same names; the computation itself is fused into the triangle-attention kernels."""
+
+    def __init__(self, c_in, c_hidden, no_heads, init):
+        super().__init__()
+        hc = c_hidden * no_heads
+        self.c_hidden = c_hidden
+        self.no_heads = no_heads
+        self.linear_q = nn.Linear(c_in, hc, bias=False)
+        self.linear_k = nn.Linear(c_in, hc, bias=False)
+        self.linear_v = nn.Linear(c_in, hc, bias=False)
+        self.linear_o = nn.Linear(hc, c_in, bias=False)
+        self.linear_g = nn.Linear(c_in, hc, bias=False)
+        for name, default in TRI_ATT_INIT["mha"].items():
+            _init_linear(getattr(self, name), _init_name(init, name, default))
+
+
+class TriangleAttention(nn.Module):
+    """AF3 Algorithms 14 and 15 (tri_att.py:31-167).  c_hidden is the per-head width, as
+    the reference's Attention treats it (attention.py:240-242)."""
+
+    def __init__(self, c_in, c_hidden, no_heads, starting=True, inf=1e9, linear_init_params=None):
+        super().__init__()
+        self.c_in = c_in
+        self.c_hidden = c_hidden
+        self.no_heads = no_heads
+        self.starting = starting
+        self.inf = inf
+        self.layer_norm = nn.LayerNorm(c_in, eps=1e-5)
+        self.linear_z = nn.Linear(c_in, no_heads, bias=False)
+        _init_linear(self.linear_z, _init_name(linear_init_params, "linear_z", TRI_ATT_INIT["linear_z"]))
+        mha_init = None
+        if linear_init_params is not None:
+            mha_init = linear_init_params["mha"] if "mha" in linear_init_params else None
+        self.mha = _GatedAttentionParams(c_in, c_hidden, no_heads, mha_init)
+
+    @torch.no_grad()
+    def forward(self, x, mask=None, chunk_size=None, use_deepspeed_evo_attention=False,
+                use_cueq_triangle_kernels=False, use_lma=False, inplace_safe=False,
+                _add_residual=False):
+        """x [*, I, J, C_in], mask [*, I, J] -> [*, I, J, C_in] (the update).
+
+        The back-end flags and chunk_size of the reference are accepted and ignored: the
+        flash kernel never materialises the logits, so there is nothing to chunk.
+        _add_residual (not in the reference) returns x + update from the output kernel; the
+        pair-stack runner uses it to fuse the caller's add of base_blocks.py:364-378."""
+        if not self.starting:
+            x = x.transpose(-2, -3)
+            mask = mask.transpose(-1, -2) if mask is not None else None
+        out = F3.triangle_attention(
+            x, mask,
+            self.layer_norm.weight, self.layer_norm.bias, self.linear_z.weight,
+            self.mha.linear_q.weight, self.mha.linear_k.weight, self.mha.linear_v.weight,
+            self.mha.linear_g.weight, self.mha.linear_o.weight,
+            no_heads=self.no_heads, inf=self.inf, add_residual=bool(_add_residual), inplace=False,
+        )
+        if not self.starting:
+            out = out.transpose(-2, -3)
+        return out
+
+
+TriangleAttentionStartingNode = TriangleAttention
+
+
+class TriangleAttentionEndingNode(TriangleAttention):
+    """AF3 Algorithm 15."""
+
+    __init__ = partialmethod(TriangleAttention.__init__, starting=False)

@@ -1,0 +1,84 @@
+"""The pair-stack half of the reference's PairBlock: sequencing of the four modules with
+their residual adds, as in openfold3/core/model/latent/base_blocks.py:307-406, and the
+per-template variant of template_module.py:148-166 (templates are independent pair
+representations, so they are folded into the batch instead of looped over).
+
+Unlike the reference, no physical transpose of z is made around the ending-node attention
+(base_blocks.py:380-404): the kernels walk the transposed view through strides.  The
+residual adds are fused into each module's output kernel.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import functional as F3
+from .layers import (TriangleAttention, TriangleMultiplicationIncoming, TriangleMultiplicationOutgoing)
+
+
+class PairStack(nn.Module):
+    """tri_mul_out -> tri_mul_in -> tri_att_start -> tri_att_end, each followed by its
+    residual add (dropout is the identity in eval mode, dropout.py:57-58).  Sub-module names
+    match PairBlock's, so `pair_stack.<name>.<param>` checkpoint keys load unchanged.  The
+    pair transition that follows in PairBlock.forward (base_blocks.py:470-478) is not part of
+    this module."""
+
+    def __init__(self, c_z: int, c_hidden_mul: int, c_hidden_pair_att: int, no_heads_pair: int,
+                 inf: float = 1e9, linear_init_params=None):
+        super().__init__()
+        tm = None if linear_init_params is None else linear_init_params["tri_mul"]
+        ta = None if linear_init_params is None else linear_init_params["tri_att"]
+        self.tri_mul_out = TriangleMultiplicationOutgoing(c_z, c_hidden_mul, linear_init_params=tm)
+        self.tri_mul_in = TriangleMultiplicationIncoming(c_z, c_hidden_mul, linear_init_params=tm)
+        self.tri_att_start = TriangleAttention(c_z, c_hidden_pair_att, no_heads_pair, inf=inf,
+                                               linear_init_params=ta)
+        # like the reference, a *starting* module that is handed the transposed tensor
+        self.tri_att_end = TriangleAttention(c_z, c_hidden_pair_att, no_heads_pair, inf=inf,
+                                             linear_init_params=ta)
+
+    @staticmethod
+    def _mul(module, z, mask, inplace):
+        return F3.triangle_multiplicative_update(
+            z, mask,
+            module.layer_norm_in.weight, module.layer_norm_in.bias,
+            module.layer_norm_out.weight, module.layer_norm_out.bias,
+            module.linear_a_p.weight, module.linear_a_g.weight, module.linear_b_p.weight, module.linear_b_g.weight,
+            module.linear_g.weight, module.linear_z.weight,
+            outgoing=module._outgoing, add_residual=True, inplace=inplace)
+
+    @staticmethod
+    def _att(module, z, mask, inplace):
+        return F3.triangle_attention(
+            z, mask, module.layer_norm.weight, module.layer_norm.bias, module.linear_z.weight,
+            module.mha.linear_q.weight, module.mha.linear_k.weight, module.mha.linear_v.weight,
+            module.mha.linear_g.weight, module.mha.linear_o.weight,
+            no_heads=module.no_heads, inf=module.inf, add_residual=True, inplace=inplace)
+
+    @torch.no_grad()
+    def tri_mul_out_in(self, z, pair_mask, inplace_safe: bool = False, use_cueq_triangle_kernels: bool = False):
+        """base_blocks.py:307-351.  Without inplace_safe the caller's tensor is left intact:
+        the first z + update lands in a new tensor, which the second module then overwrites."""
+        z = self._mul(self.tri_mul_out, z, pair_mask, inplace=inplace_safe)
+        return self._mul(self.tri_mul_in, z, pair_mask, inplace=True)
+
+    @torch.no_grad()
+    def tri_att_start_end(self, z, pair_mask, _attn_chunk_size=None, use_deepspeed_evo_attention=False,
+                          use_cueq_triangle_kernels=False, use_lma=False, inplace_safe: bool = False):
+        """base_blocks.py:353-406; the ending node is the starting-node module run on the
+        transposed view of z and of the mask."""
+        z = self._att(self.tri_att_start, z, pair_mask, inplace=inplace_safe)
+        zt = z.transpose(-2, -3)
+        mt = pair_mask.transpose(-1, -2) if pair_mask is not None else None
+        zt = self._att(self.tri_att_end, zt, mt, inplace=True)
+        return zt.transpose(-2, -3)
+
+    @torch.no_grad()
+    def forward(self, z, pair_mask, chunk_size=None, use_deepspeed_evo_attention=False,
+                use_cueq_triangle_kernels=False, use_lma=False, inplace_safe: bool = False,
+                _attn_chunk_size=None):
+        """z [*, N, N, C_z], pair_mask [*, N, N] -> z after the four residual updates.
+        Leading dimensions (batch, templates) are independent and processed together.  With
+        inplace_safe the input tensor is overwritten; otherwise it is left intact."""
+        z = self.tri_mul_out_in(z, pair_mask, inplace_safe=inplace_safe)
+        # z is now a tensor this module owns (or the caller allowed overwriting)
+        return self.tri_att_start_end(z, pair_mask, inplace_safe=True)

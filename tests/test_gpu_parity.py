@@ -1,0 +1,155 @@
+"""Parity of the HIP path (drop-in modules -> C ABI -> kernels) with the CPU oracle on the
+same seeded inputs and weights.
+
+bf16 bound (north star: "2e-2 relative in bf16"): inputs and weights are rounded to bf16
+once, the oracle computes in fp32 from those rounded values, and every output element must
+satisfy  |got - want| <= 2e-2 * (|want| + rms(want)).  The rms term is the absolute floor
+for elements near zero.  A second, tighter check bounds the overall error:
+rms(got - want) <= 5e-3 * rms(want) for update tensors."""
+import math
+
+import pytest
+import torch
+
+from gpu_util import lib, report  # noqa: F401  (lib() makes sure the library is built)
+from oracle import pairstack_oracle as orc
+
+import of3pair
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+REL = 2e-2
+
+
+def _check(name, got, want, rms_rel=5e-3):
+    got = got.float().cpu()
+    want = want.float()
+    rms = float(want.pow(2).mean().sqrt())
+    report(name, got, want, atol=REL * rms, rtol=REL)
+    erms = float((got - want).pow(2).mean().sqrt())
+    assert erms <= rms_rel * rms, "%s: rms error %.3g vs rms %.3g" % (name, erms, rms)
+
+
+def _round_params(p):
+    return {k: orc.round_bf16(v) for k, v in p.items()}
+
+
+def _load(module, params):
+    module.load_state_dict(params, strict=True)
+    return module.to(DEV).to(torch.bfloat16).eval()
+
+
+@pytest.mark.parametrize("outgoing", [True, False])
+@pytest.mark.parametrize("c,n,batch", [(128, 64, ()), (128, 100, (2,)), (64, 96, (1, 3))])
+def test_trimul_module(outgoing, c, n, batch):
+    lib()
+    gen = torch.Generator().manual_seed(100 + n)
+    p = _round_params(orc.make_trimul_params(gen, c, c))
+    z = orc.round_bf16(orc.make_pair_input(1, batch, n, c))
+    mask = (torch.rand(*batch, n, n, generator=gen) > 0.2).float()
+    cls = of3pair.TriangleMultiplicationOutgoing if outgoing else of3pair.TriangleMultiplicationIncoming
+    m = _load(cls(c, c), p)
+    print("trimul module", outgoing, c, n, batch, flush=True)
+    zg = z.to(DEV).to(torch.bfloat16)
+    got = m(zg, mask=mask.to(DEV))
+    want = orc.trimul_update(z, mask, p, outgoing)
+    _check("trimul update", got, want)
+    assert torch.equal(zg.float().cpu(), z), "out-of-place call must not touch z"
+    # the reference's inference contract: inplace_safe + _add_with_inplace returns z + update in z
+    res = m(zg, mask=mask.to(DEV), inplace_safe=True, _add_with_inplace=True)
+    assert res.data_ptr() == zg.data_ptr()
+    _check("trimul z+update", res, z + want, rms_rel=4e-3)
+
+
+def test_trimul_no_mask_is_all_ones():
+    lib()
+    gen = torch.Generator().manual_seed(5)
+    p = _round_params(orc.make_trimul_params(gen, 128, 128))
+    z = orc.round_bf16(orc.make_pair_input(2, (), 40, 128))
+    m = _load(of3pair.TriangleMultiplicationOutgoing(128, 128), p)
+    got = m(z.to(DEV).to(torch.bfloat16))
+    _check("trimul maskless", got, orc.trimul_update(z, None, p, True))
+
+
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("c,d,n,batch", [(128, 32, 64, ()), (128, 32, 100, (2,)), (64, 16, 96, (1, 3))])
+def test_triattn_module(starting, c, d, n, batch):
+    lib()
+    gen = torch.Generator().manual_seed(200 + n)
+    p = _round_params(orc.make_triattn_params(gen, c, d, 4))
+    z = orc.round_bf16(orc.make_pair_input(3, batch, n, c))
+    mask = (torch.rand(*batch, n, n, generator=gen) > 0.2).float()
+    mask[..., 5, :] = 0  # one fully masked row
+    mask[..., :, 7] = 0  # and one fully masked column (a fully masked row for the ending node)
+    m = _load(of3pair.TriangleAttention(c, d, 4, starting=starting), p)
+    print("triattn module", starting, c, d, n, batch, flush=True)
+    got = m(z.to(DEV).to(torch.bfloat16), mask=mask.to(DEV), chunk_size=4, use_lma=True)
+    want = orc.triattn_update(z, mask, p, 4, starting=starting)
+    _check("triattn update", got, want)
+
+
+def test_triattn_transposed_view_input():
+    """PairBlock hands the ending-node module a transposed, non-contiguous view."""
+    lib()
+    gen = torch.Generator().manual_seed(9)
+    p = _round_params(orc.make_triattn_params(gen, 128, 32, 4))
+    z = orc.round_bf16(orc.make_pair_input(4, (1,), 72, 128))
+    mask = orc.tail_padding_mask((1,), 72, 9)
+    m = _load(of3pair.TriangleAttention(128, 32, 4), p)
+    zg = z.to(DEV).to(torch.bfloat16)
+    got = m(zg.transpose(-2, -3), mask=mask.to(DEV).transpose(-1, -2))
+    want = orc.triattn_update(z.transpose(-2, -3), mask.transpose(-1, -2), p, 4)
+    _check("triattn on transposed view", got, want)
+
+
+def _pair_stack(c, ch, d, seed):
+    p = _round_params(orc.make_block_params(seed, c, ch, d, 4))
+    return _load(of3pair.PairStack(c, ch, d, 4), p), p
+
+
+def test_block_config2_n384_padded():
+    """BASELINE config 2: N=384, c_z=128, last 10% of the tokens padded."""
+    lib()
+    n = 384
+    m, p = _pair_stack(128, 128, 32, seed=0)
+    z = orc.round_bf16(orc.make_pair_input(1, (1,), n, 128))
+    mask = orc.tail_padding_mask((1,), n, n - math.ceil(0.9 * n))
+    print("block config 2", flush=True)
+    zg = z.to(DEV).to(torch.bfloat16)
+    got = m(zg, mask.to(DEV))
+    assert torch.equal(zg.float().cpu(), z), "inplace_safe=False must leave the input intact"
+    want = orc.pair_stack_block(z, mask, p, 4, row_chunk=64)
+    _check("block n=384", got, want, rms_rel=1e-2)
+
+
+def test_block_config3_n768():
+    """BASELINE config 3 (headline shape): N=768, all-ones mask; in place."""
+    lib()
+    n = 768
+    m, p = _pair_stack(128, 128, 32, seed=0)
+    z = orc.round_bf16(orc.make_pair_input(1, (1,), n, 128))
+    mask = torch.ones(1, n, n)
+    print("block config 3", flush=True)
+    zg = z.to(DEV).to(torch.bfloat16)
+    got = m(zg, mask.to(DEV), inplace_safe=True)
+    want = orc.pair_stack_block(z, mask, p, 4, row_chunk=32)
+    _check("block n=768", got, want, rms_rel=1e-2)
+
+
+def test_template_stack_config4():
+    """BASELINE config 4: 2 blocks, 4 templates, N=512, c_t=64, 4 heads x 16, each template
+    with its own padded tail (0-20% of the tokens)."""
+    lib()
+    n, t = 512, 4
+    gen = torch.Generator().manual_seed(2)
+    blocks = [_pair_stack(64, 64, 16, seed=s) for s in (10, 11)]
+    z = orc.round_bf16(orc.make_pair_input(1, (1, t), n, 64))
+    pad = torch.randint(0, 103, (1, t), generator=gen)
+    mask = orc.tail_padding_mask((1, t), n, pad)
+    print("template config 4 pads", pad.tolist(), flush=True)
+    zg = z.to(DEV).to(torch.bfloat16)
+    mg = mask.to(DEV)
+    for m, _ in blocks:
+        zg = m(zg, mg, inplace_safe=True)
+    want = orc.template_pair_stack(z, mask, [p for _, p in blocks], 4, row_chunk=64)
+    _check("template stack", zg, want, rms_rel=1.5e-2)
