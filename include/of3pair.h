@@ -76,7 +76,8 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
                     int64_t CH, int outgoing, void* stream);
 
 /* x[b][c][i][j] = sum_k a[b][c][i][k] * b[b][c][j][k]  over the padded planes.
- * variant: 0 = automatic, 1/2/3 = 128x128 / 256x128 / 256x256 work-group tile. */
+ * variant: 0 = automatic; 1/2/3 = 128x128 / 256x128 / 256x256 tile, one per work-group;
+ * 4/5/6 = 256x192 / 256x256 / 256x128 tiles, persistent work-groups, direct-to-LDS ring. */
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream);
 

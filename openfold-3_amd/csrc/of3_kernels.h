@@ -29,9 +29,13 @@ struct TrimulProjArgs {
 };
 hipError_t trimul_proj_launch(const TrimulProjArgs& args, int C, int CH, hipStream_t stream);
 
-// variant: 1 = 128x128, 2 = 256x128, 3 = 256x256 work-group tile
+// variant: 1 = 128x128, 2 = 256x128, 3 = 256x256 work-group tile (one tile per work-group)
 hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
                                   hipStream_t stream);
+// variant: 4 = 256x192, 5 = 256x256, 6 = 256x128 tiles, persistent work-groups with a
+// direct-to-LDS operand ring
+hipError_t trimul_contract_pipe_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
+                                       hipStream_t stream);
 
 struct TrimulOutArgs {
   const bf16_t* x;  // [B][CH][Np][Np]

@@ -22,6 +22,7 @@ SOURCES = [
     "of3pair_api.hip",
     "trimul_proj.hip",
     "trimul_contract.hip",
+    "trimul_contract_pipe.hip",
     "trimul_out.hip",
     "triattn_proj.hip",
     "triattn_flash.hip",

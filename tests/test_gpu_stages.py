@@ -30,12 +30,12 @@ def _ln(x, w, b):
 
 
 # ---------------------------------------------------------------------------------------
-@pytest.mark.parametrize("variant", [1, 2, 3])
-@pytest.mark.parametrize("n", [128, 384])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("n", [128, 384, 640])
 def test_contract(variant, n):
     L = lib()
     gen = _gen(n + variant)
-    planes, B, CH = 64, 1, 64
+    planes, B, CH = 64, 1, 64  # 64 planes: enough tiles that persistent work-groups take several each
     np_ = L.of3_padded_n(n)
     a = bf(_randn(gen, planes, np_, np_))
     b = bf(_randn(gen, planes, np_, np_))
