@@ -67,17 +67,17 @@ int64_t of3_padded_n(int64_t n);
 /* Bytes of scratch of3_trimul_fwd needs: a, b, x = 3 * B*CH*NP*NP bf16. */
 int64_t of3_trimul_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t CH);
 
-/* a, b [B][CH][NP][NP]: gated, masked projections, channel-major and contiguous along
- * the contracted index: a[b][c][i][k] = a_ref[b,i,k,c] (outgoing) or a_ref[b,k,i,c]
- * (incoming); entries with k >= N are zero, rows i >= N are left untouched. */
+/* a, b: gated, masked projections, channel-major in "k-panels" of 32 contracted indices:
+ * shape [B][CH][NP/32][NP][32], a[b][c][k/32][i][k%32] = a_ref[b,i,k,c] (outgoing) or
+ * a_ref[b,k,i,c] (incoming); entries with k >= N are zero, rows i >= N are left untouched. */
 int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
                     const void* ln_in_w, const void* ln_in_b, const void* w_a_p, const void* w_a_g,
                     const void* w_b_p, const void* w_b_g, void* a, void* b, int64_t B, int64_t N, int64_t C,
                     int64_t CH, int outgoing, void* stream);
 
-/* x[b][c][i][j] = sum_k a[b][c][i][k] * b[b][c][j][k]  over the padded planes.
- * variant: 0 = automatic; 1/2/3 = 128x128 / 256x128 / 256x256 tile, one per work-group;
- * 4/5/6 = 256x192 / 256x256 / 256x128 tiles, persistent work-groups, direct-to-LDS ring. */
+/* x[b][c][i][j] = sum_k a[b][c][i][k] * b[b][c][j][k] over the padded planes; a, b in the
+ * k-panel layout above, x row-major [B][CH][NP][NP].
+ * variant: 0 = automatic; 1 / 2 = 256x192 / 256x128 output tiles. */
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream);
 

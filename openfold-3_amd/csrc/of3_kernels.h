@@ -24,18 +24,15 @@ struct TrimulProjArgs {
   PairView z_view, mask_view;
   const bf16_t *ln_w, *ln_b;                  // [C]
   const bf16_t *w_ap, *w_ag, *w_bp, *w_bg;    // [CH][C]
-  bf16_t *a, *b;                              // [B][CH][Np][Np]
+  bf16_t *a, *b;                              // [B][CH][Np/32][Np][32]  (k-panels)
   int B, N, Np;
 };
 hipError_t trimul_proj_launch(const TrimulProjArgs& args, int C, int CH, hipStream_t stream);
 
-// variant: 1 = 128x128, 2 = 256x128, 3 = 256x256 work-group tile (one tile per work-group)
+// a, b: k-panel layout [planes][Np/32][Np][32]; x: row-major [planes][Np][Np].
+// variant: 1 = 256x192 output tiles, 2 = 256x128
 hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
                                   hipStream_t stream);
-// variant: 4 = 256x192, 5 = 256x256, 6 = 256x128 tiles, persistent work-groups with a
-// direct-to-LDS operand ring
-hipError_t trimul_contract_pipe_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
-                                       hipStream_t stream);
 
 struct TrimulOutArgs {
   const bf16_t* x;  // [B][CH][Np][Np]

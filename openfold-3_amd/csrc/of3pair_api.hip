@@ -53,9 +53,10 @@ inline const of3::bf16_t* bf(const void* p) { return static_cast<const of3::bf16
 inline of3::bf16_t* bf(void* p) { return static_cast<of3::bf16_t*>(p); }
 
 inline int contract_variant_auto(int64_t Np) {
-  // 256x128 tiles divide N = 768 into 9 full waves over 256 CUs; small problems keep the
-  // 128x128 tile so that every CU still gets work.
-  return Np >= 512 ? 2 : 1;
+  // 256x192 tiles: 12 per plane at Np = 768, i.e. 6 tiles for each of 256 persistent
+  // work-groups with 128 planes
+  (void)Np;
+  return 1;
 }
 
 }  // namespace
@@ -118,14 +119,12 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
 
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream) {
-  if (B < 1 || N < 1 || (CH != 128 && CH != 64) || variant < 0 || variant > 7) return OF3_EINVAL;
+  if (B < 1 || N < 1 || (CH != 128 && CH != 64) || variant < 0 || variant > 2) return OF3_EINVAL;
   if (!a || !b || !x || !aligned16(a) || !aligned16(b) || !aligned16(x)) return OF3_EINVAL;
   const int64_t Np = padded(N);
   if (variant == 0) variant = contract_variant_auto(Np);
-  hipError_t e = variant >= 4 ? of3::trimul_contract_pipe_launch(bf(a), bf(b), bf(x), (int)(B * CH), (int)Np, variant,
-                                                                  static_cast<hipStream_t>(stream))
-                             : of3::trimul_contract_launch(bf(a), bf(b), bf(x), (int)(B * CH), (int)Np, variant,
-                                                             static_cast<hipStream_t>(stream));
+  hipError_t e = of3::trimul_contract_launch(bf(a), bf(b), bf(x), (int)(B * CH), (int)Np, variant,
+                                             static_cast<hipStream_t>(stream));
   return e == hipSuccess ? OF3_OK : fail_hip(e);
 }
 

@@ -1,15 +1,36 @@
 // Triangle-multiplication contraction: for every (batch, channel) plane
 //     X[i][j] = sum_k A[i][k] * Bm[j][k]
-// with A, Bm, X dense row-major [Np][Np] bf16 planes (Np a multiple of 128, zero-padded
-// along k by the projection kernel).  This is the reference's per-channel matrix product
-// of _combine_projections (triangular_multiplicative_update.py:71-97); the projection
-// kernel has already laid both operands out k-contiguous for either direction, so one
-// "row times row" kernel serves the outgoing and the incoming update.
+// i.e. the reference's per-channel matrix product of _combine_projections
+// (triangular_multiplicative_update.py:71-97).  The projection pass has already laid both
+// operands out k-contiguous for either direction, so one "row times row" kernel serves the
+// outgoing and the incoming update.
 //
-// MFMA bound.  Work-group = 4 waves, tile BM (j) x BN (i); k is consumed 64 at a time
-// through a double-buffered, XOR-swizzled LDS stage filled with coalesced 16-byte loads.
-// The j side is the MFMA M side so that a lane ends up owning 16*TM consecutive j of one
-// output row i and can store them as 16-byte vectors.
+// Operand layout ("k-panels"): plane[kb][row][32] bf16 with kb = k / 32, Np rows per panel.
+// The 16 rows x 32 k-values that one direct-to-LDS wave instruction moves are then 1 KB of
+// contiguous memory, and a whole pipeline stage is two contiguous runs.
+// Output layout: plain row-major X[plane][i][j], Np x Np.
+//
+// Organisation (MFMA-bound kernel, tuned for the MI355X memory system):
+//  * persistent work-groups (one per CU, 4 waves, each wave a 128 x BN/2 sub-tile held in
+//    AGPRs) walk a list of 256 x BN output tiles; tiles of one plane are dealt to
+//    work-groups of one XCD so that operand re-reads hit that XCD's L2;
+//  * operands stream global -> LDS with direct-to-LDS loads (no VGPR staging) through a
+//    ring of 4 stages of 32 k-values that runs across tile boundaries, so the next tile's
+//    operands are in flight while a tile's accumulators are converted and stored;
+//  * one barrier per stage, placed between the stage's two k-steps: by then every wave
+//    holds the stage's last fragments in registers, so the stage's buffer is refilled at
+//    once (stage s+4) and the first fragments of stage s+1 are fetched under the second
+//    k-step's MFMAs; the refill's loads are issued one by one between those MFMAs;
+//  * the k-blocks of a tile are visited in rotated order, starting at (tm + tn) mod nk:
+//    tiles that share operand rows never ask for the same cache line at the same time (the
+//    first asks HBM, the others find the line in L2 a stage or two later);
+//  * the j side is the MFMA M side with permuted rows so that a lane ends up owning 64
+//    consecutive j of one output row; the epilogue transposes 32-row blocks through a
+//    wave-private LDS region and stores whole 256-byte row segments.
+//
+// LDS layout of a stage: rows of 4 chunks of 16 bytes, slot = row*4 + (chunk ^ key(row)).
+// A direct-to-LDS instruction fills 64 consecutive slots (lane l -> slot base + l), so the
+// lane chooses its *global* chunk as chunk' ^ key(row).
 #include "of3_device.h"
 #include "of3_kernels.h"
 
@@ -17,175 +38,285 @@ namespace of3 {
 
 namespace {
 
-constexpr int kBK = 64;  // k per stage (128 bytes per row = 8 chunks)
+#define OF3_GLOBAL_AS __attribute__((address_space(1)))
+#define OF3_LDS_AS __attribute__((address_space(3)))
 
-template <int HB>
-__device__ __forceinline__ int key_m(int row) { return (row & 3) | (((row >> HB) & 1) << 2); }
-__device__ __forceinline__ int key_n(int row) { return row & 7; }
+constexpr int kBK = 32;  // k per stage = one k-panel
+constexpr int kNS = 4;   // ring depth
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
-__global__ __launch_bounds__(256) void contract_kernel(const bf16_t* __restrict__ pm,  // j side [batch][Np][Np]
-                                                       const bf16_t* __restrict__ pn,  // i side
-                                                       bf16_t* __restrict__ x, int Np, int tiles_m,
-                                                       int tiles_n, int total, int per_xcd) {
-  static_assert(WAVES_M * WAVES_N == 4, "four waves per work-group");
-  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+// j side: rows are read in the permuted order {x..x+3, x+64..x+67, x+4..}: (row&1, key)
+// must differ within each group of 8 and (row&3, key) within each group of 16 lanes
+__device__ __forceinline__ int key_m(int row) { return (((row >> 1) ^ (row >> 2)) & 1) | (((row >> 6) & 1) << 1); }
+// i side: natural rows
+__device__ __forceinline__ int key_n(int row) { return ((row >> 1) ^ (row >> 3)) & 3; }
+
+__device__ __forceinline__ void compiler_fence() { __asm__ volatile("" ::: "memory"); }
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  // gfx9 encoding: vmcnt[3:0] | expcnt[6:4]=7 | lgkmcnt[11:8]=15 | vmcnt[5:4] at [15:14]
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 15) | 0x70 | 0xF00 | ((N >> 4) << 14));
+}
+
+template <int BN>
+__global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restrict__ pm,  // j side planes (b)
+                                                          const bf16_t* __restrict__ pn,  // i side planes (a)
+                                                          bf16_t* __restrict__ x, int Np, int tiles_m, int tiles_n,
+                                                          int total_tiles, int tiles_per_xcd) {
+  constexpr int BM = 256;
+  constexpr int WM = BM / 2, WN = BN / 2;
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int HB = (TM == 4) ? 6 : (TM == 2 ? 5 : 4);  // log2(16*TM)
-  static_assert(TM == 1 || TM == 2 || TM == 4, "TM");
-  constexpr int STAGE = (BM + BN) * 8;  // u32x4 slots per stage
+  static_assert(TM == 4, "a wave's j range is 128 wide");
+  constexpr int ROWS = BM + BN;
+  constexpr int STAGE = ROWS * 4;       // u32x4 slots per stage
+  constexpr int MI = BM / 16 / 4;       // j-side direct-to-LDS instructions per wave (16 rows each)
+  constexpr int NI = BN / 16 / 4;       // i-side
+  constexpr int IPW = MI + NI;
+  constexpr int NMMA = TM * TN;
+  static_assert(IPW <= NMMA, "a stage's loads are issued between the MFMAs of one k-step");
+  static_assert(2 * IPW + 8 * TN < 64, "vmcnt budget");
 
   extern __shared__ u32x4_t lds[];
 
-  const int logical = xcd_logical_block(blockIdx.x, per_xcd);
-  if (logical >= total) return;
-  const int per_plane = tiles_m * tiles_n;
-  const int plane = logical / per_plane;
-  const int rem = logical - plane * per_plane;
-  const int tm = rem / tiles_n, tn = rem - tm * tiles_n;
-
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
-  const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
 
-  const size_t plane_off = (size_t)plane * Np * Np;
-  const bf16_t* gm = pm + plane_off;
-  const bf16_t* gn = pn + plane_off;
+  // ---- tile list of this work-group: XCD x owns logical tiles [x*tiles_per_xcd, ...)
+  const int xcd = blockIdx.x & 7, slot_in_xcd = blockIdx.x >> 3, wgs_per_xcd = gridDim.x >> 3;
+  const int xcd_first = xcd * tiles_per_xcd;
+  int xcd_count = total_tiles - xcd_first;
+  xcd_count = xcd_count < 0 ? 0 : (xcd_count > tiles_per_xcd ? tiles_per_xcd : xcd_count);
+  const int my_tiles = slot_in_xcd < xcd_count ? (xcd_count - slot_in_xcd + wgs_per_xcd - 1) / wgs_per_xcd : 0;
+  if (my_tiles == 0) return;
+  const int per_plane = tiles_m * tiles_n;
+  const int nk = Np / kBK;
+  const size_t panel_bytes = (size_t)Np * kBK * 2;
 
-  // ---- global -> register staging: thread covers row (tid/8 + 32*rr), chunk tid%8
-  constexpr int RM = BM / 32, RN = BN / 32;
-  const int ld_row = tid >> 3, ld_chunk = tid & 7;
-  const bf16_t* src_m[RM];
-  const bf16_t* src_n[RN];
-  int dst_m[RM], dst_n[RN];
+  auto tile_coords = [&](int t_local, int& plane, int& tm, int& tn) {
+    const int logical = xcd_first + slot_in_xcd + t_local * wgs_per_xcd;
+    plane = logical / per_plane;
+    const int rem = logical - plane * per_plane;
+    tm = rem / tiles_n;
+    tn = rem - tm * tiles_n;
+  };
+
+  // ---- direct-to-LDS issue.  One instruction = 16 rows x 64 bytes (1 KB contiguous in a
+  // k-panel); lane l -> row l/4, LDS chunk' = l%4, global chunk = chunk' ^ key(row).  The key
+  // depends on the lane and on one bit of the (wave-uniform) row block, so two per-lane byte
+  // offsets per side serve every instruction; everything else lives in scalar registers.
+  const int lrow = lane >> 2, lchunk = lane & 3;
+  const uint32_t off_m[2] = {(uint32_t)(lrow * 64 + 16 * (lchunk ^ key_m(lrow))),
+                             (uint32_t)(lrow * 64 + 16 * (lchunk ^ key_m(lrow + 64)))};
+  const uint32_t off_n[2] = {(uint32_t)(lrow * 64 + 16 * (lchunk ^ key_n(lrow))),
+                             (uint32_t)(lrow * 64 + 16 * (lchunk ^ key_n(lrow + 16)))};
+  const char* dma_base[IPW];  // first row of each 16-row block in panel 0 of the tile being loaded
+  int issue_tile = 0, issue_kb = 0, issue_left = nk, issue_buf = 0;
+  auto dma_setup_tile = [&](int t_local) {
+    int plane, tm, tn;
+    tile_coords(t_local < my_tiles ? t_local : my_tiles - 1, plane, tm, tn);  // past the end: reload the last tile
+    const size_t plane_off = (size_t)plane * Np * Np * 2;
+    const int rows_m_left = Np - tm * BM, rows_n_left = Np - tn * BN;
 #pragma unroll
-  for (int r = 0; r < RM; ++r) {
-    const int row = ld_row + 32 * r;
-    int grow = tm * BM + row;
-    grow = grow < Np ? grow : Np - 1;
-    src_m[r] = gm + (size_t)grow * Np + ld_chunk * 8;
-    dst_m[r] = row * 8 + (ld_chunk ^ key_m<HB>(row));
-  }
+    for (int n = 0; n < MI; ++n) {
+      const int rb = 16 * (wave * MI + n);
+      const int rbc = rb + 16 <= rows_m_left ? rb : rows_m_left - 16;  // whole blocks stay inside the plane
+      dma_base[n] = reinterpret_cast<const char*>(pm) + plane_off + (size_t)(tm * BM + rbc) * (kBK * 2);
+    }
 #pragma unroll
-  for (int r = 0; r < RN; ++r) {
-    const int row = ld_row + 32 * r;
-    int grow = tn * BN + row;
-    grow = grow < Np ? grow : Np - 1;
-    src_n[r] = gn + (size_t)grow * Np + ld_chunk * 8;
-    dst_n[r] = BM * 8 + row * 8 + (ld_chunk ^ key_n(row));
-  }
+    for (int n = 0; n < NI; ++n) {
+      const int rb = 16 * (wave * NI + n);
+      const int rbc = rb + 16 <= rows_n_left ? rb : rows_n_left - 16;
+      dma_base[MI + n] = reinterpret_cast<const char*>(pn) + plane_off + (size_t)(tn * BN + rbc) * (kBK * 2);
+    }
+    issue_kb = (tm + tn) % nk;  // rotated start
+    issue_left = nk;
+  };
+  auto issue_one = [&](int n) {
+    u32x4_t* buf = lds + issue_buf * STAGE;
+    const char* src = dma_base[n] + (size_t)issue_kb * panel_bytes;
+    if (n < MI) {
+      const int rb = 16 * (wave * MI + n);
+      __builtin_amdgcn_global_load_lds((const void OF3_GLOBAL_AS*)(src + off_m[(rb >> 6) & 1]),
+                                       (void OF3_LDS_AS*)(buf + rb * 4), 16, 0, 0);
+    } else {
+      const int rb = 16 * (wave * NI + (n - MI));
+      __builtin_amdgcn_global_load_lds((const void OF3_GLOBAL_AS*)(src + off_n[(rb >> 4) & 1]),
+                                       (void OF3_LDS_AS*)(buf + (BM + rb) * 4), 16, 0, 0);
+    }
+  };
+  auto issue_advance = [&]() {
+    issue_buf = (issue_buf + 1) & (kNS - 1);
+    issue_kb = issue_kb + 1 == nk ? 0 : issue_kb + 1;
+    if (--issue_left == 0) dma_setup_tile(++issue_tile);
+  };
 
-  // ---- MFMA operand fetch addresses (slot of chunk 0; chunk index XOR-ed per k-step)
-  int am_row[TM], am_key[TM], bn_row[TN], bn_key[TN];
+  // ---- MFMA operand fetch slots.  k-step ks, lane-half lh reads chunk (2*ks + lh) ^ key;
+  // row*4 has its two low bits clear, so slot(ks) = slot(0) ^ (2*ks).
+  int am_slot[TM], bn_slot[TN];
   {
     const int g = l32 >> 3, hb = (l32 >> 2) & 1, e = l32 & 3;
 #pragma unroll
     for (int mt = 0; mt < TM; ++mt) {
       const int row = wm0 + 16 * TM * hb + 16 * mt + 4 * g + e;
-      am_row[mt] = row * 8;
-      am_key[mt] = key_m<HB>(row);
+      am_slot[mt] = row * 4 + (lh ^ key_m(row));
     }
 #pragma unroll
     for (int nt = 0; nt < TN; ++nt) {
       const int row = wn0 + 32 * nt + l32;
-      bn_row[nt] = BM * 8 + row * 8;
-      bn_key[nt] = key_n(row);
+      bn_slot[nt] = (BM + row) * 4 + (lh ^ key_n(row));
     }
   }
+  auto fetch = [&](const u32x4_t* buf, int ks, u32x4_t (&af)[TM], u32x4_t (&bfr)[TN]) {
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) af[mt] = buf[am_slot[mt] ^ (2 * ks)];
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) bfr[nt] = buf[bn_slot[nt] ^ (2 * ks)];
+  };
 
   f32x16_t acc[TM][TN];
 #pragma unroll
   for (int mt = 0; mt < TM; ++mt)
 #pragma unroll
     for (int nt = 0; nt < TN; ++nt) acc[mt][nt] = zero16();
-
-  u32x4_t st_m[RM], st_n[RN];
-  const int nk = Np / kBK;
-
-  // prologue: stage 0
+  auto mma = [&](const u32x4_t (&af)[TM], const u32x4_t (&bfr)[TN]) {
 #pragma unroll
-  for (int r = 0; r < RM; ++r) st_m[r] = *reinterpret_cast<const u32x4_t*>(src_m[r]);
+    for (int mt = 0; mt < TM; ++mt)
 #pragma unroll
-  for (int r = 0; r < RN; ++r) st_n[r] = *reinterpret_cast<const u32x4_t*>(src_n[r]);
+      for (int nt = 0; nt < TN; ++nt) acc[mt][nt] = mfma_32x32x16(af[mt], bfr[nt], acc[mt][nt]);
+  };
+  // the same, with the refill's loads issued in between
+  auto mma_and_issue = [&](const u32x4_t (&af)[TM], const u32x4_t (&bfr)[TN]) {
+    int n = 0;
 #pragma unroll
-  for (int r = 0; r < RM; ++r) lds[dst_m[r]] = st_m[r];
+    for (int mt = 0; mt < TM; ++mt)
 #pragma unroll
-  for (int r = 0; r < RN; ++r) lds[dst_n[r]] = st_n[r];
-  __syncthreads();
-
-  for (int kt = 0; kt < nk; ++kt) {
-    const u32x4_t* cur = lds + (kt & 1) * STAGE;
-    u32x4_t* nxt = lds + ((kt + 1) & 1) * STAGE;
-    const bool more = (kt + 1) < nk;
-    if (more) {
-      const int koff = (kt + 1) * kBK;
-#pragma unroll
-      for (int r = 0; r < RM; ++r) st_m[r] = *reinterpret_cast<const u32x4_t*>(src_m[r] + koff);
-#pragma unroll
-      for (int r = 0; r < RN; ++r) st_n[r] = *reinterpret_cast<const u32x4_t*>(src_n[r] + koff);
-    }
-#pragma unroll
-    for (int ks = 0; ks < kBK / 16; ++ks) {
-      const int ch = 2 * ks + lh;
-      u32x4_t af[TM], bfr[TN];
-#pragma unroll
-      for (int mt = 0; mt < TM; ++mt) af[mt] = cur[am_row[mt] + (ch ^ am_key[mt])];
-#pragma unroll
-      for (int nt = 0; nt < TN; ++nt) bfr[nt] = cur[bn_row[nt] + (ch ^ bn_key[nt])];
-#pragma unroll
-      for (int mt = 0; mt < TM; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < TN; ++nt) acc[mt][nt] = mfma_32x32x16(af[mt], bfr[nt], acc[mt][nt]);
-    }
-    if (more) {
-#pragma unroll
-      for (int r = 0; r < RM; ++r) nxt[dst_m[r]] = st_m[r];
-#pragma unroll
-      for (int r = 0; r < RN; ++r) nxt[dst_n[r]] = st_n[r];
-    }
-    __syncthreads();
-  }
-
-  // ---- epilogue: lane (i = column l32, half lh) owns j = j0 + 16*mt + v
-  bf16_t* xo = x + plane_off;
-#pragma unroll
-  for (int nt = 0; nt < TN; ++nt) {
-    const int i = tn * BN + wn0 + 32 * nt + l32;
-    if (i >= Np) continue;
-#pragma unroll
-    for (int mt = 0; mt < TM; ++mt) {
-      const int j = tm * BM + wm0 + 16 * TM * lh + 16 * mt;
-      if (j >= Np) continue;
-      u32x4_t lo, hi;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        lo[q] = pack_bf16(acc[mt][nt][2 * q], acc[mt][nt][2 * q + 1]);
-        hi[q] = pack_bf16(acc[mt][nt][8 + 2 * q], acc[mt][nt][8 + 2 * q + 1]);
+      for (int nt = 0; nt < TN; ++nt) {
+        acc[mt][nt] = mfma_32x32x16(af[mt], bfr[nt], acc[mt][nt]);
+        if (n < IPW) issue_one(n++);
       }
-      u32x4_t* dst = reinterpret_cast<u32x4_t*>(xo + (size_t)i * Np + j);
-      dst[0] = lo;
-      dst[1] = hi;
-    }
+    issue_advance();
+  };
+
+  // ---- prologue: fill the ring, make stage 0 visible, fetch its first fragments
+  dma_setup_tile(0);
+#pragma unroll
+  for (int s = 0; s < kNS; ++s) {
+#pragma unroll
+    for (int n = 0; n < IPW; ++n) issue_one(n);
+    issue_advance();
   }
+  wait_vmcnt<3 * IPW>();
+  compiler_fence();
+  __builtin_amdgcn_s_barrier();
+  compiler_fence();
+
+  u32x4_t a0[TM], b0[TN], a1[TM], b1[TN];
+  fetch(lds, 0, a0, b0);
+
+  int cur_buf = 0;
+  bool stores_pending = false;  // the previous tile's full set of output stores may still be in the queue
+  for (int t_local = 0; t_local < my_tiles; ++t_local) {
+    for (int kb = 0; kb < nk; ++kb) {
+      const u32x4_t* cur = lds + cur_buf * STAGE;
+      fetch(cur, 1, a1, b1);
+      mma(a0, b0);
+      __builtin_amdgcn_sched_barrier(0);
+
+      // This wave holds all of stage s in registers.  Stages s+1..s+3 are in flight and
+      // stage s+1 must have landed, in every wave (hence the barrier).  VMEM operations
+      // retire in order, so "at most n outstanding" means everything older than the newest
+      // n has completed.  The output stores of a tile that has just ended sit in the same
+      // queue behind the loads of three stages; during the next three stages they are
+      // simply allowed to stay outstanding, otherwise the wait would drain the whole ring
+      // at every tile boundary.
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): a1/b1 have arrived
+      if (stores_pending && kb < 3) wait_vmcnt<2 * IPW + 8 * TN>();
+      else wait_vmcnt<2 * IPW>();
+      compiler_fence();
+      __builtin_amdgcn_s_barrier();
+      compiler_fence();
+      __builtin_amdgcn_sched_barrier(0);
+
+      // after the barrier no wave reads the buffer of stage s any more: refill it with
+      // stage s+4 while the second k-step's MFMAs run
+      cur_buf = (cur_buf + 1) & (kNS - 1);
+      fetch(lds + cur_buf * STAGE, 0, a0, b0);  // after the last stage this reads data that is never used
+      mma_and_issue(a1, b1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- tile finished.  Each wave transposes its 32-row blocks through a private 8 KB
+    // LDS region (row-major [32 i][128 j] bf16, 16-byte chunks XOR-swizzled by the row) and
+    // writes whole 256-byte row segments.
+    int plane, tm, tn;
+    tile_coords(t_local, plane, tm, tn);
+    bf16_t* xo = x + (size_t)plane * Np * Np;
+    u32x4_t* epi = lds + kNS * STAGE + wave * 512;
+    const int jbase = tm * BM + wm0;
+    int n_stores = 0;
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) {
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+        u32x4_t lo, hi;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          lo[q] = pack_bf16(acc[mt][nt][2 * q], acc[mt][nt][2 * q + 1]);
+          hi[q] = pack_bf16(acc[mt][nt][8 + 2 * q], acc[mt][nt][8 + 2 * q + 1]);
+        }
+        const int chunk = 8 * lh + 2 * mt;  // j-local = 64*lh + 16*mt + (0..15)
+        epi[l32 * 16 + (chunk ^ (l32 & 7))] = lo;
+        epi[l32 * 16 + ((chunk + 1) ^ (l32 & 7))] = hi;
+        acc[mt][nt] = zero16();
+      }
+      // Np is a multiple of 128, so a 32-row block and the wave's 128 columns are either
+      // entirely inside the plane or entirely outside: the guard is wave-uniform
+      const int i0 = tn * BN + wn0 + 32 * nt;
+      if (i0 < Np && jbase < Np) {
+#pragma unroll
+        for (int rr = 0; rr < 8; ++rr) {
+          const int row = 4 * rr + (lane >> 4), chunk = lane & 15;
+          const u32x4_t v = epi[row * 16 + (chunk ^ (row & 7))];
+          *reinterpret_cast<u32x4_t*>(xo + (size_t)(i0 + row) * Np + jbase + 8 * chunk) = v;
+        }
+        n_stores += 8;
+      }
+      __builtin_amdgcn_sched_barrier(0);  // one block at a time keeps the live registers low
+    }
+    // only a complete set of stores is accounted for exactly; otherwise the next waits
+    // simply cover them too (waiting for more than necessary is always safe)
+    stores_pending = (n_stores == 8 * TN);
+  }
+  wait_vmcnt<0>();  // loads issued past the end must not outlive the work-group's LDS
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BN>
 hipError_t launch_contract(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, hipStream_t stream) {
-  auto kern = contract_kernel<BM, BN, WAVES_M, WAVES_N>;
-  const int tiles_m = (Np + BM - 1) / BM, tiles_n = (Np + BN - 1) / BN;
-  const long total = (long)planes * tiles_m * tiles_n;
-  const int per_xcd = (int)((total + 7) / 8);
-  const size_t smem = 2 * (size_t)(BM + BN) * 8 * sizeof(u32x4_t);
-  static bool attr_set = false;  // idempotent; a race only repeats the same call
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  constexpr int BM = 256;
+  auto kern = contract_kernel<BN>;
+  const size_t smem = ((size_t)kNS * (BM + BN) * 4 + 4 * 512) * sizeof(u32x4_t);  // ring + epilogue staging
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
-    attr_set = true;
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem);
+    if (e != hipSuccess) return e;
+    cus = n;
   }
+  const int tiles_m = (Np + BM - 1) / BM, tiles_n = (Np + BN - 1) / BN;
+  const int total = planes * tiles_m * tiles_n;
+  const int tiles_per_xcd = (total + 7) / 8;
+  int grid = (cus / 8) * 8;  // a multiple of the 8 XCDs
+  if (grid < 8) grid = 8;
   // M side (register-contiguous output index j) is b, N side (lane index i) is a
-  hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(256), smem, stream, b, a, x, Np, tiles_m, tiles_n, (int)total,
-                     per_xcd);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, stream, b, a, x, Np, tiles_m, tiles_n, total, tiles_per_xcd);
   return hipGetLastError();
 }
 
@@ -195,11 +326,9 @@ hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, i
                                   hipStream_t stream) {
   switch (variant) {
     case 1:
-      return launch_contract<128, 128, 2, 2>(a, b, x, planes, Np, stream);
+      return launch_contract<192>(a, b, x, planes, Np, stream);
     case 2:
-      return launch_contract<256, 128, 2, 2>(a, b, x, planes, Np, stream);
-    case 3:
-      return launch_contract<256, 256, 2, 2>(a, b, x, planes, Np, stream);
+      return launch_contract<128>(a, b, x, planes, Np, stream);
     default:
       return hipErrorInvalidValue;
   }

@@ -1,16 +1,17 @@
 // Triangle-multiplication input pass: LayerNorm(z) and the four gated projections
 //     a = mask * sigmoid(zn Wag^T) * (zn Wap^T),   b = mask * sigmoid(zn Wbg^T) * (zn Wbp^T)
-// (triangular_multiplicative_update.py:485-493), written channel-major and k-contiguous
-// as a[b][c][r][k] so that the contraction is a plain "row times row" product for both
-// directions: the caller's PairView makes (r, k) = (i, k) for the outgoing update and
-// (r, k) = (i, k) of the transposed tensor for the incoming one.
+// (triangular_multiplicative_update.py:485-493), written channel-major in the k-panel
+// layout a[b][c][k/32][r][k%32] the contraction kernel streams from, so that the
+// contraction is a plain "row times row" product for both directions: the caller's PairView
+// makes (r, k) = (i, k) for the outgoing update and (r, k) = (i, k) of the transposed tensor
+// for the incoming one.
 //
 // HBM bound (reads z once, writes a and b once).  Persistent work-groups keep their slice
 // of the four weight matrices in registers as MFMA A operands; each tile of 128
 // positions is normalised in registers, staged once in LDS as bf16 and consumed as the
 // MFMA B operand by all four waves.  Position 4*l+t of the tile sits in column l of
 // position-tile t, so after four tiles a lane owns 4 consecutive positions of a channel
-// and stores them as one 8-byte vector (256 contiguous bytes per 32 lanes).
+// and stores them as one 8-byte vector (8 lanes fill one 64-byte panel row).
 #include "of3_device.h"
 #include "of3_kernels.h"
 
@@ -139,7 +140,9 @@ __global__ __launch_bounds__(256) void trimul_proj_kernel(TrimulProjArgs p, int 
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int ch = 32 * ot + 8 * (v >> 2) + 4 * lh + (v & 3);
-        bf16_t* dst = out + (((size_t)b * CH + ch) * Np + r) * Np + k0 + 4 * l32;
+        // k-panel layout: plane[k / 32][row][k % 32]
+        const int k = k0 + 4 * l32;
+        bf16_t* dst = out + ((size_t)b * CH + ch) * Np * Np + (size_t)(k >> 5) * (Np * 32) + r * 32 + (k & 31);
         u32x2_t w2 = {pk[0][v], pk[1][v]};
         *reinterpret_cast<u32x2_t*>(dst) = w2;
       }

@@ -22,7 +22,6 @@ SOURCES = [
     "of3pair_api.hip",
     "trimul_proj.hip",
     "trimul_contract.hip",
-    "trimul_contract_pipe.hip",
     "trimul_out.hip",
     "triattn_proj.hip",
     "triattn_flash.hip",

@@ -30,8 +30,14 @@ def _ln(x, w, b):
 
 
 # ---------------------------------------------------------------------------------------
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
-@pytest.mark.parametrize("n", [128, 384, 640])
+def _to_panels(t):
+    """[..., rows, k] -> k-panel layout [..., k/32, rows, 32]"""
+    *lead, rows, k = t.shape
+    return t.reshape(*lead, rows, k // 32, 32).transpose(-2, -3).contiguous()
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("n", [128, 384, 640, 768])
 def test_contract(variant, n):
     L = lib()
     gen = _gen(n + variant)
@@ -41,7 +47,8 @@ def test_contract(variant, n):
     b = bf(_randn(gen, planes, np_, np_))
     x = torch.full((planes, np_, np_), float("nan"), dtype=torch.bfloat16, device=DEV)
     print("contract variant", variant, "n", n, flush=True)
-    st = L.of3_trimul_contract(a.data_ptr(), b.data_ptr(), x.data_ptr(), B, n, CH, variant, stream())
+    ap, bp = _to_panels(a), _to_panels(b)
+    st = L.of3_trimul_contract(ap.data_ptr(), bp.data_ptr(), x.data_ptr(), B, n, CH, variant, stream())
     assert st == 0, L.of3_status_string(st)
     torch.cuda.synchronize()
     want = torch.bmm(a.float(), b.float().transpose(1, 2))
@@ -69,7 +76,7 @@ def test_trimul_proj(outgoing, C, n, B):
     z = bf(_randn(gen, B, n, n, C))
     mask = (torch.rand(B, n, n, generator=gen) > 0.3).float().to(DEV)
     w = _trimul_weights(gen, C, CH)
-    a = torch.full((B, CH, np_, np_), float("nan"), dtype=torch.bfloat16, device=DEV)
+    a = torch.full((B, CH, np_ // 32, np_, 32), float("nan"), dtype=torch.bfloat16, device=DEV)
     b = torch.full_like(a, float("nan"))
     print("trimul_proj", outgoing, C, n, B, flush=True)
     st = L.of3_trimul_proj(z.data_ptr(), s3(z), mask.data_ptr(), s3(mask), w["ln_in_w"].data_ptr(),
@@ -82,7 +89,8 @@ def test_trimul_proj(outgoing, C, n, B):
     ar = m * torch.sigmoid(zn @ w["a_g"].float().t()) * (zn @ w["a_p"].float().t())
     br = m * torch.sigmoid(zn @ w["b_g"].float().t()) * (zn @ w["b_p"].float().t())
     for name, got, ref in (("a", a, ar), ("b", b, br)):
-        # expected layout [b][c][r][k]: outgoing (r,k) = (i,k); incoming (r,k) from ref[b,k,r,c]
+        got = got.transpose(-2, -3).reshape(B, CH, np_, np_)  # k-panels -> [b][c][r][k]
+        # expected [b][c][r][k]: outgoing (r,k) = (i,k); incoming (r,k) from ref[b,k,r,c]
         want = ref.permute(0, 3, 1, 2) if outgoing else ref.permute(0, 3, 2, 1)
         report("trimul_proj %s valid" % name, got[:, :, :n, :n], want, atol=2e-2, rtol=1e-2)
         pad = got[:, :, :n, n:]
