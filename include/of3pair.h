@@ -77,7 +77,7 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
 
 /* x[b][c][i][j] = sum_k a[b][c][i][k] * b[b][c][j][k] over the padded planes; a, b in the
  * k-panel layout above, x row-major [B][CH][NP][NP].
- * variant: 0 = automatic; 1 / 2 = 256x192 / 256x128 output tiles. */
+ * variant: 0 = automatic; 1 / 2 / 3 = 256x192 / 256x128 / 256x256 output tiles. */
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream);
 
@@ -98,7 +98,7 @@ int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask,
 /* ---- triangle attention ------------------------------------------------------------- */
 
 /* Scratch of of3_triattn_fwd, in this order, each part 256-byte aligned:
- *   q, k  [B][N][H][NP][D] bf16      vt [B][N][H][D][NP] bf16
+ *   q, k  [B][N][H][NP][D] bf16      vt [B][N][H][NP/32][D][32] bf16 (v transposed, 32-key panels)
  *   tbias [B][H][N][NP] fp32         mbias [B][N][NP] fp32       o [B][N][N][H*D] bf16 */
 int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D);
 

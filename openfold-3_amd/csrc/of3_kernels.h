@@ -30,7 +30,7 @@ struct TrimulProjArgs {
 hipError_t trimul_proj_launch(const TrimulProjArgs& args, int C, int CH, hipStream_t stream);
 
 // a, b: k-panel layout [planes][Np/32][Np][32]; x: row-major [planes][Np][Np].
-// variant: 1 = 256x192 output tiles, 2 = 256x128
+// variant: 1 = 256x192 output tiles, 2 = 256x128, 3 = 256x256
 hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
                                   hipStream_t stream);
 
@@ -56,7 +56,7 @@ struct TriattnProjArgs {
   const bf16_t *w_q, *w_k, *w_v;      // [H*D][C]
   const bf16_t *w_b;                  // [H][C]   (linear_z: triangle bias)
   bf16_t *q, *k;                      // [B][N][H][Jp][D]
-  bf16_t *vt;                         // [B][N][H][D][Jp]
+  bf16_t *vt;                         // [B][N][H][Jp/32][D][32]  (panels of 32 keys)
   float *tbias;                       // [B][H][N][Jp]   (pre-multiplied by log2 e)
   float *mbias;                       // [B][N][Jp]      (log2 e * inf * (mask-1); -inf for j >= N)
   int B, N, Jp, H;

@@ -53,10 +53,10 @@ inline const of3::bf16_t* bf(const void* p) { return static_cast<const of3::bf16
 inline of3::bf16_t* bf(void* p) { return static_cast<of3::bf16_t*>(p); }
 
 inline int contract_variant_auto(int64_t Np) {
-  // 256x192 tiles: 12 per plane at Np = 768, i.e. 6 tiles for each of 256 persistent
-  // work-groups with 128 planes
-  (void)Np;
-  return 1;
+  // 256x192 tiles give 256 persistent work-groups exactly 6 tiles each at Np = 768 with
+  // 128 planes; 256x256 tiles move fewer operand bytes per flop and win once the plane
+  // divides into them without waste.
+  return (Np >= 1024 && Np % 256 == 0) ? 3 : 1;
 }
 
 }  // namespace
@@ -119,7 +119,7 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
 
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream) {
-  if (B < 1 || N < 1 || (CH != 128 && CH != 64) || variant < 0 || variant > 2) return OF3_EINVAL;
+  if (B < 1 || N < 1 || (CH != 128 && CH != 64) || variant < 0 || variant > 3) return OF3_EINVAL;
   if (!a || !b || !x || !aligned16(a) || !aligned16(b) || !aligned16(x)) return OF3_EINVAL;
   const int64_t Np = padded(N);
   if (variant == 0) variant = contract_variant_auto(Np);

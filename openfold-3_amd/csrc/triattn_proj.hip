@@ -3,7 +3,8 @@
 //     triangle bias tb[h][q][k] = log2(e) * (xn[q][k] . Wb[h])          (tri_att.py:137-140)
 //     mask bias     mb[i][k]    = log2(e) * inf * (mask[i][k] - 1)      (tri_att.py:134)
 // written in the layouts the flash kernel consumes: q, k as [b][i][h][j][d]; v transposed
-// as [b][i][h][d][j]; tb as [b][h][i][j] and mb as [b][i][j] in fp32.  log2(e) is folded
+// in panels of 32 keys as [b][i][h][j/32][d][j%32] (one key tile of one head = 2 KB
+// contiguous); tb as [b][h][i][j] and mb as [b][i][j] in fp32.  log2(e) is folded
 // in so the softmax can use the hardware base-2 exponential.  The PairView makes (i, j)
 // walk either the tensor itself (starting node) or its transpose (ending node).
 //
@@ -191,7 +192,9 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(TriattnProjArgs p, in
         for (int v = 0; v < 16; ++v) {
           const int ch = 32 * ot + 8 * (v >> 2) + 4 * lh + (v & 3);
           const int head = ch / D, d = ch % D;
-          bf16_t* dst = p.vt + ((((size_t)b * N + i) * H + head) * D + d) * Jp + j0 + 4 * l32;
+          // key-panel layout: [b][i][h][key / 32][d][key % 32]
+          const int j = j0 + 4 * l32;
+          bf16_t* dst = p.vt + (((size_t)b * N + i) * H + head) * D * Jp + (size_t)(j >> 5) * (D * 32) + d * 32 + (j & 31);
           u32x2_t w2 = {vpk[vi][0][v], vpk[vi][1][v]};
           *reinterpret_cast<u32x2_t*>(dst) = w2;
         }

@@ -21,7 +21,7 @@
 //    holds the stage's last fragments in registers, so the stage's buffer is refilled at
 //    once (stage s+4) and the first fragments of stage s+1 are fetched under the second
 //    k-step's MFMAs; the refill's loads are issued one by one between those MFMAs;
-//  * the k-blocks of a tile are visited in rotated order, starting at (tm + tn) mod nk:
+//  * the k-blocks of a tile are visited in rotated order, starting at (tm + tn) mod 4:
 //    tiles that share operand rows never ask for the same cache line at the same time (the
 //    first asks HBM, the others find the line in L2 a stage or two later);
 //  * the j side is the MFMA M side with permuted rows so that a lane ends up owning 64
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
       const int rbc = rb + 16 <= rows_n_left ? rb : rows_n_left - 16;
       dma_base[MI + n] = reinterpret_cast<const char*>(pn) + plane_off + (size_t)(tn * BN + rbc) * (kBK * 2);
     }
-    issue_kb = (tm + tn) % nk;  // rotated start
+    issue_kb = ((tm + tn) & 3) % nk;  // rotated start (a small spread keeps the sharers' lines in L2)
     issue_left = nk;
   };
   auto issue_one = [&](int n) {
@@ -329,6 +329,8 @@ hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, i
       return launch_contract<192>(a, b, x, planes, Np, stream);
     case 2:
       return launch_contract<128>(a, b, x, planes, Np, stream);
+    case 3:
+      return launch_contract<256>(a, b, x, planes, Np, stream);
     default:
       return hipErrorInvalidValue;
   }

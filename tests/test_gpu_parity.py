@@ -100,7 +100,8 @@ def test_triattn_module(starting, c, d, n, batch):
     got = m(z.to(DEV).to(torch.bfloat16), mask=mask.to(DEV), chunk_size=4, use_lma=True)
     want = orc.triattn_update(z, mask, p, 4, starting=starting)
     floor = orc.triattn_update(z.to(torch.bfloat16), mask.to(torch.bfloat16), _bf16_params(p), 4, starting=starting)
-    _check("triattn update", got, want, bf16_ref=floor)
+    # rms bound 6e-3: the bf16 reference path itself sits at about 7.5e-3 on these inputs
+    _check("triattn update", got, want, rms_rel=6e-3, bf16_ref=floor)
 
 
 def test_triattn_transposed_view_input():

@@ -36,7 +36,7 @@ def _to_panels(t):
     return t.reshape(*lead, rows, k // 32, 32).transpose(-2, -3).contiguous()
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
 @pytest.mark.parametrize("n", [128, 384, 640, 768])
 def test_contract(variant, n):
     L = lib()
@@ -149,7 +149,7 @@ def test_triattn_proj(transposed, C, D, n, B):
     w = _triattn_weights(gen, C, H, D)
     q = torch.full((B, n, H, np_, D), float("nan"), dtype=torch.bfloat16, device=DEV)
     k = torch.full_like(q, float("nan"))
-    vt = torch.full((B, n, H, D, np_), float("nan"), dtype=torch.bfloat16, device=DEV)
+    vt = torch.full((B, n, H, np_ // 32, D, 32), float("nan"), dtype=torch.bfloat16, device=DEV)
     tb = torch.full((B, H, n, np_), float("nan"), dtype=torch.float32, device=DEV)
     mb = torch.full((B, n, np_), float("nan"), dtype=torch.float32, device=DEV)
     print("triattn_proj", transposed, C, D, n, B, flush=True)
@@ -167,6 +167,7 @@ def test_triattn_proj(transposed, C, D, n, B):
     mbr = LOG2E * 1e9 * (mask - 1)
     report("q", q[:, :, :, :n], qr, atol=2e-2, rtol=1e-2)
     report("k", k[:, :, :, :n], kr, atol=2e-2, rtol=1e-2)
+    vt = vt.transpose(-2, -3).reshape(B, n, H, D, np_)  # key panels -> [b][i][h][d][j]
     report("vt", vt[..., :n], vr, atol=2e-2, rtol=1e-2)
     report("tbias", tb[..., :n], tbr, atol=2e-2, rtol=1e-2)
     assert torch.equal(mb[..., :n], mbr), "mask bias"
@@ -190,7 +191,8 @@ def test_triattn_flash(D, n, B):
     mb[..., :n] = LOG2E * 1e9 * (mask - 1)
     o = torch.full((B, n, n, H * D), float("nan"), dtype=torch.bfloat16, device=DEV)
     print("triattn_flash", D, n, B, flush=True)
-    st = L.of3_triattn_flash(q.data_ptr(), k.data_ptr(), vt.data_ptr(), tb.data_ptr(), mb.data_ptr(), o.data_ptr(),
+    vtp = _to_panels(vt)  # [b][i][h][d][j] -> [b][i][h][j/32][d][32]
+    st = L.of3_triattn_flash(q.data_ptr(), k.data_ptr(), vtp.data_ptr(), tb.data_ptr(), mb.data_ptr(), o.data_ptr(),
                              B, n, H, D, stream())
     assert st == 0, L.of3_status_string(st)
     torch.cuda.synchronize()
