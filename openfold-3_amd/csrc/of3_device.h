@@ -84,11 +84,21 @@ __device__ __forceinline__ float sigmoidf_fast(float x) {
   return fast_rcp(1.f + fast_exp2(-kLog2e * x));
 }
 
-// all-reduce (sum) over the LPP consecutive lanes that share one position
+// all-reduce (sum) over the LPP (8 or 16) consecutive lanes that share one position, with
+// DPP lane permutations (no LDS round trips): xor 1 and xor 2 inside each quad, then
+// row_half_mirror (lane i <-> 7-i of each 8) and row_mirror (i <-> 15-i of each 16), which
+// pair every quad / half-row with the one holding the other partial sum.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
 template <int LPP>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int o = 1; o < LPP; o <<= 1) v += __shfl_xor(v, o, 64);
+  static_assert(LPP == 8 || LPP == 16, "8 or 16 lanes per position");
+  v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_move<0x141>(v);  // row_half_mirror
+  if (LPP == 16) v += dpp_move<0x140>(v);  // row_mirror
   return v;
 }
 
