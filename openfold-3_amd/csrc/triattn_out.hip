@@ -15,23 +15,25 @@ namespace of3 {
 namespace {
 
 template <int C, int HD>
-__global__ __launch_bounds__(256) void triattn_out_kernel(TriattnOutArgs p, int tiles_per_row, int total_tiles) {
+__global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int tiles_per_row, int total_tiles) {
   static_assert(C == HD, "o tile shares the x tile geometry");
   constexpr int NCH = C / 8;
   constexpr int LPP = NCH;
   constexpr int PPI = 64 / LPP;
   constexpr int TP = 128;
-  constexpr int LN_ITERS = 32 / PPI;
+  constexpr int NW = 8;                  // waves per work-group (two per SIMD)
+  constexpr int LN_ITERS = (TP / NW) / PPI;
   constexpr int KS = C / 16;
   constexpr int NOT = C / 32;
-  constexpr int WPG = 4 / NOT;
+  constexpr int WPG = NW / NOT;
   constexpr int TPW = 4 / WPG;
 
   __shared__ u32x4_t xtile[TP * NCH];  // LayerNorm(x), bf16
   __shared__ u32x4_t otile[TP * NCH];  // o, then o * gate
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
   const int ln_chunk = lane % LPP, ln_pp = lane / LPP;
 
   float lw[8], lb[8];
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(256) void triattn_out_kernel(TriattnOutArgs p, int 
     u32x4_t xraw[LN_ITERS], oraw[LN_ITERS];
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int j = j0 + wave * 32 + it * PPI + ln_pp;
+      const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
       u32x4_t vx = {0u, 0u, 0u, 0u}, vo = {0u, 0u, 0u, 0u};
       if (j < N) {
         vx = *reinterpret_cast<const u32x4_t*>(xrow + j * p.x_view.stride_k + 8 * ln_chunk);
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(256) void triattn_out_kernel(TriattnOutArgs p, int 
     }
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int pos = wave * 32 + it * PPI + ln_pp;
+      const int pos = wave * (TP / NW) + it * PPI + ln_pp;
       const int slot = tile_slot<NCH, 0>(pos, ln_chunk);
       xtile[slot] = layer_norm_chunk<C>(xraw[it], lw, lb);
       otile[slot] = oraw[it];
@@ -151,14 +153,14 @@ hipError_t launch(const TriattnOutArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, 0);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 512, 0);
     if (e != hipSuccess) return e;
     grid_cap = cus * (per_cu > 0 ? per_cu : 1);
   }
   const int tiles_per_row = (a.N + 127) / 128;
   const long total = (long)a.B * a.N * tiles_per_row;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), 0, stream, a, tiles_per_row, (int)total);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, tiles_per_row, (int)total);
   return hipGetLastError();
 }
 

@@ -9,8 +9,9 @@
 // walk either the tensor itself (starting node) or its transpose (ending node).
 //
 // HBM bound (reads x once, writes q, k, v once).  Same structure as the
-// triangle-multiplication input pass: weights resident in registers as MFMA A operands,
-// 128-position tiles normalised in registers and staged once in LDS.
+// triangle-multiplication input pass: 8 waves per work-group, weights resident in registers
+// as MFMA A operands, 128-position tiles normalised in registers and staged once in a
+// double-buffered LDS tile (one barrier per tile).
 #include "of3_device.h"
 #include "of3_kernels.h"
 
@@ -19,57 +20,69 @@ namespace of3 {
 namespace {
 
 template <int C, int D>
-__global__ __launch_bounds__(256) void triattn_proj_kernel(TriattnProjArgs p, int tiles_per_row, int total_tiles) {
+__global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, int tiles_per_row, int total_tiles) {
   constexpr int H = 4;
   constexpr int HD = H * D;
   constexpr int NCH = C / 8;
   constexpr int LPP = NCH;
   constexpr int PPI = 64 / LPP;
   constexpr int TP = 128;
-  constexpr int LN_ITERS = 32 / PPI;
+  constexpr int NW = 8;                // waves per work-group
+  constexpr int LN_ITERS = (TP / NW) / PPI;
   constexpr int KS = C / 16;
   constexpr int NT = HD / 32;          // 32-row output tiles per matrix (4 or 2)
-  constexpr bool WIDE = (NT == 4);     // HD = 128: wave w owns tile w of q, k and v
-  constexpr int NJ = WIDE ? 3 : 2;     // HD = 64: wave m (< 3) owns both tiles of matrix m
+  constexpr bool WIDE = (NT == 4);
+  // WIDE (H*D = 128): waves 0..3 own output tile w of q and of k, waves 4..7 own tile w-4 of
+  //   v plus the bias of position tile w-4; waves w and w+4 share a SIMD, so every SIMD
+  //   carries the same MFMA load.
+  // else (H*D = 64): waves 0..5 own one (matrix, tile) job, waves 6 and 7 do the bias of two
+  //   position tiles each.
+  constexpr int NJ = WIDE ? 2 : 1;     // q/k/v jobs per wave (the second one only on waves 0..3)
+  constexpr int TPW = 4;               // every wave visits all four position tiles
+  constexpr int KSH = 2;               // swizzle key from pos / 4
   static_assert(NT == 4 || NT == 2, "H*D must be 128 or 64");
 
-  __shared__ u32x4_t tile[TP * NCH];
+  __shared__ u32x4_t tile[2][TP * NCH];
+  __shared__ u32x4_t wb_lds[KS * 64];  // triangle-bias weights in MFMA A-operand order (rows >= H are zero)
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
   const int ln_chunk = lane % LPP, ln_pp = lane / LPP;
 
   float lw[8], lb[8];
   load_affine8(p.ln_w, ln_chunk, lw);
   load_affine8(p.ln_b, ln_chunk, lb);
 
-  const bool has_jobs = WIDE || wave < 3;
-  // job jj of this wave: matrix (0 q, 1 k, 2 v) and output tile
-  auto job_matrix = [&](int jj) { return WIDE ? jj : wave; };
-  auto job_tile = [&](int jj) { return WIDE ? wave : jj; };
+  const int tgroup = 0;
+  const bool has_jobs = WIDE || wave < 6;
+  // 0 q, 1 k, 2 v
+  auto job_matrix = [&](int jj) { return WIDE ? (wave < 4 ? jj : 2) : wave / 2; };
+  auto job_live = [&](int jj) { return WIDE ? (jj == 0 || wave < 4) : wave < 6; };
+  const int ot = WIDE ? wave % 4 : wave % 2;
 
   u32x4_t wj[NJ][KS];
 #pragma unroll
   for (int jj = 0; jj < NJ; ++jj) {
-    const int m = job_matrix(jj), ot = job_tile(jj);
+    const int m = job_matrix(jj);
     const bf16_t* W = (m == 0) ? p.w_q : (m == 1 ? p.w_k : p.w_v);
     // q, k: lane owns 16 consecutive channels (rowperm16); v: natural rows
     const int row = 32 * ot + ((m == 2) ? l32 : rowperm16(l32));
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       u32x4_t w = {0u, 0u, 0u, 0u};
-      if (has_jobs) w = *reinterpret_cast<const u32x4_t*>(W + row * C + 16 * s + 8 * lh);
+      if (job_live(jj)) w = *reinterpret_cast<const u32x4_t*>(W + row * C + 16 * s + 8 * lh);
       wj[jj][s] = w;
     }
   }
-  // triangle-bias weights: A rows 0..H-1 hold Wb, the rest are zero
-  u32x4_t wb[KS];
+  if (wave == 0) {
 #pragma unroll
-  for (int s = 0; s < KS; ++s) {
-    u32x4_t w = {0u, 0u, 0u, 0u};
-    if (l32 < H) w = *reinterpret_cast<const u32x4_t*>(p.w_b + l32 * C + 16 * s + 8 * lh);
-    wb[s] = w;
-  }
+    for (int s = 0; s < KS; ++s) {
+      u32x4_t w = {0u, 0u, 0u, 0u};
+      if (l32 < H) w = *reinterpret_cast<const u32x4_t*>(p.w_b + l32 * C + 16 * s + 8 * lh);
+      wb_lds[s * 64 + lane] = w;
+    }
+  }  // published by the first tile's barrier
   const float qscale = kLog2e * __builtin_amdgcn_rsqf((float)D);
 
   const int N = p.N, Jp = p.Jp;
@@ -84,17 +97,20 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(TriattnProjArgs p, in
     const bf16_t* xrow = p.x + b * p.x_view.stride_b + i * p.x_view.stride_r;
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int j = j0 + wave * 32 + it * PPI + ln_pp;
+      const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
       u32x4_t v = {0u, 0u, 0u, 0u};
       if (j < N) v = *reinterpret_cast<const u32x4_t*>(xrow + j * p.x_view.stride_k + 8 * ln_chunk);
       raw[it] = v;
     }
   };
 
+  // position 32*TPW*tgroup + TPW*l32 + tt is column l32 of this wave's position tile tt
+  const int pos0 = 32 * TPW * tgroup + TPW * l32;
+
   int tile_id = blockIdx.x;
   if (tile_id < total_tiles) load_tile(tile_id);
 
-  for (; tile_id < total_tiles; tile_id += gridDim.x) {
+  for (int buf = 0; tile_id < total_tiles; tile_id += gridDim.x, buf ^= 1) {
     const int b = tile_id / tiles_per_batch;
     const int rem = tile_id - b * tiles_per_batch;
     const int i = rem / tiles_per_row;
@@ -103,8 +119,8 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(TriattnProjArgs p, in
     // ---- LayerNorm phase (+ mask bias, one lane per position)
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int pos = wave * 32 + it * PPI + ln_pp;
-      tile[tile_slot<NCH, 2>(pos, ln_chunk)] = layer_norm_chunk<C>(raw[it], lw, lb);
+      const int pos = wave * (TP / NW) + it * PPI + ln_pp;
+      tile[buf][tile_slot<NCH, KSH>(pos, ln_chunk)] = layer_norm_chunk<C>(raw[it], lw, lb);
       if (ln_chunk == 0) {
         const int j = j0 + pos;
         float mb = -__builtin_inff();
@@ -116,36 +132,30 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(TriattnProjArgs p, in
         p.mbias[((size_t)b * N + i) * Jp + j] = mb;
       }
     }
-    __syncthreads();
-
     if (tile_id + (int)gridDim.x < total_tiles) load_tile(tile_id + gridDim.x);
+    __syncthreads();  // the only barrier per tile (the LDS tile is double buffered)
 
-    // ---- projection phase: position 4*l32 + t is column l32 of position-tile t
-    uint32_t vpk[2][2][16];   // v jobs only: [tile][position pair][register]
-    float vprev[2][16];
+    // ---- projection phase
+    const size_t bi = (size_t)b * N + i;
+    float vres[TPW][16];  // v job only
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      u32x4_t bop[KS];
-      const int pos = 4 * l32 + t;
-#pragma unroll
-      for (int s = 0; s < KS; ++s) bop[s] = tile[tile_slot<NCH, 2>(pos, 2 * s + lh)];
+    for (int tt = 0; tt < TPW; ++tt) {
+      // the B operand (this lane's position, k-step s) is re-read from LDS by every job: cheaper
+      // than holding it in 32 registers across the jobs
+      auto bop = [&](int s) { return tile[buf][tile_slot<NCH, KSH>(pos0 + tt, 2 * s + lh)]; };
+      const int j = j0 + pos0 + tt;
 
       if (has_jobs) {
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj) {
-          const int m = job_matrix(jj), ot = job_tile(jj);
+          if (!job_live(jj)) continue;  // wave-uniform
+          const int m = job_matrix(jj);
           f32x16_t acc = zero16();
 #pragma unroll
-          for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wj[jj][s], bop[s], acc);
+          for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wj[jj][s], bop(s), acc);
           if (m == 2) {
-            const int vi = WIDE ? 0 : jj;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-              if (t & 1)
-                vpk[vi][t >> 1][v] = pack_bf16(vprev[vi][v], acc[v]);
-              else
-                vprev[vi][v] = acc[v];
-            }
+            for (int v = 0; v < 16; ++v) vres[tt][v] = acc[v];
           } else {
             // lane owns channels 32*ot + 16*lh + v  ->  head, d0 .. d0+15
             const int ch0 = 32 * ot + 16 * lh;
@@ -158,49 +168,46 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(TriattnProjArgs p, in
               o1[q] = pack_bf16(acc[8 + 2 * q] * sc, acc[8 + 2 * q + 1] * sc);
             }
             bf16_t* base = (m == 0) ? p.q : p.k;
-            bf16_t* dst = base + ((((size_t)b * N + i) * H + head) * Jp + (j0 + pos)) * D + d0;
+            bf16_t* dst = base + ((bi * H + head) * Jp + j) * D + d0;
             *reinterpret_cast<u32x4_t*>(dst) = o0;
             *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
           }
         }
       }
 
-      // triangle bias of this position tile: WIDE -> wave t, else wave 3
-      const bool bias_here = WIDE ? (wave == t) : (wave == 3);
+      // triangle bias: WIDE -> wave 4+tt does position tile tt; else waves 6, 7 take position
+      // tiles {0,1} and {2,3}
+      const bool bias_here = WIDE ? (wave == 4 + tt) : (wave >= 6 && (tt >> 1) == (wave - 6));
       if (bias_here) {
         f32x16_t acc = zero16();
 #pragma unroll
-        for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wb[s], bop[s], acc);
+        for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wb_lds[s * 64 + lane], bop(s), acc);
         // rows 0..3 of the result sit in registers 0..3 of lanes 0..31
-        const int j = j0 + pos;
-        if (lh == 0 && j < Jp) {
+        if (lh == 0) {
 #pragma unroll
-          for (int h = 0; h < H; ++h)
-            p.tbias[(((size_t)b * H + h) * N + i) * Jp + j] = (j < N) ? acc[h] * kLog2e : 0.f;
+          for (int h = 0; h < H; ++h) p.tbias[(((size_t)b * H + h) * N + i) * Jp + j] = (j < N) ? acc[h] * kLog2e : 0.f;
         }
       }
     }
 
-    // ---- v stores: register v is channel 32*ot + 8*(v/4) + 4*lh + v%4 = head*D + d
-    if (has_jobs) {
+    // ---- v stores: register v is channel 32*ot + 8*(v/4) + 4*lh + v%4 = head*D + d;
+    // key-panel layout [b][i][h][key / 32][d][key % 32]
+    const bool v_job = WIDE ? wave >= 4 : (wave / 2) == 2;
+    if (has_jobs && v_job) {
+      const int j = j0 + pos0;
 #pragma unroll
-      for (int jj = 0; jj < NJ; ++jj) {
-        if (job_matrix(jj) != 2) continue;
-        const int ot = job_tile(jj);
-        const int vi = WIDE ? 0 : jj;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int ch = 32 * ot + 8 * (v >> 2) + 4 * lh + (v & 3);
-          const int head = ch / D, d = ch % D;
-          // key-panel layout: [b][i][h][key / 32][d][key % 32]
-          const int j = j0 + 4 * l32;
-          bf16_t* dst = p.vt + (((size_t)b * N + i) * H + head) * D * Jp + (size_t)(j >> 5) * (D * 32) + d * 32 + (j & 31);
-          u32x2_t w2 = {vpk[vi][0][v], vpk[vi][1][v]};
+      for (int v = 0; v < 16; ++v) {
+        const int ch = 32 * ot + 8 * (v >> 2) + 4 * lh + (v & 3);
+        const int head = ch / D, d = ch % D;
+        bf16_t* dst = p.vt + (bi * H + head) * D * Jp + (size_t)(j >> 5) * (D * 32) + d * 32 + (j & 31);
+        if (TPW == 4) {
+          u32x2_t w2 = {pack_bf16(vres[0][v], vres[1][v]), pack_bf16(vres[2 % TPW][v], vres[3 % TPW][v])};
           *reinterpret_cast<u32x2_t*>(dst) = w2;
+        } else {
+          *reinterpret_cast<uint32_t*>(dst) = pack_bf16(vres[0][v], vres[1][v]);
         }
       }
     }
-    __syncthreads();
   }
 }
 
@@ -214,14 +221,14 @@ hipError_t launch(const TriattnProjArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, 0);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 512, 0);
     if (e != hipSuccess) return e;
     grid_cap = cus * (per_cu > 0 ? per_cu : 1);
   }
   const int tiles_per_row = a.Jp / 128;
   const long total = (long)a.B * a.N * tiles_per_row;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), 0, stream, a, tiles_per_row, (int)total);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, tiles_per_row, (int)total);
   return hipGetLastError();
 }
 

@@ -15,24 +15,26 @@ namespace of3 {
 namespace {
 
 template <int C, int CH>
-__global__ __launch_bounds__(256) void trimul_out_kernel(TrimulOutArgs p, int tiles_per_row, int total_tiles) {
+__global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int tiles_per_row, int total_tiles) {
   static_assert(C == CH, "position-major x tile shares the z tile geometry");
   constexpr int NCH = C / 8;
   constexpr int LPP = NCH;
   constexpr int PPI = 64 / LPP;
   constexpr int TP = 128;
-  constexpr int LN_ITERS = 32 / PPI;
+  constexpr int NW = 8;                  // waves per work-group (two per SIMD)
+  constexpr int LN_ITERS = (TP / NW) / PPI;
   constexpr int KS = C / 16;
   constexpr int NOT = C / 32;            // output-channel tiles
-  constexpr int WPG = 4 / NOT;           // waves sharing one output tile (1 or 2)
+  constexpr int WPG = NW / NOT;          // waves sharing one output tile (2 or 4)
   constexpr int TPW = 4 / WPG;           // position tiles per wave
-  constexpr int XROUNDS = (CH / 2) * 16 / 256;  // (channel pair, 8-position group) items per thread
+  constexpr int XROUNDS = (CH / 2) * 16 / 512;  // (channel pair, 8-position group) items per thread
 
   __shared__ u32x4_t ztile[TP * NCH];
   __shared__ u32x4_t xtile[TP * NCH];
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
   const int ln_chunk = lane % LPP, ln_pp = lane / LPP;
 
   float iw[8], ib[8], ow[8], ob[8];
@@ -57,9 +59,7 @@ __global__ __launch_bounds__(256) void trimul_out_kernel(TrimulOutArgs p, int ti
 
   const int N = p.N, Np = p.Np;
   const int tiles_per_batch = N * tiles_per_row;
-  uint16_t* xt16 = reinterpret_cast<uint16_t*>(xtile);
   uint32_t* xt32 = reinterpret_cast<uint32_t*>(xtile);
-  (void)xt16;
 
   for (int tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
     const int b = tile_id / tiles_per_batch;
@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256) void trimul_out_kernel(TrimulOutArgs p, int ti
     u32x4_t zraw[LN_ITERS];
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int j = j0 + wave * 32 + it * PPI + ln_pp;
+      const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
       u32x4_t v = {0u, 0u, 0u, 0u};
       if (j < N) v = *reinterpret_cast<const u32x4_t*>(zrow + j * p.z_view.stride_k + 8 * ln_chunk);
       zraw[it] = v;
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void trimul_out_kernel(TrimulOutArgs p, int ti
     u32x4_t xa[XROUNDS], xb[XROUNDS];
 #pragma unroll
     for (int rr = 0; rr < XROUNDS; ++rr) {
-      const int item = rr * 256 + tid;
+      const int item = rr * 512 + tid;
       const int cp = item >> 4, pg = item & 15;  // channels 2cp, 2cp+1; positions 8pg..8pg+7
       const bf16_t* src = p.x + (((size_t)b * CH + 2 * cp) * Np + i) * Np + j0 + 8 * pg;
       xa[rr] = *reinterpret_cast<const u32x4_t*>(src);
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void trimul_out_kernel(TrimulOutArgs p, int ti
     // x: transpose into xtile[pos][c] with 4-byte (channel pair) writes
 #pragma unroll
     for (int rr = 0; rr < XROUNDS; ++rr) {
-      const int item = rr * 256 + tid;
+      const int item = rr * 512 + tid;
       const int cp = item >> 4, pg = item & 15;
       const int chunk = (2 * cp) >> 3, within = (2 * cp) & 7;  // `within` is even
 #pragma unroll
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void trimul_out_kernel(TrimulOutArgs p, int ti
     // z: LayerNorm_in -> ztile
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int pos = wave * 32 + it * PPI + ln_pp;
+      const int pos = wave * (TP / NW) + it * PPI + ln_pp;
       ztile[tile_slot<NCH, 0>(pos, ln_chunk)] = layer_norm_chunk<C>(zraw[it], iw, ib);
     }
     __syncthreads();
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(256) void trimul_out_kernel(TrimulOutArgs p, int ti
     // x: LayerNorm_out in place (lane owns one 16-byte chunk of one position)
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int pos = wave * 32 + it * PPI + ln_pp;
+      const int pos = wave * (TP / NW) + it * PPI + ln_pp;
       const int slot = tile_slot<NCH, 0>(pos, ln_chunk);
       xtile[slot] = layer_norm_chunk<CH>(xtile[slot], ow, ob);
     }
@@ -173,14 +173,14 @@ hipError_t launch(const TrimulOutArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 256, 0);
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 512, 0);
     if (e != hipSuccess) return e;
     grid_cap = cus * (per_cu > 0 ? per_cu : 1);
   }
   const int tiles_per_row = (a.N + 127) / 128;
   const long total = (long)a.B * a.N * tiles_per_row;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), 0, stream, a, tiles_per_row, (int)total);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, tiles_per_row, (int)total);
   return hipGetLastError();
 }
 
