@@ -11,7 +11,8 @@ Besides the whole-block time the line carries
   roofline      the triangle-multiplication contraction (the MFMA-bound kernel the target
                 of >= 50 % of bf16 peak is set on): algorithmic 2*B*N^3*C_h flops over its
                 average launch duration, measured here with events on the launch stream;
-  kernels       the same figure for every kernel of the block, each against the roof that
+  kernels       the same figure for every kernel of the block (average over its launches in
+                the block: both directions of each module), each against the roof that
                 bounds it (MFMA for the contraction and the attention core, HBM for the
                 LayerNorm/projection passes; algorithmic bytes per launch are listed in
                 KERNEL_MODEL below);
@@ -34,6 +35,14 @@ for _p in (ROOT, os.path.join(ROOT, "openfold-3_amd")):
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
+CAL_BYTES = 256 << 20      # size of the calibration copy
+
+# HBM bytes per launch of the contraction at the headline workload (N=768, B=1), from two
+# counter passes of this command (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE), each
+# scaled by what the same counter reads for the calibration copy; the summaries are kept in
+# profiles/.  None for any other workload.
+MEASURED_TRAFFIC = {("trimul_contract", 768): 539644928}
+
 METRIC = "ms per Pairformer pair-stack block at N=768 bf16; % of MFMA peak & HBM GB/s"
 
 
@@ -55,20 +64,6 @@ def kernel_model(B, N, C, CH, H, D):
         # reads o and x, writes out
         "triattn_out": {"bound": "hbm", "bytes": B * N * N * hd * 2 + 2 * U},
     }
-
-
-def time_events(fn, steps, warmup, torch):
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
-        fn()
-    end.record()
-    torch.cuda.synchronize()
-    return start.elapsed_time(end) / steps  # ms
 
 
 def main():
@@ -106,6 +101,14 @@ def main():
     z = z_host.to(dev).to(torch.bfloat16)
     mask = torch.ones(B, N, N, device=dev)
 
+    # one plain device copy of known size (CAL_BYTES read + CAL_BYTES written): a counter
+    # profile of this command then holds its own calibration kernel for FETCH_SIZE/WRITE_SIZE
+    cal_src = torch.ones(CAL_BYTES // 4, dtype=torch.float32, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
+
     # ---- whole block, in place, inputs resident
     def step():
         block(z, mask, inplace_safe=True)
@@ -119,20 +122,23 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # ---- per-kernel durations through the stage entry points of the C ABI
+    # ---- per-kernel durations: the same block issued kernel by kernel through the stage
+    # entry points of the C ABI, every launch bracketed by its own pair of events on the
+    # launch stream, so that each kernel is timed where it runs in the block (inputs left in
+    # the caches by its producer, clocks as in the block) and not in a back-to-back loop
     lib = _lib.load()
     s = torch.cuda.current_stream().cuda_stream
     Np = lib.of3_padded_n(N)
     bf = torch.bfloat16
     zz = z_host.to(dev).to(bf)
-    zs = _lib.strides3(zz.stride()[:3])
-    ms_ = _lib.strides3(mask.stride())
-    tm = {k[len("tri_mul_out."):]: v.to(dev).to(bf).contiguous() for k, v in params.items() if k.startswith("tri_mul_out.")}
-    ta = {k[len("tri_att_start."):]: v.to(dev).to(bf).contiguous() for k, v in params.items() if k.startswith("tri_att_start.")}
+    sb, si, sj = zz.stride()[:3]
+    z_fwd, z_tr = _lib.strides3((sb, si, sj)), _lib.strides3((sb, sj, si))
+    mb_, mi, mj = mask.stride()
+    m_fwd, m_tr = _lib.strides3((mb_, mi, mj)), _lib.strides3((mb_, mj, mi))
+    dp = {k: v.to(dev).to(bf).contiguous() for k, v in params.items()}
     a = torch.zeros(B, CH, Np, Np, dtype=bf, device=dev)
     b = torch.zeros_like(a)
     x = torch.zeros_like(a)
-    out = torch.empty_like(zz)
     q = torch.zeros(B, N, H, Np, D, dtype=bf, device=dev)
     k = torch.zeros_like(q)
     vt = torch.zeros(B, N, H, D, Np, dtype=bf, device=dev)
@@ -144,30 +150,57 @@ def main():
     def ck(st):
         _lib.check(st, "bench stage")
 
-    stages = {
-        "trimul_proj": lambda: ck(lib.of3_trimul_proj(P(zz), zs, P(mask), ms_, P(tm["layer_norm_in.weight"]),
-                                                      P(tm["layer_norm_in.bias"]), P(tm["linear_a_p.weight"]),
-                                                      P(tm["linear_a_g.weight"]), P(tm["linear_b_p.weight"]),
-                                                      P(tm["linear_b_g.weight"]), P(a), P(b), B, N, C, CH, 1, s)),
-        "trimul_contract": lambda: ck(lib.of3_trimul_contract(P(a), P(b), P(x), B, N, CH, args.contract_variant, s)),
-        "trimul_out": lambda: ck(lib.of3_trimul_out(P(x), P(zz), zs, P(out), P(tm["layer_norm_in.weight"]),
-                                                    P(tm["layer_norm_in.bias"]), P(tm["layer_norm_out.weight"]),
-                                                    P(tm["layer_norm_out.bias"]), P(tm["linear_g.weight"]),
-                                                    P(tm["linear_z.weight"]), B, N, C, CH, 1, s)),
-        "triattn_proj": lambda: ck(lib.of3_triattn_proj(P(zz), zs, P(mask), ms_, P(ta["layer_norm.weight"]),
-                                                        P(ta["layer_norm.bias"]), P(ta["mha.linear_q.weight"]),
-                                                        P(ta["mha.linear_k.weight"]), P(ta["mha.linear_v.weight"]),
-                                                        P(ta["linear_z.weight"]), P(q), P(k), P(vt), P(tb), P(mb),
-                                                        B, N, C, H, D, 1e9, s)),
-        "triattn_flash": lambda: ck(lib.of3_triattn_flash(P(q), P(k), P(vt), P(tb), P(mb), P(o), B, N, H, D, s)),
-        "triattn_out": lambda: ck(lib.of3_triattn_out(P(o), P(zz), zs, P(out), P(ta["layer_norm.weight"]),
-                                                      P(ta["layer_norm.bias"]), P(ta["mha.linear_g.weight"]),
-                                                      P(ta["mha.linear_o.weight"]), B, N, C, H, D, 1, s)),
-    }
+    def trimul(prefix, outgoing):
+        w = lambda name: P(dp[prefix + name])  # noqa: E731
+        return [
+            ("trimul_proj", lambda: ck(lib.of3_trimul_proj(
+                P(zz), z_fwd, P(mask), m_fwd, w("layer_norm_in.weight"), w("layer_norm_in.bias"),
+                w("linear_a_p.weight"), w("linear_a_g.weight"), w("linear_b_p.weight"), w("linear_b_g.weight"),
+                P(a), P(b), B, N, C, CH, outgoing, s))),
+            ("trimul_contract", lambda: ck(lib.of3_trimul_contract(P(a), P(b), P(x), B, N, CH,
+                                                                    args.contract_variant, s))),
+            ("trimul_out", lambda: ck(lib.of3_trimul_out(
+                P(x), P(zz), z_fwd, P(zz), w("layer_norm_in.weight"), w("layer_norm_in.bias"),
+                w("layer_norm_out.weight"), w("layer_norm_out.bias"), w("linear_g.weight"), w("linear_z.weight"),
+                B, N, C, CH, 1, s))),
+        ]
+
+    def triattn(prefix, zs, ms_):
+        w = lambda name: P(dp[prefix + name])  # noqa: E731
+        return [
+            ("triattn_proj", lambda: ck(lib.of3_triattn_proj(
+                P(zz), zs, P(mask), ms_, w("layer_norm.weight"), w("layer_norm.bias"), w("mha.linear_q.weight"),
+                w("mha.linear_k.weight"), w("mha.linear_v.weight"), w("linear_z.weight"),
+                P(q), P(k), P(vt), P(tb), P(mb), B, N, C, H, D, 1e9, s))),
+            ("triattn_flash", lambda: ck(lib.of3_triattn_flash(P(q), P(k), P(vt), P(tb), P(mb), P(o), B, N, H, D, s))),
+            ("triattn_out", lambda: ck(lib.of3_triattn_out(
+                P(o), P(zz), zs, P(zz), w("layer_norm.weight"), w("layer_norm.bias"), w("mha.linear_g.weight"),
+                w("mha.linear_o.weight"), B, N, C, H, D, 1, s))),
+        ]
+
+    launches = (trimul("tri_mul_out.", 1) + trimul("tri_mul_in.", 0)
+                + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr))
+    for _ in range(max(args.warmup, 1)):
+        for _, fn in launches:
+            fn()
+    torch.cuda.synchronize()
+    marks = []
+    for _ in range(args.steps):
+        for name, fn in launches:
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            marks.append((name, e0, e1))
+    torch.cuda.synchronize()
+    durations = {}
+    for name, e0, e1 in marks:
+        durations.setdefault(name, []).append(e0.elapsed_time(e1))
     model = kernel_model(B, N, C, CH, H, D)
     kernels = {}
-    for name, fn in stages.items():
-        ms = time_events(fn, max(args.steps, 10), max(args.warmup, 3), torch)
+    for name, vals in durations.items():
+        ms = sum(vals) / len(vals)
         m = model[name]
         if m["bound"] == "mfma":
             ach = m["flops"] / (ms * 1e-3) / 1e12
@@ -179,7 +212,7 @@ def main():
                              "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4)}
     dom = kernels["trimul_contract"]
     roofline = {"kernel": "trimul_contract", "bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": dom["frac"], "traffic": None}
+                "unit": "TFLOP/s", "frac": dom["frac"], "traffic": MEASURED_TRAFFIC.get(("trimul_contract", N))}
 
     # ---- CPU baseline: the oracle on the host cores, one block of the same workload
     cpu = None

@@ -1,0 +1,140 @@
+"""CPU-side checks of the C-ABI boundary: the shared library loads without a GPU, exports
+every symbol include/of3pair.h declares, and rejects bad arguments with the documented status
+codes before any kernel would be launched.  No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "of3pair.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from of3pair import _lib
+    from of3pair import build as of3_build
+
+    if not of3_build.is_built():
+        of3_build.build()
+    return _lib.load()
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(of3_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_expected_entry_points():
+    names = _declared_symbols()
+    for required in ("of3_trimul_fwd", "of3_trimul_proj", "of3_trimul_contract", "of3_trimul_out",
+                     "of3_triattn_fwd", "of3_triattn_proj", "of3_triattn_flash", "of3_triattn_out",
+                     "of3_version", "of3_last_hip_error", "of3_status_string", "of3_padded_n",
+                     "of3_trimul_workspace_bytes", "of3_triattn_workspace_bytes"):
+        assert required in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from of3pair import _lib
+
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _declared_symbols():
+        assert hasattr(raw, name), "libof3pair.so does not export %s" % name
+        assert name in _lib.SIGNATURES, "ctypes binding lacks %s" % name
+    assert sorted(_lib.SIGNATURES) == _declared_symbols()
+
+
+def test_version_and_status_strings(lib):
+    assert lib.of3_version() >= 1
+    assert lib.of3_status_string(0) == b"ok"
+    assert b"workspace" in lib.of3_status_string(-2)
+    assert b"invalid" in lib.of3_status_string(-1)
+
+
+def test_padded_n(lib):
+    assert lib.of3_padded_n(1) == 128
+    assert lib.of3_padded_n(128) == 128
+    assert lib.of3_padded_n(129) == 256
+    assert lib.of3_padded_n(768) == 768
+    assert lib.of3_padded_n(0) == 0
+
+
+def test_workspace_sizes(lib):
+    n, np_ = 768, 768
+    assert lib.of3_trimul_workspace_bytes(1, n, 128, 128) == 3 * 128 * np_ * np_ * 2
+    qkv = n * 4 * np_ * 32 * 2
+    want = 3 * qkv + 4 * n * np_ * 4 + n * np_ * 4 + n * n * 128 * 2
+    assert lib.of3_triattn_workspace_bytes(1, n, 128, 4, 32) == want
+    # unsupported shapes are reported as OF3_EINVAL (-1)
+    assert lib.of3_trimul_workspace_bytes(1, n, 128, 64) == -1
+    assert lib.of3_trimul_workspace_bytes(1, n, 96, 96) == -1
+    assert lib.of3_triattn_workspace_bytes(1, n, 128, 8, 16) == -1
+    assert lib.of3_triattn_workspace_bytes(1, 0, 128, 4, 32) == -1
+
+
+FAKE = 0x10000  # non-null, 256-byte aligned, never dereferenced: validation fails first
+
+
+def _s3(a, b, c):
+    from of3pair import _lib
+
+    return _lib.strides3((a, b, c))
+
+
+def test_trimul_fwd_rejects_bad_arguments(lib):
+    from of3pair import _lib
+
+    zs = _s3(64 * 64 * 128, 64 * 128, 128)
+    ptrs = [FAKE] * 10
+    ws_need = lib.of3_trimul_workspace_bytes(1, 64, 128, 128)
+
+    def call(z=FAKE, strides=zs, B=1, N=64, C=128, CH=128, ws=FAKE, ws_bytes=ws_need, dtype=_lib.OF3_DTYPE_BF16):
+        return lib.of3_trimul_fwd(z, strides, None, None, *ptrs, FAKE, B, N, C, CH, 1, 0, ws, ws_bytes, dtype, None)
+
+    assert call(dtype=_lib.OF3_DTYPE_F32) == _lib.OF3_EINVAL      # only bf16 kernels exist
+    assert call(C=96, CH=96) == _lib.OF3_EINVAL                   # unsupported channel count
+    assert call(N=0) == _lib.OF3_EINVAL
+    assert call(ws=None) == _lib.OF3_EINVAL                        # null workspace
+    assert call(ws=FAKE + 8) == _lib.OF3_EINVAL                    # misaligned workspace
+    assert call(ws_bytes=ws_need - 1) == _lib.OF3_ENOSPC          # workspace too small
+    assert call(z=None) == _lib.OF3_EINVAL                         # null tensor
+    assert call(z=FAKE + 2) == _lib.OF3_EINVAL                     # misaligned tensor
+    assert call(strides=_s3(64 * 64 * 128, 64 * 128 + 4, 128)) == _lib.OF3_EINVAL  # stride not a multiple of 8
+
+
+def test_triattn_fwd_rejects_bad_arguments(lib):
+    from of3pair import _lib
+
+    xs = _s3(64 * 64 * 128, 64 * 128, 128)
+    ptrs = [FAKE] * 8
+    ws_need = lib.of3_triattn_workspace_bytes(1, 64, 128, 4, 32)
+
+    def call(x=FAKE, B=1, N=64, C=128, H=4, D=32, ws=FAKE, ws_bytes=ws_need, dtype=_lib.OF3_DTYPE_BF16):
+        return lib.of3_triattn_fwd(x, xs, None, None, *ptrs, FAKE, B, N, C, H, D, 1e9, 0, ws, ws_bytes, dtype, None)
+
+    assert call(dtype=_lib.OF3_DTYPE_F32) == _lib.OF3_EINVAL
+    assert call(H=8) == _lib.OF3_EINVAL
+    assert call(D=64) == _lib.OF3_EINVAL
+    assert call(ws_bytes=ws_need - 1) == _lib.OF3_ENOSPC
+    assert call(x=None) == _lib.OF3_EINVAL
+
+
+def test_stage_entry_points_validate(lib):
+    from of3pair import _lib
+
+    assert lib.of3_trimul_contract(None, FAKE, FAKE, 1, 64, 128, 0, None) == _lib.OF3_EINVAL
+    assert lib.of3_trimul_contract(FAKE, FAKE, FAKE, 1, 64, 128, 9, None) == _lib.OF3_EINVAL   # unknown variant
+    assert lib.of3_trimul_contract(FAKE, FAKE, FAKE, 1, 64, 96, 0, None) == _lib.OF3_EINVAL    # unsupported CH
+    assert lib.of3_triattn_flash(FAKE, FAKE, FAKE, FAKE, FAKE, None, 1, 64, 4, 32, None) == _lib.OF3_EINVAL
+
+
+def test_check_maps_status_to_exceptions(lib):
+    from of3pair import _lib
+
+    _lib.check(0, "ok")
+    with pytest.raises(ValueError):
+        _lib.check(_lib.OF3_EINVAL, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.OF3_ENOSPC, "x")
