@@ -4,25 +4,32 @@
 // fp32, no [N][N] logits in memory.  Inputs come from the projection pass already
 // multiplied by log2(e) (q also by 1/sqrt(D)), so exp() is the hardware exp2.
 //
-// With head width 16 or 32 the kernel is bound by the softmax's VALU work, not by the
-// MFMAs, so the organisation minimises vector instructions per logit:
+// With head width 16 or 32 the kernel is bound by the softmax's vector work and by
+// latencies, not by the MFMAs, so the organisation keeps the vector pipe fed:
 //  * work-group = 8 waves = 8 consecutive rows i of one (head, 128-query range).  The
 //    triangle bias of that range does not depend on i: each 32-key slice of it is brought
-//    into LDS once per work-group (double-buffered) and every wave reads it
-//    straight into the MFMA accumulator, which adds it for free.
+//    into LDS once per work-group and every wave reads it straight into the MFMA
+//    accumulator, which adds it for free.
+//  * everything a key tile needs (the work-group's bias slice, the wave's own K tile and
+//    V^T tile) travels global -> LDS with direct-to-LDS loads, one tile ahead, into
+//    double buffers; the only wait is one vmcnt(0) + barrier per key tile, a whole tile of
+//    arithmetic after the loads were issued.  The XOR swizzles are applied on the global
+//    side (a lane picks which 16-byte chunk it fetches for its fixed LDS slot).
 //  * S^T = K Q^T: A = K tile (row r of the tile is key rowperm16(r), so a lane ends up with
-//    16 consecutive keys of one query), B = Q tile.  O^T = V^T P^T: A = V^T, B = P^T taken
-//    directly from the S^T accumulator registers (no cross-lane movement).  K and V^T are
-//    loaded straight from global memory in operand layout and prefetched one tile ahead.
+//    16 consecutive keys of one query), B = Q tile (registers).  O^T = V^T P^T: A = V^T,
+//    B = P^T taken directly from the S^T accumulator registers (no cross-lane movement).
+//  * inside a key tile the four 32-query tiles are software pipelined: the bias reads and
+//    the q.k MFMAs of the next query tile are issued in the middle of the current one's
+//    exponentials, so a wave overlaps its own matrix and vector work.
 //  * the running maximum is only raised when a logit exceeds it by more than 2^8 (checked
-//    wave-wide with one ballot); otherwise the tile costs per logit one subtract, one exp2,
-//    one add and half a pack.  Any common offset gives the same softmax; the bound keeps
-//    every term far from overflow.
-//  * rows without masked keys never touch the mask bias.  Otherwise, and in the last tile
-//    when N is not a multiple of 32 (padded keys carry -inf), it is added to the triangle
-//    bias first: masked keys get weight exactly 0, and a fully masked row degenerates to a
-//    uniform average over all real keys exactly as the reference's does (-1e9 absorbs the
-//    logits in fp32).
+//    wave-wide with one ballot); otherwise a logit costs one subtract, one exp2, one add
+//    and half a pack.  Any common offset gives the same softmax; the bound keeps every
+//    term far from overflow.
+//  * the mask bias of a key tile rides on one more k-step of the S^T product (A = [mb[key],
+//    0, ...], B = [1, 0, ...]) right after the triangle bias, i.e. (tb + mb) + q.k in the
+//    fp32 accumulator: masked keys get weight exactly 0, padded keys (N not a multiple of
+//    32) carry -inf, and a fully masked row degenerates to a uniform average over all real
+//    keys exactly as the reference's does (-1e9 absorbs the logits in fp32).
 #include "of3_device.h"
 #include "of3_kernels.h"
 
@@ -30,25 +37,48 @@ namespace of3 {
 
 namespace {
 
+#define OF3_GLOBAL_AS __attribute__((address_space(1)))
+#define OF3_LDS_AS __attribute__((address_space(3)))
+
 constexpr int kRows = 8;          // rows i (= waves) per work-group
 constexpr int kRQ = 4;            // 32-query tiles per wave
 constexpr float kRaise = 8.0f;    // raise the running maximum only beyond 2^8
+constexpr int kTbSlots = kRQ * 32 * 8;  // 16-byte slots of one [32*kRQ q][32 k] fp32 bias slice
+constexpr int kTbLoads = kRQ * 4 / kRows;  // direct-to-LDS instructions (8 queries each) per wave and slice
+static_assert(kTbLoads * kRows == kRQ * 4, "the bias slice is split evenly over the waves");
+constexpr int kStages = 3;        // LDS ring: tiles kt (in use), kt+1 (landing or landed), kt+2 (requested)
 
 __device__ __forceinline__ float xhalf(float v) { return __shfl_xor(v, 32, 64); }
+__device__ __forceinline__ void compiler_fence() { __asm__ volatile("" ::: "memory"); }
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {  // vmcnt(N) only (gfx9 encoding, N < 16)
+  static_assert(N >= 0 && N < 16, "low field only");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+}
+
+// swizzle keys of the K / V^T tiles in LDS: rows are read in the order rowperm16(lane), i.e.
+// {x..x+3, x+16..x+19, x+4..x+7, x+20..x+23} per 16 lanes; (row & 1, key) must differ inside
+// every group of 8 lanes and (row & 3, key) inside every group of 16
+__device__ __forceinline__ int key4(int row) {  // 4 chunks (64 bytes) per row
+  return ((((row >> 4) ^ (row >> 1)) & 1) << 1) | (((row >> 2) ^ (row >> 1)) & 1);
+}
+__device__ __forceinline__ int key2(int row) { return (row >> 4) & 1; }  // 2 chunks per row
 
 template <int D>
 __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashArgs p, int n_qc, int n_rg, int total,
                                                                    int per_xcd) {
   constexpr int H = 4;
   constexpr int HD = H * D;
-  constexpr int KSQ = D / 16;           // k-steps of the q.k product
-  constexpr int TBQ = 32 * 8;           // u32x4 slots of one 32 x 32 fp32 bias tile
-  constexpr int TBBUF = kRQ * TBQ;      // one key slice of the whole query range
+  constexpr int KSQ = D / 16;            // k-steps of the q.k product
+  constexpr int QCH = D / 8;             // 16-byte chunks per K row
+  constexpr int KSLOTS = 32 * QCH;       // K tile: 32 keys x D
+  constexpr int VSLOTS = D * 4;          // V^T tile: D channels x 32 keys
+  constexpr int KVS = KSLOTS + VSLOTS;   // one wave's stage
+  constexpr int KI = KSLOTS / 64, VI = VSLOTS / 64;  // direct-to-LDS instructions per tile
 
-  constexpr int QCH = D / 8;             // 16-byte chunks per query row
-  constexpr int QSLOTS = 32 * kRQ * QCH; // one wave's 128 query rows
-  __shared__ u32x4_t tb_lds[2 * TBBUF];          // 32 KB
-  __shared__ u32x4_t q_lds[kRows * QSLOTS];      // 64 KB (D = 32): every wave's own query operands
+  extern __shared__ u32x4_t lds[];
+  u32x4_t* tb_lds = lds;                           // [kStages][kTbSlots]
+  u32x4_t* kv_lds = lds + kStages * kTbSlots;      // [kRows][kStages][KVS]
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -62,7 +92,7 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
   const int rg = (logical / n_qc) % n_rg;
   const int bh = logical / (n_qc * n_rg);
   const int i_raw = rg * kRows + wave;
-  const bool row_valid = i_raw < N;          // wave-uniform; idle waves still take part in the barriers
+  const bool row_valid = i_raw < N;          // wave-uniform; idle waves still take part in the loads and barriers
   const int i = row_valid ? i_raw : N - 1;
   const int b = bh / H, h = bh % H;
   const int q0 = qc * (32 * kRQ);
@@ -73,77 +103,84 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
   const bf16_t* Vt = p.vt + bih * D * Jp;
   const float* tb = p.tbias + ((size_t)b * H + h) * N * Jp;
   const float* mb = p.mbias + ((size_t)b * N + i) * Jp;
-
-  // ---- does this row have masked keys at all?  (wave-uniform)
-  bool row_masked = false;
-  {
-    float acc = 0.f;
-    for (int j = lane * 4; j < N; j += 256) {
-      const float4 t4 = *reinterpret_cast<const float4*>(mb + j);  // j+3 < Jp; entries >= N are -inf
-      acc += (j < N ? t4.x : 0.f) + (j + 1 < N ? t4.y : 0.f) + (j + 2 < N ? t4.z : 0.f) + (j + 3 < N ? t4.w : 0.f);
-    }
-    row_masked = __builtin_amdgcn_ballot_w64(acc != 0.f) != 0;
-  }
-  const bool tail_keys = (N & 31) != 0;
   const int nkt = (N + 31) / 32;
 
-  // ---- query operands (B side of S^T = K Q^T): parked in LDS, 128 rows per wave, chunk
-  // index XOR-ed with a row key so that the operand reads (8 lanes = 8 consecutive rows, same
-  // chunk) are conflict free; fetched again for every key tile instead of living in 32 VGPRs
-  u32x4_t* q_mine = q_lds + wave * QSLOTS;
-  auto q_key = [](int r) { return D == 32 ? ((r >> 1) & 3) : ((r >> 2) & 1); };
-  {
-    constexpr int RPI = 64 / QCH;  // query rows per wave instruction
+  // ---- query operands (B side of S^T = K Q^T) stay in registers
+  u32x4_t qop[kRQ][KSQ];
 #pragma unroll
-    for (int it = 0; it < 32 * kRQ / RPI; ++it) {
-      const int r = it * RPI + lane / QCH, c = lane % QCH;
-      int qrow = q0 + r;
-      qrow = qrow < Jp ? qrow : Jp - 1;
-      q_mine[r * QCH + (c ^ q_key(r))] = *reinterpret_cast<const u32x4_t*>(Q + (size_t)qrow * D + 8 * c);
-    }
+  for (int rq = 0; rq < kRQ; ++rq) {
+    int qrow = q0 + 32 * rq + l32;
+    qrow = qrow < Jp ? qrow : Jp - 1;
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ++ks)
+      qop[rq][ks] = *reinterpret_cast<const u32x4_t*>(Q + (size_t)qrow * D + 16 * ks + 8 * lh);
   }
-  int q_rd[KSQ];
-#pragma unroll
-  for (int ks = 0; ks < KSQ; ++ks) q_rd[ks] = l32 * QCH + ((2 * ks + lh) ^ q_key(l32));
 
-  // ---- triangle-bias slices: 128 queries x 32 keys fp32 = 16 KB per key tile, fetched by
-  // the whole work-group (two 16-byte pieces per thread, 8 lanes per 128-byte query row),
-  // held in registers during the current tile's arithmetic and written to the other LDS
-  // buffer afterwards.  LDS slot of (tile rq, query r, chunk c) = rq*256 + r*8 + (c ^ (r & 7)).
-  const float* tb_src[2];
-  int tb_dst[2];
+  // ---- direct-to-LDS sources.  LDS slot of an instruction = its base + lane.
+  // bias slice: instruction n of wave w fills slots 64*(2w+n)..+63; slot t holds chunk
+  // (t & 7) ^ (q & 7) of query q = t >> 3 (128-byte rows of 32 keys)
+  // (byte offsets from wave-uniform bases, so that the loads use scalar base + 32-bit lane offset)
+  uint32_t tb_off[kTbLoads];
 #pragma unroll
-  for (int n = 0; n < 2; ++n) {
-    const int qloc = 64 * n + (tid >> 3), chunk = tid & 7;  // query within the 128 range
+  for (int n = 0; n < kTbLoads; ++n) {
+    const int t = 64 * (kTbLoads * wave + n) + lane;
+    const int qloc = t >> 3, chunk = (t & 7) ^ (qloc & 7);
     int qrow = q0 + qloc;
     qrow = qrow < N ? qrow : N - 1;
-    tb_src[n] = tb + (size_t)qrow * Jp + 4 * chunk;
-    tb_dst[n] = (qloc >> 5) * TBQ + (qloc & 31) * 8 + (chunk ^ (qloc & 7));
+    tb_off[n] = (uint32_t)(((size_t)qrow * Jp + 4 * chunk) * sizeof(float));
   }
-  auto load_tb = [&](int kt, u32x4_t (&r)[2]) {
+  // K tile: slot t holds chunk (t % QCH) ^ key(row) of key row t / QCH
+  uint32_t k_off[KI];
 #pragma unroll
-    for (int n = 0; n < 2; ++n) r[n] = *reinterpret_cast<const u32x4_t*>(tb_src[n] + 32 * kt);
-  };
-  auto store_tb = [&](const u32x4_t (&r)[2], int buf) {
+  for (int n = 0; n < KI; ++n) {
+    const int t = 64 * n + lane;
+    const int row = t / QCH, chunk = (t % QCH) ^ (QCH == 4 ? key4(row) : key2(row));
+    k_off[n] = (uint32_t)((row * D + 8 * chunk) * sizeof(bf16_t));
+  }
+  // V^T tile: slot t holds chunk (t & 3) ^ key4(row) of channel row t >> 2 (64-byte rows of 32 keys)
+  uint32_t v_off[VI];
 #pragma unroll
-    for (int n = 0; n < 2; ++n) tb_lds[buf * TBBUF + tb_dst[n]] = r[n];
+  for (int n = 0; n < VI; ++n) {
+    const int t = 64 * n + lane;
+    const int row = t >> 2, chunk = (t & 3) ^ key4(row);
+    v_off[n] = (uint32_t)((row * 32 + 8 * chunk) * sizeof(bf16_t));
+  }
+  u32x4_t* kv_mine = kv_lds + wave * (kStages * KVS);
+  auto issue_loads = [&](int kt, int buf) {
+    u32x4_t* tdst = tb_lds + buf * kTbSlots + 64 * kTbLoads * wave;
+    u32x4_t* kdst = kv_mine + buf * KVS;
+    const char* tbase = reinterpret_cast<const char*>(tb + 32 * kt);
+    const char* kbase = reinterpret_cast<const char*>(K + (size_t)kt * (32 * D));
+    const char* vbase = reinterpret_cast<const char*>(Vt + (size_t)kt * (32 * D));
+#pragma unroll
+    for (int n = 0; n < kTbLoads; ++n)
+      __builtin_amdgcn_global_load_lds((const void OF3_GLOBAL_AS*)(tbase + tb_off[n]),
+                                       (void OF3_LDS_AS*)(tdst + 64 * n), 16, 0, 0);
+#pragma unroll
+    for (int n = 0; n < KI; ++n)
+      __builtin_amdgcn_global_load_lds((const void OF3_GLOBAL_AS*)(kbase + k_off[n]),
+                                       (void OF3_LDS_AS*)(kdst + 64 * n), 16, 0, 0);
+#pragma unroll
+    for (int n = 0; n < VI; ++n)
+      __builtin_amdgcn_global_load_lds((const void OF3_GLOBAL_AS*)(vbase + v_off[n]),
+                                       (void OF3_LDS_AS*)(kdst + KSLOTS + 64 * n), 16, 0, 0);
   };
 
-  // ---- key / value operands of one tile, loaded in operand layout
+  // ---- operand read slots
   const int krow = rowperm16(l32);
   const bool vvalid = krow < D;
-  auto load_kv = [&](int kt, u32x4_t (&kop)[KSQ], u32x4_t (&vop)[2]) {
-    const int key0 = 32 * kt;
+  int k_rd[KSQ], v_rd[2];
 #pragma unroll
-    for (int s = 0; s < KSQ; ++s)
-      kop[s] = *reinterpret_cast<const u32x4_t*>(K + (size_t)(key0 + krow) * D + 16 * s + 8 * lh);
+  for (int ks = 0; ks < KSQ; ++ks) k_rd[ks] = krow * QCH + ((2 * ks + lh) ^ (QCH == 4 ? key4(krow) : key2(krow)));
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      u32x4_t v = {0u, 0u, 0u, 0u};
-      if (vvalid) v = *reinterpret_cast<const u32x4_t*>(Vt + (size_t)kt * (D * 32) + krow * 32 + 16 * lh + 8 * s2);
-      vop[s2] = v;
-    }
-  };
+  for (int s2 = 0; s2 < 2; ++s2) {
+    const int vr = krow & (D - 1);
+    v_rd[s2] = KSLOTS + vr * 4 + ((2 * lh + s2) ^ key4(vr));
+  }
+  // bias slot this lane reads for tile rq, chunk c: rq*256 + l32*8 + ((4*lh + c) ^ (l32 & 7))
+  int tb_rd[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) tb_rd[c] = l32 * 8 + ((4 * lh + c) ^ (l32 & 7));
 
   float m_run[kRQ], l_run[kRQ];
   f32x16_t oacc[kRQ];
@@ -154,39 +191,47 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
     oacc[rq] = zero16();
   }
 
-  u32x4_t kop[2][KSQ], vop[2][2], tbr[2];
-  load_tb(0, tbr);
-  load_kv(0, kop[0], vop[0]);
-  store_tb(tbr, 0);
-
-  // the bias slot this lane reads for tile rq, chunk c: rq*256 + l32*8 + ((4*lh + c) ^ (l32 & 7))
-  const int tb_rd = l32 * 8;
-  const int tb_key = l32 & 7;
-
-  auto tile = [&](int kt, const u32x4_t (&kc)[KSQ], const u32x4_t (&vc)[2], const u32x4_t* tbuf) {
-    const bool use_mb = row_masked || (tail_keys && kt == nkt - 1);  // wave-uniform
-    const float* mbt = mb + 32 * kt + 16 * lh;
+  // One key tile.
+  // Mask bias of a tile: one more k-step of the S^T product with A = [mb[key], 0, ...] and
+  // B = [1, 0, ...] adds mb[key] to every query's logit inside the matrix pipe, right after
+  // the triangle bias ((tb + mb) + q.k).  bf16 holds 0 and -inf exactly and -1e9*log2(e) to
+  // 3 digits, which is all a mask bias has to be.
+  float mb_cur = 0.f;  // mb[32*kt + rowperm16(l32)] of the current tile
+  const u32x4_t one_op = {lh == 0 ? 0x3F80u : 0u, 0u, 0u, 0u};
+  auto tile = [&](int buf) {
+    const u32x4_t mb_op = {lh == 0 ? pack_bf16(mb_cur, 0.f) : 0u, 0u, 0u, 0u};
+    const u32x4_t* tbuf = tb_lds + buf * kTbSlots;
+    const u32x4_t* kvb = kv_mine + buf * KVS;
+    u32x4_t kc[KSQ], vc[2];
 #pragma unroll
-    for (int rq = 0; rq < kRQ; ++rq) {
+    for (int ks = 0; ks < KSQ; ++ks) kc[ks] = kvb[k_rd[ks]];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const u32x4_t v = kvb[v_rd[s2]];
+      const u32x4_t z = {0u, 0u, 0u, 0u};
+      vc[s2] = vvalid ? v : z;
+    }
+    auto bias_init = [&](int rq) {
       f32x16_t s;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        const u32x4_t t = tbuf[rq * TBQ + tb_rd + ((4 * lh + c) ^ tb_key)];
+        const u32x4_t t = tbuf[rq * 256 + tb_rd[c]];
 #pragma unroll
         for (int e = 0; e < 4; ++e) s[4 * c + e] = __uint_as_float(t[e]);
       }
-      if (use_mb) {
+      return s;
+    };
+
+    f32x16_t s = bias_init(0);
+    s = mfma_32x32x16(mb_op, one_op, s);
 #pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4) {
-          const float4 t4 = *reinterpret_cast<const float4*>(mbt + 4 * c4);  // same 64 bytes for every rq: L1 hits
-          s[4 * c4] += t4.x;
-          s[4 * c4 + 1] += t4.y;
-          s[4 * c4 + 2] += t4.z;
-          s[4 * c4 + 3] += t4.w;
-        }
-      }
+    for (int ks = 0; ks < KSQ; ++ks) s = mfma_32x32x16(kc[ks], qop[0][ks], s);
+
 #pragma unroll
-      for (int ks = 0; ks < KSQ; ++ks) s = mfma_32x32x16(kc[ks], q_mine[rq * 32 * QCH + q_rd[ks]], s);
+    for (int rq = 0; rq < kRQ; ++rq) {
+      // bias of the next query tile: LDS reads in flight during the maximum search
+      f32x16_t sn;
+      if (rq + 1 < kRQ) sn = bias_init(rq + 1);
 
       float mx = fmaxf(s[0], s[1]);
 #pragma unroll
@@ -201,37 +246,62 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
         m_run[rq] = m_new;
       }
       const float m = m_run[rq];
-      float rs = 0.f;
+
+      // exponentials in groups; the next tile's q.k MFMAs and this tile's P V MFMAs are
+      // slipped in between so that the matrix pipe works under the vector work.  The row
+      // sum is taken over the bf16-rounded weights (the ones the P V product uses), two per
+      // instruction with the bf16 dot product.
+      float rs = l_run[rq];  // this lane's 16 keys; the two halves are combined at the end
+      auto expw = [&](int w) {  // weights 2w, 2w+1 -> one packed register
+        const uint32_t pk = pack_bf16(fast_exp2(s[2 * w] - m), fast_exp2(s[2 * w + 1] - m));
+        rs = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3F803F80u),
+                                             rs, false);
+        return pk;
+      };
+      u32x4_t pop0, pop1;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        s[v] = fast_exp2(s[v] - m);
-        rs += s[v];
+      for (int w = 0; w < 4; ++w) pop0[w] = expw(w);
+      __builtin_amdgcn_sched_barrier(0);
+      if (rq + 1 < kRQ) {
+        sn = mfma_32x32x16(mb_op, one_op, sn);
+        sn = mfma_32x32x16(kc[0], qop[rq + 1 < kRQ ? rq + 1 : 0][0], sn);
       }
-      l_run[rq] += rs;  // this lane's 16 keys; the two halves are combined at the end
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2) {
-        u32x4_t pop;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) pop[w] = pack_bf16(s[8 * s2 + 2 * w], s[8 * s2 + 2 * w + 1]);
-        oacc[rq] = mfma_32x32x16(vc[s2], pop, oacc[rq]);
-      }
-      __builtin_amdgcn_sched_barrier(0);  // one query tile at a time keeps the live registers within budget
+      __builtin_amdgcn_sched_barrier(0);
+      pop1[0] = expw(4);
+      pop1[1] = expw(5);
+      __builtin_amdgcn_sched_barrier(0);
+      if (KSQ == 2 && rq + 1 < kRQ) sn = mfma_32x32x16(kc[KSQ - 1], qop[rq + 1 < kRQ ? rq + 1 : 0][KSQ - 1], sn);
+      oacc[rq] = mfma_32x32x16(vc[0], pop0, oacc[rq]);
+      __builtin_amdgcn_sched_barrier(0);
+      pop1[2] = expw(6);
+      pop1[3] = expw(7);
+      __builtin_amdgcn_sched_barrier(0);
+      oacc[rq] = mfma_32x32x16(vc[1], pop1, oacc[rq]);
+      __builtin_amdgcn_sched_barrier(0);
+      l_run[rq] = rs;
+      if (rq + 1 < kRQ) s = sn;
     }
   };
 
+  constexpr int LPT = kTbLoads + KI + VI;  // direct-to-LDS instructions per tile and wave
+  float mb_next = mb[krow];
+  constexpr int PD = kStages - 1;  // prefetch distance in tiles
+#pragma unroll
+  for (int t = 0; t < PD; ++t)
+    if (t < nkt) issue_loads(t, t);
+  int buf = 0;  // kt % kStages
   for (int kt = 0; kt < nkt; ++kt) {
-    __syncthreads();  // bias slice kt is visible; nobody reads the other buffer any more
-    const bool more = kt + 1 < nkt;
-    if (more) {  // next tile's operands and bias slice travel while this tile is computed
-      load_tb(kt + 1, tbr);
-      load_kv(kt + 1, kop[1], vop[1]);
-    }
-    tile(kt, kop[0], vop[0], tb_lds + (kt & 1) * TBBUF);
-    if (more) store_tb(tbr, (kt + 1) & 1);
-#pragma unroll
-    for (int s = 0; s < KSQ; ++s) kop[0][s] = kop[1][s];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) vop[0][s] = vop[1][s];
+    // this wave's loads of tile kt have landed (those of later tiles may still be in flight) ...
+    if (PD >= 2 && kt + PD - 1 < nkt) wait_vmcnt<(PD - 1) * LPT>();
+    else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();      // ... and everybody's; nobody reads tile kt-1's buffers any more
+    compiler_fence();
+    mb_cur = mb_next;
+    if (kt + 1 < nkt) mb_next = mb[32 * (kt + 1) + krow];  // an ordinary load, issued before the prefetch
+    if (kt + PD < nkt) issue_loads(kt + PD, buf == 0 ? kStages - 1 : buf - 1);
+    tile(buf);
+    buf = buf == kStages - 1 ? 0 : buf + 1;
+    compiler_fence();
   }
 
   // ---- finalize: lane (query l32, half lh) owns head channels 16*lh + v
@@ -258,12 +328,25 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
 }
 
 template <int D>
+constexpr int lds_bytes() {
+  return (kStages * kTbSlots + kRows * kStages * (32 * (D / 8) + D * 4)) * 16;
+}
+
+template <int D>
 hipError_t launch(const TriattnFlashArgs& a, hipStream_t stream) {
+  auto kern = triattn_flash_kernel<D>;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<D>());
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
   const int n_qc = (a.N + 32 * kRQ - 1) / (32 * kRQ), n_rg = (a.N + kRows - 1) / kRows;
   const long total = (long)n_qc * n_rg * a.B * a.H;
   const int per_xcd = (int)((total + 7) / 8);
-  hipLaunchKernelGGL((triattn_flash_kernel<D>), dim3(per_xcd * 8), dim3(64 * kRows), 0, stream, a, n_qc, n_rg,
-                     (int)total, per_xcd);
+  hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(64 * kRows), lds_bytes<D>(), stream, a, n_qc, n_rg, (int)total,
+                     per_xcd);
   return hipGetLastError();
 }
 
