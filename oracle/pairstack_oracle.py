@@ -162,6 +162,68 @@ def triattn_update(x, mask, p, no_heads: int, starting: bool = True, inf: float 
 
 
 # --------------------------------------------------------------------------
+# the same two updates restricted to a few output positions (for sizes at which
+# the full fp32 evaluation does not finish in seconds); 3-D inputs only
+# --------------------------------------------------------------------------
+def trimul_update_at(z, mask, p, outgoing: bool, rows, cols):
+    """trimul_update(z, mask, p, outgoing)[rows][:, cols] for z [N, N, C], computed from the
+    2*(len(rows)+len(cols)) rows/columns of z the result depends on (tmu.py:77-82:
+    outgoing x[i,j] contracts row i of a with row j of b, incoming column i with column j)."""
+    rows = torch.as_tensor(rows)
+    cols = torch.as_tensor(cols)
+    if mask is None:
+        mask = z.new_ones(z.shape[:-1])
+
+    def gated(zs, ms, which):
+        zn = layer_norm(zs, p["layer_norm_in.weight"], p["layer_norm_in.bias"])
+        t = ms.to(z.dtype).unsqueeze(-1)
+        t = t * torch.sigmoid(linear(zn, p["linear_%s_g.weight" % which]))
+        return t * linear(zn, p["linear_%s_p.weight" % which])
+
+    if outgoing:
+        a = gated(z[rows], mask[rows], "a")                                  # [R, N(k), C]
+        b = gated(z[cols], mask[cols], "b")                                  # [S, N(k), C]
+    else:
+        a = gated(z[:, rows].transpose(0, 1), mask[:, rows].transpose(0, 1), "a")   # a[k, i] -> [R, N(k), C]
+        b = gated(z[:, cols].transpose(0, 1), mask[:, cols].transpose(0, 1), "b")
+    x = torch.einsum("ikc,jkc->ijc", a, b)
+    x = layer_norm(x, p["layer_norm_out.weight"], p["layer_norm_out.bias"])
+    x = linear(x, p["linear_z.weight"])
+    zn = layer_norm(z[rows][:, cols], p["layer_norm_in.weight"], p["layer_norm_in.bias"])
+    return x * torch.sigmoid(linear(zn, p["linear_g.weight"]))
+
+
+def triattn_update_rows(x, mask, p, no_heads: int, rows, starting: bool = True, inf: float = INF):
+    """Rows ``rows`` of the module frame of triattn_update(x, mask, p, no_heads, starting) for
+    x [N, N, C]: result[r] = update[rows[r], :, :] (starting) or update[:, rows[r], :]
+    (ending).  Needs the triangle bias of the whole tensor but q, k, v of those rows only."""
+    rows = torch.as_tensor(rows)
+    if mask is None:
+        mask = x.new_ones(x.shape[:-1])
+    if not starting:
+        x = x.transpose(0, 1)
+        mask = mask.transpose(0, 1)
+    H = no_heads
+    tb = torch.empty(H, x.shape[0], x.shape[1], dtype=x.dtype)
+    for r0 in range(0, x.shape[0], 256):  # linear_z(LayerNorm(x)) in slabs, [I, J, H] -> [H, I, J]
+        xn = layer_norm(x[r0:r0 + 256], p["layer_norm.weight"], p["layer_norm.bias"])
+        tb[:, r0:r0 + 256] = linear(xn, p["linear_z.weight"]).permute(2, 0, 1)
+    xr = layer_norm(x[rows], p["layer_norm.weight"], p["layer_norm.bias"])   # [R, J, C]
+    mask_bias = (inf * (mask[rows].to(x.dtype) - 1))[:, None, None, :]        # [R, 1, 1, J]
+    q = linear(xr, p["mha.linear_q.weight"])
+    k = linear(xr, p["mha.linear_k.weight"])
+    v = linear(xr, p["mha.linear_v.weight"])
+    c = q.shape[-1] // H
+    q = q.view(q.shape[:-1] + (H, c)).transpose(-2, -3) / math.sqrt(c)
+    k = k.view(k.shape[:-1] + (H, c)).transpose(-2, -3)
+    v = v.view(v.shape[:-1] + (H, c)).transpose(-2, -3)
+    o = attention_core(q, k, v, [mask_bias, tb.unsqueeze(0)]).transpose(-2, -3)  # [R, J, H, c]
+    g = torch.sigmoid(linear(xr, p["mha.linear_g.weight"]))
+    o = (o * g.view(g.shape[:-1] + (H, c))).reshape(o.shape[:-2] + (H * c,))
+    return linear(o, p["mha.linear_o.weight"])
+
+
+# --------------------------------------------------------------------------
 # block sequencing
 # --------------------------------------------------------------------------
 def _sub(p, prefix):

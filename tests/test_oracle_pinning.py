@@ -167,3 +167,33 @@ def test_template_stack_is_per_template_blocks():
         for p in blocks:
             zt = orc.pair_stack_block(zt, mask[:, ti], p, heads)
         assert torch.equal(got[:, ti], zt)
+
+
+# ---- the position-restricted forms used at sizes the full oracle cannot reach -----------------
+@pytest.mark.parametrize("outgoing", [True, False])
+def test_trimul_update_at_equals_full(outgoing):
+    gen = torch.Generator().manual_seed(21)
+    n, c = 12, 16
+    z = torch.randn(n, n, c, generator=gen)
+    mask = (torch.rand(n, n, generator=gen) > 0.2).float()
+    p = orc.make_trimul_params(gen, c, c)
+    rows, cols = [0, 5, 11], [2, 3, 7, 10]
+    full = orc.trimul_update(z, mask, p, outgoing)
+    part = orc.trimul_update_at(z, mask, p, outgoing, rows, cols)
+    assert (part - full[rows][:, cols]).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("starting", [True, False])
+def test_triattn_update_rows_equals_full(starting):
+    gen = torch.Generator().manual_seed(22)
+    n, c, heads, d = 12, 16, 2, 4
+    x = torch.randn(n, n, c, generator=gen)
+    mask = (torch.rand(n, n, generator=gen) > 0.2).float()
+    mask[4, :] = 0.0
+    mask[:, 6] = 0.0
+    p = orc.make_triattn_params(gen, c, d, heads)
+    rows = [0, 4, 6, 11]
+    full = orc.triattn_update(x, mask, p, heads, starting=starting)
+    part = orc.triattn_update_rows(x, mask, p, heads, rows, starting=starting)
+    want = full[rows] if starting else full[:, rows].transpose(0, 1)
+    assert (part - want).abs().max() < 1e-5
