@@ -37,6 +37,13 @@
  * ending-node attention of base_blocks.py:380-404, tri_att.py:126-128) is expressed by
  * swapping stride_i and stride_j, no copy is needed.  Masks are fp32 [B,N,N] with their
  * own element strides; a null mask means all ones (tmu.py:482-483, tri_att.py:120-124).
+ *
+ * dtype: OF3_DTYPE_BF16 selects the MFMA kernels described above.  OF3_DTYPE_F32 (the
+ * reference's default inference precision) is served by of3_trimul_fwd / of3_triattn_fwd
+ * only: every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
+ * element counts, any N, C and CH <= 256, H*D <= 256 with D in {16, 32, 64}; plain fp32
+ * arithmetic in the reference's order of operations (no MFMA, not the fast path).  The
+ * stage entry points are bf16 only.
  */
 #ifndef OF3PAIR_H
 #define OF3PAIR_H
@@ -66,6 +73,8 @@ int64_t of3_padded_n(int64_t n);
 
 /* Bytes of scratch of3_trimul_fwd needs: a, b, x = 3 * B*CH*NP*NP bf16. */
 int64_t of3_trimul_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t CH);
+/* The same for either dtype (fp32: a, b, x = 3 * B*CH*N*N floats). */
+int64_t of3_trimul_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t CH);
 
 /* a, b: gated, masked projections, channel-major in "k-panels" of 32 contracted indices:
  * shape [B][CH][NP/32][NP][32], a[b][c][k/32][i][k%32] = a_ref[b,i,k,c] (outgoing) or
@@ -101,6 +110,8 @@ int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask,
  *   q, k  [B][N][H][NP][D] bf16      vt [B][N][H][NP/32][D][32] bf16 (v transposed, 32-key panels)
  *   tbias [B][H][N][NP] fp32         mbias [B][N][NP] fp32       o [B][N][N][H*D] bf16 */
 int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D);
+/* The same for either dtype (fp32: q, k, v, o = 4 * B*N*N*H*D floats, triangle bias B*H*N*N floats). */
+int64_t of3_triattn_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t H, int64_t D);
 
 /* q is pre-multiplied by log2(e)/sqrt(D); tbias and mbias by log2(e); mbias is -inf for
  * j >= N.  (i, j) are the module's frame as given by x_strides / mask_strides. */

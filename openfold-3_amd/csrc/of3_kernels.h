@@ -85,4 +85,32 @@ struct TriattnOutArgs {
 };
 hipError_t triattn_out_launch(const TriattnOutArgs& args, int C, int HD, hipStream_t stream);
 
+// ---- fp32 path (pair_f32.hip): whole updates, any N, C and C_hidden <= 256, head width 16/32/64
+struct TrimulF32Args {
+  const float* z;
+  const float* mask;                 // may be null
+  PairView z_view, mask_view;        // as the projection pass walks them (swapped for incoming)
+  PairView z_canonical;              // (i, j) orientation of z and out
+  const float *ln_in_w, *ln_in_b, *ln_out_w, *ln_out_b;
+  const float *w_ap, *w_ag, *w_bp, *w_bg, *w_g, *w_z;
+  float *a, *b, *x;                  // workspace, [B][CH][N][N] each
+  float* out;
+  int B, N, C, CH, add_residual;
+};
+hipError_t trimul_fwd_f32(const TrimulF32Args& args, hipStream_t stream);
+
+struct TriattnF32Args {
+  const float* x;
+  const float* mask;                 // may be null
+  PairView x_view, mask_view;        // module frame
+  const float *ln_w, *ln_b, *w_q, *w_k, *w_v, *w_b, *w_g, *w_o;
+  float *q, *k, *v;                  // workspace, [B][N][H][N][D] each
+  float *tb;                         // workspace, [B][H][N][N]
+  float *o;                          // workspace, [B][N][N][H*D]
+  float* out;
+  int B, N, C, H, D, add_residual;
+  float inf;
+};
+hipError_t triattn_fwd_f32(const TriattnF32Args& args, hipStream_t stream);
+
 }  // namespace of3

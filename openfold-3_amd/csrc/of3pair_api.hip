@@ -36,6 +36,16 @@ inline bool mask_ok(const float* mask, const int64_t s[3]) {
   return s && s[0] >= 0 && s[1] >= 0 && s[2] >= 0;
 }
 
+inline bool f32_trimul_dims_ok(int64_t B, int64_t N, int64_t C, int64_t CH) {
+  return B >= 1 && N >= 1 && N <= (1 << 16) && C >= 1 && C <= 256 && CH >= 1 && CH <= 256;
+}
+inline bool f32_triattn_dims_ok(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
+  return B >= 1 && N >= 1 && N <= (1 << 16) && C >= 1 && C <= 256 && H >= 1 && (D == 16 || D == 32 || D == 64) &&
+         H * D <= 256;
+}
+inline bool f32_strides_ok(const int64_t s[3]) { return s && s[0] >= 0 && s[1] > 0 && s[2] > 0; }
+inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+
 inline of3::PairView view(const int64_t s[3], bool swap) {
   of3::PairView v;
   v.stride_b = s[0];
@@ -87,6 +97,12 @@ int64_t of3_trimul_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t CH) 
   if (!trimul_dims_ok(B, N, C, CH)) return OF3_EINVAL;
   const int64_t Np = padded(N);
   return 3 * align256(B * CH * Np * Np * 2);
+}
+
+int64_t of3_trimul_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t CH) {
+  if (dtype == OF3_DTYPE_BF16) return of3_trimul_workspace_bytes(B, N, C, CH);
+  if (dtype != OF3_DTYPE_F32 || !f32_trimul_dims_ok(B, N, C, CH)) return OF3_EINVAL;
+  return 3 * align256(B * CH * N * N * 4);
 }
 
 int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
@@ -159,6 +175,44 @@ int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask,
                    const void* w_a_p, const void* w_a_g, const void* w_b_p, const void* w_b_g, const void* w_g,
                    const void* w_z, void* out, int64_t B, int64_t N, int64_t C, int64_t CH, int outgoing,
                    int add_residual, void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
+  if (dtype == OF3_DTYPE_F32) {
+    if (!f32_trimul_dims_ok(B, N, C, CH) || !f32_strides_ok(z_strides) || !mask_ok(mask, mask_strides)) return OF3_EINVAL;
+    const void* ptrs[] = {z, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_a_p, w_a_g, w_b_p, w_b_g, w_g, w_z, out};
+    for (const void* p : ptrs)
+      if (!p || !aligned4(p)) return OF3_EINVAL;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OF3_EINVAL;
+    if (workspace_bytes < of3_trimul_workspace_bytes_for(dtype, B, N, C, CH)) return OF3_ENOSPC;
+    const int64_t part = align256(B * CH * N * N * 4);
+    char* ws = static_cast<char*>(workspace);
+    auto f = [](const void* p) { return static_cast<const float*>(p); };
+    of3::TrimulF32Args a;
+    a.z = f(z);
+    a.mask = mask;
+    a.z_view = view(z_strides, !outgoing);
+    a.mask_view = mask_view(mask, mask_strides, !outgoing);
+    a.z_canonical = view(z_strides, false);
+    a.ln_in_w = f(ln_in_w);
+    a.ln_in_b = f(ln_in_b);
+    a.ln_out_w = f(ln_out_w);
+    a.ln_out_b = f(ln_out_b);
+    a.w_ap = f(w_a_p);
+    a.w_ag = f(w_a_g);
+    a.w_bp = f(w_b_p);
+    a.w_bg = f(w_b_g);
+    a.w_g = f(w_g);
+    a.w_z = f(w_z);
+    a.a = reinterpret_cast<float*>(ws);
+    a.b = reinterpret_cast<float*>(ws + part);
+    a.x = reinterpret_cast<float*>(ws + 2 * part);
+    a.out = static_cast<float*>(out);
+    a.B = (int)B;
+    a.N = (int)N;
+    a.C = (int)C;
+    a.CH = (int)CH;
+    a.add_residual = add_residual ? 1 : 0;
+    hipError_t e = of3::trimul_fwd_f32(a, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? OF3_OK : (e == hipErrorInvalidValue ? (int)OF3_EINVAL : fail_hip(e));
+  }
   if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
   if (!trimul_dims_ok(B, N, C, CH)) return OF3_EINVAL;
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OF3_EINVAL;
@@ -183,6 +237,12 @@ int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, 
   const int64_t Np = padded(N);
   const int64_t qkv = align256(B * N * H * Np * D * 2);
   return 3 * qkv + align256(B * H * N * Np * 4) + align256(B * N * Np * 4) + align256(B * N * N * H * D * 2);
+}
+
+int64_t of3_triattn_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
+  if (dtype == OF3_DTYPE_BF16) return of3_triattn_workspace_bytes(B, N, C, H, D);
+  if (dtype != OF3_DTYPE_F32 || !f32_triattn_dims_ok(B, N, C, H, D)) return OF3_EINVAL;
+  return 4 * align256(B * N * N * H * D * 4) + align256(B * H * N * N * 4);
 }
 
 int of3_triattn_proj(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
@@ -268,6 +328,45 @@ int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask
                     const void* w_v, const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C,
                     int64_t H, int64_t D, float inf, int add_residual, void* workspace, int64_t workspace_bytes,
                     int dtype, void* stream) {
+  if (dtype == OF3_DTYPE_F32) {
+    if (!f32_triattn_dims_ok(B, N, C, H, D) || !f32_strides_ok(x_strides) || !mask_ok(mask, mask_strides)) return OF3_EINVAL;
+    const void* ptrs[] = {x, ln_w, ln_b, w_bias, w_q, w_k, w_v, w_g, w_o, out};
+    for (const void* p : ptrs)
+      if (!p || !aligned4(p)) return OF3_EINVAL;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OF3_EINVAL;
+    if (workspace_bytes < of3_triattn_workspace_bytes_for(dtype, B, N, C, H, D)) return OF3_ENOSPC;
+    const int64_t part = align256(B * N * N * H * D * 4);
+    char* ws = static_cast<char*>(workspace);
+    auto f = [](const void* p) { return static_cast<const float*>(p); };
+    of3::TriattnF32Args a;
+    a.x = f(x);
+    a.mask = mask;
+    a.x_view = view(x_strides, false);
+    a.mask_view = mask_view(mask, mask_strides, false);
+    a.ln_w = f(ln_w);
+    a.ln_b = f(ln_b);
+    a.w_q = f(w_q);
+    a.w_k = f(w_k);
+    a.w_v = f(w_v);
+    a.w_b = f(w_bias);
+    a.w_g = f(w_g);
+    a.w_o = f(w_o);
+    a.q = reinterpret_cast<float*>(ws);
+    a.k = reinterpret_cast<float*>(ws + part);
+    a.v = reinterpret_cast<float*>(ws + 2 * part);
+    a.o = reinterpret_cast<float*>(ws + 3 * part);
+    a.tb = reinterpret_cast<float*>(ws + 4 * part);
+    a.out = static_cast<float*>(out);
+    a.B = (int)B;
+    a.N = (int)N;
+    a.C = (int)C;
+    a.H = (int)H;
+    a.D = (int)D;
+    a.add_residual = add_residual ? 1 : 0;
+    a.inf = inf;
+    hipError_t e = of3::triattn_fwd_f32(a, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? OF3_OK : (e == hipErrorInvalidValue ? (int)OF3_EINVAL : fail_hip(e));
+  }
   if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
   if (!triattn_dims_ok(B, N, C, H, D)) return OF3_EINVAL;
   if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return OF3_EINVAL;

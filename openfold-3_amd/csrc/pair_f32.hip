@@ -1,0 +1,391 @@
+// fp32 path of the two pair-stack updates (OF3_DTYPE_F32): the reference's default inference
+// precision (fp32 end to end).  Same mathematics and the same rounding-free order of
+// operations as the reference's stock PyTorch path:
+//   triangle multiplication   triangular_multiplicative_update.py:482-503, :71-97
+//   triangle attention        triangular_attention.py:102-167, attention.py:94-135,265-302
+// These kernels are written for exactness and generality (any N, C, C_hidden <= 256, head
+// width <= 64), with plain fp32 FMA arithmetic, full-precision expf and no MFMA; they are the
+// precision reference of the library on the GPU, not its fast path (that is the bf16 path).
+//
+// Layouts (workspace, fp32): a, b, x  [B][CH][N][N] with a[b][c][i][k] (k contracted);
+// q, k, v [B][N(i)][H][N(j)][D]; triangle bias [B][H][N][N]; o [B][N][N][H*D].
+#include "of3_kernels.h"
+
+namespace of3 {
+
+namespace {
+
+constexpr int kP = 8;        // positions per work-group in the position-wise kernels
+constexpr int kThreads = 256;
+constexpr int kMaxC = 256;
+constexpr float kEps = 1e-5f;
+
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// LayerNorm of kP positions (32 lanes each) from global rows into shared xn[kP][C].
+// src(pos) returns the pointer to the C channels of position pos or nullptr (out of range).
+template <typename Src>
+__device__ __forceinline__ void layer_norm_rows(Src src, const float* __restrict__ w, const float* __restrict__ bsh,
+                                                int C, float (*xn)[kMaxC]) {
+  const int pos = threadIdx.x >> 5, l = threadIdx.x & 31;
+  const float* row = src(pos);
+  float s = 0.f;
+  if (row)
+    for (int c = l; c < C; c += 32) s += row[c];
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, 32);
+  const float mean = s / (float)C;
+  float q = 0.f;
+  if (row)
+    for (int c = l; c < C; c += 32) {
+      const float d = row[c] - mean;
+      q += d * d;
+    }
+#pragma unroll
+  for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 32);
+  const float rstd = 1.0f / sqrtf(q / (float)C + kEps);
+  for (int c = l; c < C; c += 32) xn[pos][c] = row ? (row[c] - mean) * rstd * w[c] + bsh[c] : 0.f;
+}
+
+__device__ __forceinline__ float dot_row(const float* __restrict__ x, const float* __restrict__ w, int n) {
+  float acc = 0.f;
+  for (int k = 0; k < n; ++k) acc = fmaf(x[k], w[k], acc);
+  return acc;
+}
+
+// ---- triangle multiplication -----------------------------------------------------------------
+struct TrimulF32 {
+  const float *z, *mask;
+  PairView zv, mv;          // view used by the projection pass (swapped for the incoming update)
+  PairView zc;              // canonical view (output pass)
+  const float *ln_in_w, *ln_in_b, *ln_out_w, *ln_out_b;
+  const float *w_ap, *w_ag, *w_bp, *w_bg, *w_g, *w_z;
+  float *a, *b, *x, *out;
+  int B, N, C, CH, add_residual;
+};
+
+__global__ __launch_bounds__(kThreads) void trimul_proj_f32(TrimulF32 p, int groups) {
+  __shared__ float xn[kP][kMaxC];
+  __shared__ float msk[kP];
+  const int N = p.N, C = p.C, CH = p.CH;
+  const int g = blockIdx.x % groups, r = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int k0 = g * kP;
+  layer_norm_rows(
+      [&](int pos) -> const float* {
+        const int k = k0 + pos;
+        return k < N ? p.z + b * p.zv.stride_b + r * p.zv.stride_r + k * p.zv.stride_k : nullptr;
+      },
+      p.ln_in_w, p.ln_in_b, C, xn);
+  if (threadIdx.x < kP) {
+    const int k = k0 + threadIdx.x;
+    msk[threadIdx.x] = (k < N && p.mask) ? p.mask[b * p.mv.stride_b + r * p.mv.stride_r + k * p.mv.stride_k] : 1.f;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * CH; idx += kThreads) {
+    const int pos = idx % kP, c = idx / kP, k = k0 + pos;
+    if (k >= N) continue;
+    const float m = msk[pos];
+    // a = mask * sigmoid(gate) * projection, in the reference's order of multiplication
+    const float av = m * sigmoid_f32(dot_row(xn[pos], p.w_ag + c * C, C)) * dot_row(xn[pos], p.w_ap + c * C, C);
+    const float bv = m * sigmoid_f32(dot_row(xn[pos], p.w_bg + c * C, C)) * dot_row(xn[pos], p.w_bp + c * C, C);
+    const size_t o = (((size_t)b * CH + c) * N + r) * N + k;
+    p.a[o] = av;
+    p.b[o] = bv;
+  }
+}
+
+// x[p][i][j] = sum_k a[p][i][k] * b[p][j][k]: 64 x 64 tile, 4 x 4 outputs per thread
+__global__ __launch_bounds__(kThreads) void trimul_contract_f32(const float* __restrict__ a, const float* __restrict__ b,
+                                                               float* __restrict__ x, int N) {
+  constexpr int T = 64, BK = 16;
+  __shared__ float as[BK][T + 4], bs[BK][T + 4];
+  const size_t plane = (size_t)blockIdx.z * N * N;
+  const int i0 = blockIdx.y * T, j0 = blockIdx.x * T;
+  const int ty = threadIdx.x / 16, tx = threadIdx.x % 16;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < N; k0 += BK) {
+    for (int e = threadIdx.x; e < T * BK; e += kThreads) {
+      const int row = e / BK, kk = e % BK;
+      const bool kin = k0 + kk < N;
+      as[kk][row] = (kin && i0 + row < N) ? a[plane + (size_t)(i0 + row) * N + k0 + kk] : 0.f;
+      bs[kk][row] = (kin && j0 + row < N) ? b[plane + (size_t)(j0 + row) * N + k0 + kk] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        av[u] = as[kk][ty * 4 + u];
+        bv[u] = bs[kk][tx * 4 + u];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[u][v] = fmaf(av[u], bv[v], acc[u][v]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int i = i0 + ty * 4 + u, j = j0 + tx * 4 + v;
+      if (i < N && j < N) x[plane + (size_t)i * N + j] = acc[u][v];
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void trimul_out_f32(TrimulF32 p, int groups) {
+  __shared__ float zn[kP][kMaxC];
+  __shared__ float xs[kP][kMaxC];
+  __shared__ float xo[kP][kMaxC];
+  const int N = p.N, C = p.C, CH = p.CH;
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kP;
+  auto zrow = [&](int pos) -> const float* {
+    const int j = j0 + pos;
+    return j < N ? p.z + b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k : nullptr;
+  };
+  layer_norm_rows(zrow, p.ln_in_w, p.ln_in_b, C, zn);
+  for (int idx = threadIdx.x; idx < kP * CH; idx += kThreads) {
+    const int pos = idx % kP, c = idx / kP, j = j0 + pos;
+    xs[pos][c] = j < N ? p.x[(((size_t)b * CH + c) * N + i) * N + j] : 0.f;
+  }
+  __syncthreads();
+  layer_norm_rows([&](int pos) -> const float* { return j0 + pos < N ? xs[pos] : nullptr; }, p.ln_out_w, p.ln_out_b,
+                  CH, xo);
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * C; idx += kThreads) {
+    const int pos = idx / C, co = idx % C, j = j0 + pos;
+    if (j >= N) continue;
+    float res = dot_row(xo[pos], p.w_z + co * CH, CH) * sigmoid_f32(dot_row(zn[pos], p.w_g + co * C, C));
+    const size_t o = b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k + co;
+    if (p.add_residual) res = p.z[o] + res;
+    p.out[o] = res;
+  }
+}
+
+// ---- triangle attention ----------------------------------------------------------------------
+struct TriattnF32 {
+  const float *x, *mask;
+  PairView xv, mv;
+  const float *ln_w, *ln_b, *w_q, *w_k, *w_v, *w_b, *w_g, *w_o;
+  float *q, *k, *v, *tb, *o, *out;
+  int B, N, C, H, D, add_residual;
+  float inf;
+};
+
+__global__ __launch_bounds__(kThreads) void triattn_proj_f32(TriattnF32 p, int groups) {
+  __shared__ float xn[kP][kMaxC];
+  const int N = p.N, C = p.C, H = p.H, D = p.D, HD = H * D;
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kP;
+  layer_norm_rows(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+      },
+      p.ln_w, p.ln_b, C, xn);
+  __syncthreads();
+  const float scale = 1.0f / sqrtf((float)D);
+  for (int idx = threadIdx.x; idx < kP * (3 * HD + H); idx += kThreads) {
+    const int pos = idx % kP, ch = idx / kP, j = j0 + pos;
+    if (j >= N) continue;
+    if (ch < 3 * HD) {
+      const int which = ch / HD, hd = ch % HD, h = hd / D, d = hd % D;
+      const float* w = (which == 0 ? p.w_q : which == 1 ? p.w_k : p.w_v) + hd * C;
+      float val = dot_row(xn[pos], w, C);
+      if (which == 0) val = val * scale;  // q / sqrt(c) after the projection (attention.py:283-284)
+      float* dst = which == 0 ? p.q : which == 1 ? p.k : p.v;
+      dst[((((size_t)b * N + i) * H + h) * N + j) * D + d] = val;
+    } else {
+      const int h = ch - 3 * HD;
+      p.tb[(((size_t)b * H + h) * N + i) * N + j] = dot_row(xn[pos], p.w_b + h * C, C);
+    }
+  }
+}
+
+// one thread per query of one (b, i, h); keys in chunks of 32 through LDS; online softmax
+template <int D>
+__global__ __launch_bounds__(128) void triattn_core_f32(TriattnF32 p, int qgroups) {
+  constexpr int KC = 32;
+  __shared__ float ks[KC][D], vs[KC][D], mbs[KC];
+  const int N = p.N, H = p.H;
+  const int qg = blockIdx.x % qgroups, h = (blockIdx.x / qgroups) % H, i = (blockIdx.x / (qgroups * H)) % N,
+            b = blockIdx.x / (qgroups * H * N);
+  const int qi = qg * 128 + threadIdx.x;
+  const bool active = qi < N;
+  const size_t bih = (((size_t)b * N + i) * H + h) * N;
+  float qv[D], ov[D];
+#pragma unroll
+  for (int d = 0; d < D; ++d) {
+    qv[d] = active ? p.q[(bih + qi) * D + d] : 0.f;
+    ov[d] = 0.f;
+  }
+  const float* tbrow = p.tb + (((size_t)b * H + h) * N + (active ? qi : 0)) * N;
+  float m = -__builtin_inff(), l = 0.f;
+  for (int k0 = 0; k0 < N; k0 += KC) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < KC * D; e += 128) {
+      const int kk = e / D, d = e % D;
+      const bool in = k0 + kk < N;
+      ks[kk][d] = in ? p.k[(bih + k0 + kk) * D + d] : 0.f;
+      vs[kk][d] = in ? p.v[(bih + k0 + kk) * D + d] : 0.f;
+    }
+    if (threadIdx.x < KC) {
+      const int kx = k0 + threadIdx.x;
+      float mv = 1.f;
+      if (kx < N && p.mask) mv = p.mask[b * p.mv.stride_b + i * p.mv.stride_r + kx * p.mv.stride_k];
+      mbs[threadIdx.x] = p.inf * (mv - 1.f);
+    }
+    __syncthreads();
+    const int kn = N - k0 < KC ? N - k0 : KC;
+    float s[KC];
+    float cmax = -__builtin_inff();
+#pragma unroll
+    for (int kk = 0; kk < KC; ++kk) {
+      float acc = 0.f;
+#pragma unroll
+      for (int d = 0; d < D; ++d) acc = fmaf(qv[d], ks[kk][d], acc);
+      // logits in the reference's order: q.k, then the mask bias, then the triangle bias
+      acc = acc + mbs[kk];
+      acc = acc + (kk < kn ? tbrow[k0 + kk] : 0.f);
+      s[kk] = kk < kn ? acc : -__builtin_inff();
+      cmax = fmaxf(cmax, s[kk]);
+    }
+    const float m_new = fmaxf(m, cmax);
+    const float alpha = expf(m - m_new);
+    l *= alpha;
+#pragma unroll
+    for (int d = 0; d < D; ++d) ov[d] *= alpha;
+#pragma unroll
+    for (int kk = 0; kk < KC; ++kk) {
+      const float pw = expf(s[kk] - m_new);
+      l += pw;
+#pragma unroll
+      for (int d = 0; d < D; ++d) ov[d] = fmaf(pw, vs[kk][d], ov[d]);
+    }
+    m = m_new;
+  }
+  if (active) {
+    const float inv = 1.0f / l;
+    float* dst = p.o + ((((size_t)b * N + i) * N + qi) * H + h) * D;
+#pragma unroll
+    for (int d = 0; d < D; ++d) dst[d] = ov[d] * inv;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void triattn_out_f32(TriattnF32 p, int groups) {
+  __shared__ float xn[kP][kMaxC];
+  __shared__ float og[kP][kMaxC];
+  const int N = p.N, C = p.C, HD = p.H * p.D;
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kP;
+  layer_norm_rows(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+      },
+      p.ln_w, p.ln_b, C, xn);
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * HD; idx += kThreads) {
+    const int pos = idx / HD, hd = idx % HD, j = j0 + pos;
+    og[pos][hd] = j < N ? p.o[(((size_t)b * N + i) * N + j) * HD + hd] * sigmoid_f32(dot_row(xn[pos], p.w_g + hd * C, C))
+                        : 0.f;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * C; idx += kThreads) {
+    const int pos = idx / C, co = idx % C, j = j0 + pos;
+    if (j >= N) continue;
+    float res = dot_row(og[pos], p.w_o + co * HD, HD);
+    const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
+    if (p.add_residual) res = p.x[o] + res;
+    p.out[o] = res;
+  }
+}
+
+}  // namespace
+
+hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
+  TrimulF32 p;
+  p.z = a.z;
+  p.mask = a.mask;
+  p.zv = a.z_view;
+  p.mv = a.mask_view;
+  p.zc = a.z_canonical;
+  p.ln_in_w = a.ln_in_w;
+  p.ln_in_b = a.ln_in_b;
+  p.ln_out_w = a.ln_out_w;
+  p.ln_out_b = a.ln_out_b;
+  p.w_ap = a.w_ap;
+  p.w_ag = a.w_ag;
+  p.w_bp = a.w_bp;
+  p.w_bg = a.w_bg;
+  p.w_g = a.w_g;
+  p.w_z = a.w_z;
+  p.a = a.a;
+  p.b = a.b;
+  p.x = a.x;
+  p.out = a.out;
+  p.B = a.B;
+  p.N = a.N;
+  p.C = a.C;
+  p.CH = a.CH;
+  p.add_residual = a.add_residual;
+  const int groups = (a.N + kP - 1) / kP;
+  const long blocks = (long)a.B * a.N * groups;
+  if (a.C > kMaxC || a.CH > kMaxC || blocks > 0x7fffffffL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(trimul_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  const unsigned t = (unsigned)((a.N + 63) / 64);
+  hipLaunchKernelGGL(trimul_contract_f32, dim3(t, t, (unsigned)(a.B * a.CH)), dim3(kThreads), 0, stream, p.a, p.b, p.x,
+                     a.N);
+  hipLaunchKernelGGL(trimul_out_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  return hipGetLastError();
+}
+
+hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
+  TriattnF32 p;
+  p.x = a.x;
+  p.mask = a.mask;
+  p.xv = a.x_view;
+  p.mv = a.mask_view;
+  p.ln_w = a.ln_w;
+  p.ln_b = a.ln_b;
+  p.w_q = a.w_q;
+  p.w_k = a.w_k;
+  p.w_v = a.w_v;
+  p.w_b = a.w_b;
+  p.w_g = a.w_g;
+  p.w_o = a.w_o;
+  p.q = a.q;
+  p.k = a.k;
+  p.v = a.v;
+  p.tb = a.tb;
+  p.o = a.o;
+  p.out = a.out;
+  p.B = a.B;
+  p.N = a.N;
+  p.C = a.C;
+  p.H = a.H;
+  p.D = a.D;
+  p.add_residual = a.add_residual;
+  p.inf = a.inf;
+  const int groups = (a.N + kP - 1) / kP;
+  const long blocks = (long)a.B * a.N * groups;
+  const int qgroups = (a.N + 127) / 128;
+  const long cblocks = (long)a.B * a.N * a.H * qgroups;
+  if (a.C > kMaxC || a.H * a.D > kMaxC || blocks > 0x7fffffffL || cblocks > 0x7fffffffL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(triattn_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  if (a.D == 32)
+    hipLaunchKernelGGL(triattn_core_f32<32>, dim3((unsigned)cblocks), dim3(128), 0, stream, p, qgroups);
+  else if (a.D == 16)
+    hipLaunchKernelGGL(triattn_core_f32<16>, dim3((unsigned)cblocks), dim3(128), 0, stream, p, qgroups);
+  else if (a.D == 64)
+    hipLaunchKernelGGL(triattn_core_f32<64>, dim3((unsigned)cblocks), dim3(128), 0, stream, p, qgroups);
+  else
+    return hipErrorInvalidValue;
+  hipLaunchKernelGGL(triattn_out_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  return hipGetLastError();
+}
+
+}  // namespace of3

@@ -26,6 +26,7 @@ SOURCES = [
     "triattn_proj.hip",
     "triattn_flash.hip",
     "triattn_out.hip",
+    "pair_f32.hip",
 ]
 
 # packed fp32 VALU ops are disabled on purpose (device code only)

@@ -3,8 +3,10 @@ for alternative kernels (_cueq_triangle_mult, tmu.py:689-741; Attention's kernel
 attention.py:366-413), here with a single implementation and no dispatch.
 
 All functions run on the current CUDA(HIP) stream of the tensors' device, are forward-only
-and accept bf16 pair tensors shaped [*, N, N, C] (any number of leading batch dimensions, a
-transposed view in the two N dimensions is fine and is not copied).
+and accept bf16 or fp32 pair tensors shaped [*, N, N, C] (any number of leading batch
+dimensions, a transposed view in the two N dimensions is fine and is not copied).  bf16 runs
+the MFMA kernels; fp32 (the reference's default inference precision) runs the library's plain
+fp32 kernels; parameters are converted to the tensor's dtype.
 """
 from __future__ import annotations
 
@@ -32,11 +34,15 @@ def release_workspaces():
     _workspaces.clear()
 
 
-def _require_gpu_bf16(t: torch.Tensor, name: str):
+def _require_gpu(t: torch.Tensor, name: str) -> int:
+    """Returns the library's dtype code of t."""
     if not t.is_cuda:
         raise RuntimeError("%s must live on the GPU: the pair-stack kernels have no CPU path" % name)
-    if t.dtype != torch.bfloat16:
-        raise ValueError("%s must be bfloat16 (got %s): only the bf16 kernels are built" % (name, t.dtype))
+    if t.dtype == torch.bfloat16:
+        return _lib.OF3_DTYPE_BF16
+    if t.dtype == torch.float32:
+        return _lib.OF3_DTYPE_F32
+    raise ValueError("%s must be bfloat16 or float32 (got %s)" % (name, t.dtype))
 
 
 def _flatten_pair(z: torch.Tensor):
@@ -59,7 +65,7 @@ def _flatten_pair(z: torch.Tensor):
             z4 = z.view(-1, n1, n2, c)
         except RuntimeError:
             z4 = z.reshape(-1, n1, n2, c)
-    if any(s % 8 for s in z4.stride()[:3]) or z4.data_ptr() % 16:
+    if z.dtype == torch.bfloat16 and (any(s % 8 for s in z4.stride()[:3]) or z4.data_ptr() % 16):
         z4 = z4.contiguous()
     return z4, lead
 
@@ -77,11 +83,11 @@ def _mask_arg(mask, lead, B, N, device):
     return m3, m3.data_ptr(), _lib.strides3(m3.stride())
 
 
-def _w(t: torch.Tensor) -> torch.Tensor:
-    """Parameter as a contiguous bf16 device tensor (what a module cast with
-    .to(torch.bfloat16) holds; fp32 parameters are rounded once per call)."""
-    if t.dtype != torch.bfloat16 or not t.is_contiguous():
-        t = t.detach().to(torch.bfloat16).contiguous()
+def _w(t: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """Parameter as a contiguous device tensor of the activations' dtype (what a module cast
+    with .to(dtype) already holds; otherwise converted once per call)."""
+    if t.dtype != dtype or not t.is_contiguous():
+        t = t.detach().to(dtype).contiguous()
     return t
 
 
@@ -107,15 +113,16 @@ def triangle_multiplicative_update(z, mask, norm_in_weight, norm_in_bias, norm_o
                                    outgoing: bool, add_residual: bool = False, inplace: bool = False):
     """Update of tmu.py:482-503, or z + update when add_residual.  With inplace the result
     overwrites z (the reference's inplace_safe contract, tmu.py:154-173)."""
-    _require_gpu_bf16(z, "z")
+    code = _require_gpu(z, "z")
     lib = _lib.load()
     z4, lead = _flatten_pair(z)
     B, N, _, C = z4.shape
     CH = a_p_weight.shape[0]
-    nbytes = lib.of3_trimul_workspace_bytes(B, N, C, CH)
+    nbytes = lib.of3_trimul_workspace_bytes_for(code, B, N, C, CH)
     if nbytes < 0:
-        raise ValueError("triangle multiplication supports (c_z, c_hidden) = (128,128) or (64,64); got (%d,%d)" % (C, CH))
-    keep = [_w(t) for t in (norm_in_weight, norm_in_bias, norm_out_weight, norm_out_bias, a_p_weight, a_g_weight,
+        raise ValueError("triangle multiplication: bf16 supports (c_z, c_hidden) = (128,128) or (64,64), fp32 any "
+                         "widths up to 256; got (%d,%d) in %s" % (C, CH, z.dtype))
+    keep = [_w(t, z.dtype) for t in (norm_in_weight, norm_in_bias, norm_out_weight, norm_out_bias, a_p_weight, a_g_weight,
                             b_p_weight, b_g_weight, g_out_weight, p_out_weight)]
     m3, mptr, mstr = _mask_arg(mask, lead, B, N, z.device)
     out4 = z4 if inplace else _out_like(z4)
@@ -123,7 +130,7 @@ def triangle_multiplicative_update(z, mask, norm_in_weight, norm_in_bias, norm_o
     with torch.cuda.device(z.device):
         st = lib.of3_trimul_fwd(z4.data_ptr(), _lib.strides3(z4.stride()[:3]), mptr, mstr, *[k.data_ptr() for k in keep],
                                 out4.data_ptr(), B, N, C, CH, int(bool(outgoing)), int(bool(add_residual)),
-                                ws.data_ptr(), ws.numel(), _lib.OF3_DTYPE_BF16, _stream(z))
+                                ws.data_ptr(), ws.numel(), code, _stream(z))
     _lib.check(st, "of3_trimul_fwd")
     return _finish(z, z4, out4, lead, inplace)
 
@@ -133,23 +140,23 @@ def triangle_attention(x, mask, norm_weight, norm_bias, bias_weight, q_weight, k
                        inplace: bool = False):
     """Update of tri_att.py:102-167 for a starting-node module; hand in the transposed view
     for the ending node (base_blocks.py:380-404 does exactly that)."""
-    _require_gpu_bf16(x, "x")
+    code = _require_gpu(x, "x")
     lib = _lib.load()
     x4, lead = _flatten_pair(x)
     B, N, _, C = x4.shape
     H = int(no_heads)
     D = q_weight.shape[0] // H
-    nbytes = lib.of3_triattn_workspace_bytes(B, N, C, H, D)
+    nbytes = lib.of3_triattn_workspace_bytes_for(code, B, N, C, H, D)
     if nbytes < 0:
-        raise ValueError("triangle attention supports 4 heads with (c_in, c_head) = (128,32) or (64,16); "
-                         "got c_in=%d heads=%d c_head=%d" % (C, H, D))
-    keep = [_w(t) for t in (norm_weight, norm_bias, bias_weight, q_weight, k_weight, v_weight, g_weight, o_weight)]
+        raise ValueError("triangle attention: bf16 supports 4 heads with (c_in, c_head) = (128,32) or (64,16), fp32 "
+                         "head widths 16/32/64; got c_in=%d heads=%d c_head=%d in %s" % (C, H, D, x.dtype))
+    keep = [_w(t, x.dtype) for t in (norm_weight, norm_bias, bias_weight, q_weight, k_weight, v_weight, g_weight, o_weight)]
     m3, mptr, mstr = _mask_arg(mask, lead, B, N, x.device)
     out4 = x4 if inplace else _out_like(x4)
     ws = _workspace(x.device, nbytes)
     with torch.cuda.device(x.device):
         st = lib.of3_triattn_fwd(x4.data_ptr(), _lib.strides3(x4.stride()[:3]), mptr, mstr,
                                  *[k.data_ptr() for k in keep], out4.data_ptr(), B, N, C, H, D, float(inf),
-                                 int(bool(add_residual)), ws.data_ptr(), ws.numel(), _lib.OF3_DTYPE_BF16, _stream(x))
+                                 int(bool(add_residual)), ws.data_ptr(), ws.numel(), code, _stream(x))
     _lib.check(st, "of3_triattn_fwd")
     return _finish(x, x4, out4, lead, inplace)

@@ -32,7 +32,8 @@ def test_header_declares_expected_entry_points():
     for required in ("of3_trimul_fwd", "of3_trimul_proj", "of3_trimul_contract", "of3_trimul_out",
                      "of3_triattn_fwd", "of3_triattn_proj", "of3_triattn_flash", "of3_triattn_out",
                      "of3_version", "of3_last_hip_error", "of3_status_string", "of3_padded_n",
-                     "of3_trimul_workspace_bytes", "of3_triattn_workspace_bytes"):
+                     "of3_trimul_workspace_bytes", "of3_triattn_workspace_bytes",
+                     "of3_trimul_workspace_bytes_for", "of3_triattn_workspace_bytes_for"):
         assert required in names
 
 
@@ -93,7 +94,13 @@ def test_trimul_fwd_rejects_bad_arguments(lib):
     def call(z=FAKE, strides=zs, B=1, N=64, C=128, CH=128, ws=FAKE, ws_bytes=ws_need, dtype=_lib.OF3_DTYPE_BF16):
         return lib.of3_trimul_fwd(z, strides, None, None, *ptrs, FAKE, B, N, C, CH, 1, 0, ws, ws_bytes, dtype, None)
 
-    assert call(dtype=_lib.OF3_DTYPE_F32) == _lib.OF3_EINVAL      # only bf16 kernels exist
+    assert call(dtype=7) == _lib.OF3_EINVAL                        # unknown dtype code
+    # fp32 has its own (larger) workspace and looser shape rules; never call it with a workable argument set here
+    need32 = lib.of3_trimul_workspace_bytes_for(_lib.OF3_DTYPE_F32, 1, 64, 128, 128)
+    assert need32 == 3 * 128 * 64 * 64 * 4
+    assert call(dtype=_lib.OF3_DTYPE_F32, ws_bytes=need32 - 1) == _lib.OF3_ENOSPC
+    assert call(dtype=_lib.OF3_DTYPE_F32, C=300, CH=300) == _lib.OF3_EINVAL
+    assert call(dtype=_lib.OF3_DTYPE_F32, z=FAKE + 2, ws_bytes=need32) == _lib.OF3_EINVAL
     assert call(C=96, CH=96) == _lib.OF3_EINVAL                   # unsupported channel count
     assert call(N=0) == _lib.OF3_EINVAL
     assert call(ws=None) == _lib.OF3_EINVAL                        # null workspace
@@ -114,7 +121,11 @@ def test_triattn_fwd_rejects_bad_arguments(lib):
     def call(x=FAKE, B=1, N=64, C=128, H=4, D=32, ws=FAKE, ws_bytes=ws_need, dtype=_lib.OF3_DTYPE_BF16):
         return lib.of3_triattn_fwd(x, xs, None, None, *ptrs, FAKE, B, N, C, H, D, 1e9, 0, ws, ws_bytes, dtype, None)
 
-    assert call(dtype=_lib.OF3_DTYPE_F32) == _lib.OF3_EINVAL
+    assert call(dtype=7) == _lib.OF3_EINVAL
+    need32 = lib.of3_triattn_workspace_bytes_for(_lib.OF3_DTYPE_F32, 1, 64, 128, 4, 32)
+    assert need32 == 4 * 64 * 64 * 128 * 4 + 4 * 64 * 64 * 4
+    assert call(dtype=_lib.OF3_DTYPE_F32, ws_bytes=need32 - 1) == _lib.OF3_ENOSPC
+    assert call(dtype=_lib.OF3_DTYPE_F32, D=24, ws_bytes=need32) == _lib.OF3_EINVAL
     assert call(H=8) == _lib.OF3_EINVAL
     assert call(D=64) == _lib.OF3_EINVAL
     assert call(ws_bytes=ws_need - 1) == _lib.OF3_ENOSPC

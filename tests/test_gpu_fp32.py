@@ -1,0 +1,89 @@
+"""fp32 parity: the library's fp32 kernels against the fp32 CPU oracle on the same inputs.
+
+Tolerance (north star, fp32): max-abs error <= 1e-4.  Inputs are N(0,1), weights N(0, 1/fan_in)
+and LayerNorm affine near identity, so outputs are O(1) and an absolute bound is meaningful;
+BASELINE config 1 (N=64, c_z=128, 4 heads x 32, all-ones mask) is the first case."""
+import pytest
+import torch
+
+from gpu_util import lib  # noqa: F401
+from oracle import pairstack_oracle as orc
+
+import of3pair
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+FP32_TOL = 1e-4
+
+
+def _maxerr(name, got, want):
+    err = float((got.float().cpu() - want).abs().max())
+    print("%s: max|err| = %.3g (max|want| = %.3g)" % (name, err, float(want.abs().max())), flush=True)
+    assert err <= FP32_TOL, "%s: %.3g" % (name, err)
+
+
+def _load(module, params):
+    module.load_state_dict(params, strict=True)
+    return module.to(DEV).eval()
+
+
+@pytest.mark.parametrize("outgoing", [True, False])
+@pytest.mark.parametrize("c,ch,n,batch,masked", [(128, 128, 64, (1,), False), (64, 64, 45, (2,), True), (96, 40, 33, (), True)])
+def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
+    lib()
+    gen = torch.Generator().manual_seed(300 + n)
+    p = orc.make_trimul_params(gen, c, ch)
+    z = torch.randn(*batch, n, n, c, generator=gen)
+    mask = (torch.rand(*batch, n, n, generator=gen) > 0.2).float() if masked else None
+    cls = of3pair.TriangleMultiplicationOutgoing if outgoing else of3pair.TriangleMultiplicationIncoming
+    m = _load(cls(c, ch), p)
+    got = m(z.to(DEV), mask=None if mask is None else mask.to(DEV))
+    assert got.dtype == torch.float32
+    _maxerr("trimul fp32", got, orc.trimul_update(z, mask, p, outgoing))
+
+
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("c,d,heads,n,batch,masked", [(128, 32, 4, 64, (1,), False), (64, 16, 4, 45, (2,), True),
+                                                     (48, 64, 2, 37, (), True)])
+def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
+    lib()
+    gen = torch.Generator().manual_seed(400 + n)
+    p = orc.make_triattn_params(gen, c, d, heads)
+    x = torch.randn(*batch, n, n, c, generator=gen)
+    mask = None
+    if masked:
+        mask = (torch.rand(*batch, n, n, generator=gen) > 0.2).float()
+        mask[..., 3, :] = 0.0   # a fully masked row (starting frame) and column (ending frame)
+        mask[..., :, 5] = 0.0
+    m = _load(of3pair.TriangleAttention(c, d, heads, starting=starting), p)
+    got = m(x.to(DEV), mask=None if mask is None else mask.to(DEV))
+    _maxerr("triattn fp32", got, orc.triattn_update(x, mask, p, heads, starting=starting))
+
+
+def test_block_config1_fp32():
+    """BASELINE config 1: B=1, N=64, c_z=128, c_hidden_mul=128, 4 heads x 32, all-ones mask, fp32."""
+    lib()
+    n, c, d, heads = 64, 128, 32, 4
+    p = orc.make_block_params(0, c, c, d, heads)
+    m = _load(of3pair.PairStack(c, c, d, heads), p)
+    z = orc.make_pair_input(1, (1,), n, c)
+    mask = torch.ones(1, n, n)
+    zg = z.to(DEV)
+    got = m(zg, mask.to(DEV))
+    assert torch.equal(zg.cpu(), z)
+    want = orc.pair_stack_block(z, mask, p, heads)
+    _maxerr("block config 1 fp32", got, want)
+    got2 = m(zg, mask.to(DEV), inplace_safe=True)   # in place: same result, z overwritten
+    assert got2.data_ptr() == zg.data_ptr()
+    _maxerr("block config 1 fp32 in place", got2, want)
+
+
+def test_block_fp32_padded():
+    lib()
+    n, c, d, heads = 80, 64, 16, 4
+    p = orc.make_block_params(3, c, c, d, heads)
+    m = _load(of3pair.PairStack(c, c, d, heads), p)
+    z = orc.make_pair_input(4, (2,), n, c)
+    mask = orc.tail_padding_mask((2,), n, torch.tensor([9, 0]))
+    got = m(z.to(DEV), mask.to(DEV))
+    _maxerr("block fp32 padded", got, orc.pair_stack_block(z, mask, p, heads))

@@ -87,6 +87,8 @@ def test_no_cpu_fallback():
     a = of3pair.TriangleAttention(128, 32, 4).to(torch.bfloat16)
     with pytest.raises(RuntimeError, match="GPU"):
         a(z)
+    with pytest.raises(RuntimeError, match="GPU"):  # fp32 has no CPU path either
+        of3pair.TriangleMultiplicationOutgoing(128, 128)(z.float())
 
 
 def test_package_does_not_import_the_oracle():
