@@ -135,7 +135,7 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
 
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream) {
-  if (B < 1 || N < 1 || (CH != 128 && CH != 64) || variant < 0 || variant > 3) return OF3_EINVAL;
+  if (B < 1 || N < 1 || (CH != 128 && CH != 64) || variant < 0 || variant > 6) return OF3_EINVAL;
   if (!a || !b || !x || !aligned16(a) || !aligned16(b) || !aligned16(x)) return OF3_EINVAL;
   const int64_t Np = padded(N);
   if (variant == 0) variant = contract_variant_auto(Np);

@@ -30,6 +30,7 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int 
 
   __shared__ u32x4_t xtile[TP * NCH];  // LayerNorm(x), bf16
   __shared__ u32x4_t otile[TP * NCH];  // o, then o * gate
+  __shared__ u32x4_t rtile[TP * NCH];  // x as loaded: the residual of the output phase
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -55,17 +56,16 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int 
   const int N = p.N;
   const int tiles_per_batch = N * tiles_per_row;
 
-  for (int tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+  // The loads of a tile are issued one tile ahead (right after the previous tile's values have
+  // been consumed by the LayerNorm phase) and travel under that tile's two MFMA phases.
+  u32x4_t xraw[LN_ITERS], oraw[LN_ITERS];
+  auto load_tile = [&](int tile_id) {
     const int b = tile_id / tiles_per_batch;
     const int rem = tile_id - b * tiles_per_batch;
     const int i = rem / tiles_per_row;
     const int j0 = (rem - i * tiles_per_row) * TP;
     const bf16_t* xrow = p.x + b * p.x_view.stride_b + i * p.x_view.stride_r;
-    bf16_t* outrow = p.out + b * p.x_view.stride_b + i * p.x_view.stride_r;
     const bf16_t* orow = p.o + ((size_t)b * N + i) * N * HD;
-
-    // ---- loads + LayerNorm
-    u32x4_t xraw[LN_ITERS], oraw[LN_ITERS];
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
       const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
@@ -77,14 +77,27 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int 
       xraw[it] = vx;
       oraw[it] = vo;
     }
+  };
+  if ((int)blockIdx.x < total_tiles) load_tile(blockIdx.x);
+
+  for (int tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+    const int b = tile_id / tiles_per_batch;
+    const int rem = tile_id - b * tiles_per_batch;
+    const int i = rem / tiles_per_row;
+    const int j0 = (rem - i * tiles_per_row) * TP;
+    bf16_t* outrow = p.out + b * p.x_view.stride_b + i * p.x_view.stride_r;
+
+    // ---- LayerNorm of this tile's values, then the next tile's loads
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
       const int pos = wave * (TP / NW) + it * PPI + ln_pp;
       const int slot = tile_slot<NCH, 0>(pos, ln_chunk);
       xtile[slot] = layer_norm_chunk<C>(xraw[it], lw, lb);
+      rtile[slot] = xraw[it];
       otile[slot] = oraw[it];
     }
     __syncthreads();
+    if (tile_id + (int)gridDim.x < total_tiles) load_tile(tile_id + gridDim.x);
 
     // ---- gate: lane owns gate channels 32*ot + 16*lh + v of position 32*t + l32
 #pragma unroll
@@ -119,8 +132,8 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int 
 #pragma unroll
         for (int v = 0; v < 16; ++v) res[v] = acc[v];
         if (p.add_residual) {
-          const u32x4_t r0 = *reinterpret_cast<const u32x4_t*>(xrow + off);
-          const u32x4_t r1 = *reinterpret_cast<const u32x4_t*>(xrow + off + 8);
+          const u32x4_t r0 = rtile[tile_slot<NCH, 0>(pos, 4 * ot + 2 * lh)];
+          const u32x4_t r1 = rtile[tile_slot<NCH, 0>(pos, 4 * ot + 2 * lh + 1)];
           float xr[8];
           unpack8(r0, xr);
 #pragma unroll

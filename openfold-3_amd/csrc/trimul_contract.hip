@@ -42,7 +42,6 @@ namespace {
 #define OF3_LDS_AS __attribute__((address_space(3)))
 
 constexpr int kBK = 32;  // k per stage = one k-panel
-constexpr int kNS = 4;   // ring depth
 
 // j side: rows are read in the permuted order {x..x+3, x+64..x+67, x+4..}: (row&1, key)
 // must differ within each group of 8 and (row&3, key) within each group of 16 lanes
@@ -59,7 +58,7 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | 0x70 | 0xF00 | ((N >> 4) << 14));
 }
 
-template <int BN>
+template <int BN, int kNS>
 __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restrict__ pm,  // j side planes (b)
                                                           const bf16_t* __restrict__ pn,  // i side planes (a)
                                                           bf16_t* __restrict__ x, int Np, int tiles_m, int tiles_n,
@@ -75,7 +74,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
   constexpr int IPW = MI + NI;
   constexpr int NMMA = TM * TN;
   static_assert(IPW <= NMMA, "a stage's loads are issued between the MFMAs of one k-step");
-  static_assert(2 * IPW + 8 * TN < 64, "vmcnt budget");
+  static_assert((kNS - 2) * IPW + 8 * TN < 64, "vmcnt budget");
 
   extern __shared__ u32x4_t lds[];
 
@@ -148,7 +147,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
     }
   };
   auto issue_advance = [&]() {
-    issue_buf = (issue_buf + 1) & (kNS - 1);
+    issue_buf = issue_buf + 1 == kNS ? 0 : issue_buf + 1;
     issue_kb = issue_kb + 1 == nk ? 0 : issue_kb + 1;
     if (--issue_left == 0) dma_setup_tile(++issue_tile);
   };
@@ -208,7 +207,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
     for (int n = 0; n < IPW; ++n) issue_one(n);
     issue_advance();
   }
-  wait_vmcnt<3 * IPW>();
+  wait_vmcnt<(kNS - 1) * IPW>();
   compiler_fence();
   __builtin_amdgcn_s_barrier();
   compiler_fence();
@@ -233,8 +232,8 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
       // simply allowed to stay outstanding, otherwise the wait would drain the whole ring
       // at every tile boundary.
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): a1/b1 have arrived
-      if (stores_pending && kb < 3) wait_vmcnt<2 * IPW + 8 * TN>();
-      else wait_vmcnt<2 * IPW>();
+      if (stores_pending && kb < kNS - 1) wait_vmcnt<(kNS - 2) * IPW + 8 * TN>();
+      else wait_vmcnt<(kNS - 2) * IPW>();
       compiler_fence();
       __builtin_amdgcn_s_barrier();
       compiler_fence();
@@ -242,7 +241,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
 
       // after the barrier no wave reads the buffer of stage s any more: refill it with
       // stage s+4 while the second k-step's MFMAs run
-      cur_buf = (cur_buf + 1) & (kNS - 1);
+      cur_buf = cur_buf + 1 == kNS ? 0 : cur_buf + 1;
       fetch(lds + cur_buf * STAGE, 0, a0, b0);  // after the last stage this reads data that is never used
       mma_and_issue(a1, b1);
       __builtin_amdgcn_sched_barrier(0);
@@ -293,10 +292,10 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
   wait_vmcnt<0>();  // loads issued past the end must not outlive the work-group's LDS
 }
 
-template <int BN>
+template <int BN, int kNS>
 hipError_t launch_contract(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, hipStream_t stream) {
   constexpr int BM = 256;
-  auto kern = contract_kernel<BN>;
+  auto kern = contract_kernel<BN, kNS>;
   const size_t smem = ((size_t)kNS * (BM + BN) * 4 + 4 * 512) * sizeof(u32x4_t);  // ring + epilogue staging
   static int cus = 0;
   if (cus == 0) {
@@ -326,11 +325,17 @@ hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, i
                                   hipStream_t stream) {
   switch (variant) {
     case 1:
-      return launch_contract<192>(a, b, x, planes, Np, stream);
+      return launch_contract<192, 4>(a, b, x, planes, Np, stream);
     case 2:
-      return launch_contract<128>(a, b, x, planes, Np, stream);
+      return launch_contract<128, 4>(a, b, x, planes, Np, stream);
     case 3:
-      return launch_contract<256>(a, b, x, planes, Np, stream);
+      return launch_contract<256, 4>(a, b, x, planes, Np, stream);
+    case 4:
+      return launch_contract<128, 5>(a, b, x, planes, Np, stream);
+    case 5:
+      return launch_contract<128, 3>(a, b, x, planes, Np, stream);
+    case 6:
+      return launch_contract<192, 3>(a, b, x, planes, Np, stream);
     default:
       return hipErrorInvalidValue;
   }

@@ -31,6 +31,7 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
 
   __shared__ u32x4_t ztile[TP * NCH];
   __shared__ u32x4_t xtile[TP * NCH];
+  __shared__ u32x4_t rtile[TP * NCH];  // z as loaded: the residual of the output phase
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -61,16 +62,16 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
   const int tiles_per_batch = N * tiles_per_row;
   uint32_t* xt32 = reinterpret_cast<uint32_t*>(xtile);
 
-  for (int tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+  // The loads of a tile (z row-wise for the gate, x channel-major) are issued one tile ahead,
+  // right after the previous tile's values have gone into LDS, and travel under its MFMA phase.
+  u32x4_t zraw[LN_ITERS];
+  u32x4_t xa[XROUNDS], xb[XROUNDS];
+  auto load_tile = [&](int tile_id) {
     const int b = tile_id / tiles_per_batch;
     const int rem = tile_id - b * tiles_per_batch;
     const int i = rem / tiles_per_row;
     const int j0 = (rem - i * tiles_per_row) * TP;
     const bf16_t* zrow = p.z + b * p.z_view.stride_b + i * p.z_view.stride_r;
-    bf16_t* orow = p.out + b * p.z_view.stride_b + i * p.z_view.stride_r;
-
-    // ---- loads: z (row-wise, for the gate) and x (channel-major, transposed below)
-    u32x4_t zraw[LN_ITERS];
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
       const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
@@ -78,7 +79,6 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
       if (j < N) v = *reinterpret_cast<const u32x4_t*>(zrow + j * p.z_view.stride_k + 8 * ln_chunk);
       zraw[it] = v;
     }
-    u32x4_t xa[XROUNDS], xb[XROUNDS];
 #pragma unroll
     for (int rr = 0; rr < XROUNDS; ++rr) {
       const int item = rr * 512 + tid;
@@ -87,6 +87,15 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
       xa[rr] = *reinterpret_cast<const u32x4_t*>(src);
       xb[rr] = *reinterpret_cast<const u32x4_t*>(src + (size_t)Np * Np);
     }
+  };
+  if ((int)blockIdx.x < total_tiles) load_tile(blockIdx.x);
+
+  for (int tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
+    const int b = tile_id / tiles_per_batch;
+    const int rem = tile_id - b * tiles_per_batch;
+    const int i = rem / tiles_per_row;
+    const int j0 = (rem - i * tiles_per_row) * TP;
+    bf16_t* orow = p.out + b * p.z_view.stride_b + i * p.z_view.stride_r;
 
     // x: transpose into xtile[pos][c] with 4-byte (channel pair) writes
 #pragma unroll
@@ -107,8 +116,10 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
     for (int it = 0; it < LN_ITERS; ++it) {
       const int pos = wave * (TP / NW) + it * PPI + ln_pp;
       ztile[tile_slot<NCH, 0>(pos, ln_chunk)] = layer_norm_chunk<C>(zraw[it], iw, ib);
+      rtile[tile_slot<NCH, 0>(pos, ln_chunk)] = zraw[it];
     }
     __syncthreads();
+    if (tile_id + (int)gridDim.x < total_tiles) load_tile(tile_id + gridDim.x);
 
     // x: LayerNorm_out in place (lane owns one 16-byte chunk of one position)
 #pragma unroll
@@ -139,8 +150,8 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
 #pragma unroll
         for (int v = 0; v < 16; ++v) res[v] = accu[v] * sigmoidf_fast(accg[v]);
         if (p.add_residual) {
-          const u32x4_t r0 = *reinterpret_cast<const u32x4_t*>(zrow + off);
-          const u32x4_t r1 = *reinterpret_cast<const u32x4_t*>(zrow + off + 8);
+          const u32x4_t r0 = rtile[tile_slot<NCH, 0>(pos, 4 * ot + 2 * lh)];
+          const u32x4_t r1 = rtile[tile_slot<NCH, 0>(pos, 4 * ot + 2 * lh + 1)];
           float zr[8];
           unpack8(r0, zr);
 #pragma unroll

@@ -12,8 +12,9 @@
 // 128 positions is normalised in registers (statistics by DPP lane permutations), staged
 // once in LDS as bf16 and consumed as the MFMA B operand by all waves.  The LDS tile is
 // double buffered, which leaves a single barrier per tile.  Positions are dealt to MFMA
-// columns so that a lane finishes 4 consecutive positions of a channel and stores them as
-// one 8-byte vector (8 lanes fill one 64-byte panel row).
+// columns so that a lane finishes 4 consecutive k of one row and channel and stores them as
+// one 8-byte vector.  A tile is 4 consecutive rows r of one 32-wide k-panel: in the k-panel
+// layout these are 256 contiguous bytes per channel, so 32 lanes write whole 128-byte lines.
 #include "of3_device.h"
 #include "of3_kernels.h"
 
@@ -22,11 +23,12 @@ namespace of3 {
 namespace {
 
 template <int C, int CH>
-__global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int tiles_per_row, int total_tiles) {
+__global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int panels, int total_tiles) {
   constexpr int NCH = C / 8;        // 16-byte chunks per position
   constexpr int LPP = NCH;          // lanes sharing one position in the LayerNorm phase
   constexpr int PPI = 64 / LPP;     // positions per wave instruction
-  constexpr int TP = 128;           // positions per tile
+  constexpr int TP = 128;           // positions per tile: TR rows x one 32-wide k-panel
+  constexpr int TR = TP / 32;
   constexpr int NW = 8;             // waves per work-group (two per SIMD)
   constexpr int LN_ITERS = (TP / NW) / PPI;
   constexpr int KS = C / 16;        // MFMA k-steps
@@ -45,9 +47,10 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
   const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
   const int ln_chunk = lane % LPP, ln_pp = lane / LPP;
 
-  float lw[8], lb[8];
-  load_affine8(p.ln_w, ln_chunk, lw);
-  load_affine8(p.ln_b, ln_chunk, lb);
+  // LayerNorm affine parameters of this lane's 8 channels, kept packed (8 registers instead
+  // of 16) and unpacked once per tile
+  const u32x4_t lw_pk = *reinterpret_cast<const u32x4_t*>(p.ln_w + 8 * ln_chunk);
+  const u32x4_t lb_pk = *reinterpret_cast<const u32x4_t*>(p.ln_b + 8 * ln_chunk);
 
   // this wave's job: gate and projection rows 32*ot .. +31 of a (pair 0) or b (pair 1),
   // resident in registers as MFMA A operands for the whole kernel
@@ -67,20 +70,27 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
   bf16_t* const out = pair ? p.b : p.a;
 
   const int N = p.N, Np = p.Np;
-  const int tiles_per_batch = N * tiles_per_row;
+  const int tiles_per_batch = ((N + TR - 1) / TR) * panels;
 
+  // LayerNorm-phase positions of this lane: wave w takes positions [16w, 16w+16) of the tile,
+  // i.e. 16 consecutive k of row w/2; iteration `it` adds PPI positions.  The lane-dependent
+  // part of the address is computed once, the tile adds a wave-uniform base.
+  const int ln_pos0 = wave * (TP / NW) + ln_pp;
+  const int ln_row = ln_pos0 >> 5, ln_k = ln_pos0 & 31;
+  const int64_t ln_off = ln_row * p.z_view.stride_r + ln_k * p.z_view.stride_k + 8 * ln_chunk;
   u32x4_t raw[LN_ITERS];
   auto load_tile = [&](int tile_id) {
     const int b = tile_id / tiles_per_batch;
     const int rem = tile_id - b * tiles_per_batch;
-    const int r = rem / tiles_per_row;
-    const int k0 = (rem - r * tiles_per_row) * TP;
-    const bf16_t* zrow = p.z + b * p.z_view.stride_b + r * p.z_view.stride_r;
+    const int r0 = (rem / panels) * TR;
+    const int k0 = (rem % panels) * 32;
+    const bf16_t* base = p.z + b * p.z_view.stride_b + r0 * p.z_view.stride_r + k0 * p.z_view.stride_k;
+    const bool row_ok = r0 + ln_row < N;
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int k = k0 + wave * (TP / NW) + it * PPI + ln_pp;
       u32x4_t v = {0u, 0u, 0u, 0u};
-      if (k < N) v = *reinterpret_cast<const u32x4_t*>(zrow + k * p.z_view.stride_k + 8 * ln_chunk);
+      if (row_ok && k0 + ln_k + it * PPI < N)
+        v = *reinterpret_cast<const u32x4_t*>(base + ln_off + (it * PPI) * p.z_view.stride_k);
       raw[it] = v;
     }
   };
@@ -95,22 +105,28 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
   for (int buf = 0; tile_id < total_tiles; tile_id += gridDim.x, buf ^= 1) {
     const int b = tile_id / tiles_per_batch;
     const int rem = tile_id - b * tiles_per_batch;
-    const int r = rem / tiles_per_row;
-    const int k0 = (rem - r * tiles_per_row) * TP;
+    const int r = (rem / panels) * TR + (pos0 >> 5);  // this lane's row and first k
+    const int kfirst = (rem % panels) * 32 + (pos0 & 31);
 
     float mval[TPW];
+    const float* mrow = p.mask ? p.mask + b * p.mask_view.stride_b + r * p.mask_view.stride_r +
+                                     kfirst * p.mask_view.stride_k
+                               : nullptr;
 #pragma unroll
     for (int tt = 0; tt < TPW; ++tt) {
-      const int k = k0 + pos0 + tt;
       float m = 0.f;
-      if (k < N) {
-        m = 1.f;
-        if (p.mask) m = p.mask[b * p.mask_view.stride_b + r * p.mask_view.stride_r + k * p.mask_view.stride_k];
-      }
+      if (kfirst + tt < N && r < N) m = mrow ? mrow[tt * p.mask_view.stride_k] : 1.f;
       mval[tt] = m;
     }
 
     // ---- LayerNorm phase: wave w normalises positions [16w, 16w+16) of the tile
+    float lw[8], lb[8];
+    {
+      u32x4_t tw = lw_pk, tb = lb_pk;
+      __asm__ volatile("" : "+v"(tw), "+v"(tb));  // keeps the unpacked copies from being hoisted out of the loop
+      unpack8(tw, lw);
+      unpack8(tb, lb);
+    }
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
       const int pos = wave * (TP / NW) + it * PPI + ln_pp;
@@ -139,16 +155,21 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
     }
     // stores: register v of a lane is channel 32*ot + 8*(v/4) + 4*lh + v%4; k-panel layout
     // plane[k / 32][row][k % 32]
-    const int k = k0 + pos0;
+    if (r < N) {
+      // lane base: channel 32*ot + 4*lh of this batch element, row r, first k of the lane;
+      // the 16 registers add wave-uniform channel offsets
+      const size_t plane = (size_t)Np * Np;
+      bf16_t* dst0 = out + ((size_t)b * CH + 32 * ot + 4 * lh) * plane + (size_t)(kfirst >> 5) * (Np * 32) + r * 32 +
+                     (kfirst & 31);
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int ch = 32 * ot + 8 * (v >> 2) + 4 * lh + (v & 3);
-      bf16_t* dst = out + ((size_t)b * CH + ch) * Np * Np + (size_t)(k >> 5) * (Np * 32) + r * 32 + (k & 31);
-      if (TPW == 4) {
-        u32x2_t w2 = {pack_bf16(res[0][v], res[1][v]), pack_bf16(res[2][v], res[3][v])};
-        *reinterpret_cast<u32x2_t*>(dst) = w2;
-      } else {
-        *reinterpret_cast<uint32_t*>(dst) = pack_bf16(res[0][v], res[1][v]);
+      for (int v = 0; v < 16; ++v) {
+        bf16_t* dst = dst0 + (size_t)(8 * (v >> 2) + (v & 3)) * plane;
+        if (TPW == 4) {
+          u32x2_t w2 = {pack_bf16(res[0][v], res[1][v]), pack_bf16(res[2][v], res[3][v])};
+          *reinterpret_cast<u32x2_t*>(dst) = w2;
+        } else {
+          *reinterpret_cast<uint32_t*>(dst) = pack_bf16(res[0][v], res[1][v]);
+        }
       }
     }
   }
@@ -168,10 +189,10 @@ hipError_t launch(const TrimulProjArgs& a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     grid_cap = cus * (per_cu > 0 ? per_cu : 1);
   }
-  const int tiles_per_row = a.Np / 128;
-  const long total = (long)a.B * a.N * tiles_per_row;
+  const int panels = a.Np / 32;
+  const long total = (long)a.B * ((a.N + 3) / 4) * panels;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, tiles_per_row, (int)total);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, panels, (int)total);
   return hipGetLastError();
 }
 
