@@ -19,6 +19,16 @@ namespace of3 {
 
 namespace {
 
+// [position][channel] LDS tile.  Readers take, per 8 lanes, either 8 consecutive positions
+// (q, k, bias: natural order, so that their stores walk consecutive rows) or the positions
+// {x..x+3, x+16..x+19} (v: rowperm16 order).  The key (pos ^ (pos >> 2)) & 7 is distinct
+// within 8 lanes for both patterns.
+template <int NCH>
+__device__ __forceinline__ int proj_slot(int pos, int chunk) {
+  const int key = (pos ^ (pos >> 2)) & 7 & (NCH - 1);
+  return pos * NCH + (chunk ^ key);
+}
+
 template <int C, int D>
 __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, int tiles_per_row, int total_tiles) {
   constexpr int H = 4;
@@ -39,7 +49,6 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
   //   position tiles each.
   constexpr int NJ = WIDE ? 2 : 1;     // q/k/v jobs per wave (the second one only on waves 0..3)
   constexpr int TPW = 4;               // every wave visits all four position tiles
-  constexpr int KSH = 2;               // swizzle key from pos / 4
   static_assert(NT == 4 || NT == 2, "H*D must be 128 or 64");
 
   __shared__ u32x4_t tile[2][TP * NCH];
@@ -54,7 +63,6 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
   load_affine8(p.ln_w, ln_chunk, lw);
   load_affine8(p.ln_b, ln_chunk, lb);
 
-  const int tgroup = 0;
   const bool has_jobs = WIDE || wave < 6;
   // 0 q, 1 k, 2 v
   auto job_matrix = [&](int jj) { return WIDE ? (wave < 4 ? jj : 2) : wave / 2; };
@@ -66,7 +74,7 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
   for (int jj = 0; jj < NJ; ++jj) {
     const int m = job_matrix(jj);
     const bf16_t* W = (m == 0) ? p.w_q : (m == 1 ? p.w_k : p.w_v);
-    // q, k: lane owns 16 consecutive channels (rowperm16); v: natural rows
+    // q, k (A operands): lane owns 16 consecutive channels (rowperm16); v (B operand): natural rows
     const int row = 32 * ot + ((m == 2) ? l32 : rowperm16(l32));
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
@@ -104,8 +112,11 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
     }
   };
 
-  // position 32*TPW*tgroup + TPW*l32 + tt is column l32 of this wave's position tile tt
-  const int pos0 = 32 * TPW * tgroup + TPW * l32;
+  // every job takes the positions in natural order: position 32*tt + l32 is column l32 of
+  // position tile tt (q, k, bias: activations are the MFMA B operand) or, for v, row
+  // rowperm16(l32) of it (activations are the A operand, so that a lane ends up with 16
+  // consecutive keys of one channel: 32 contiguous bytes of the V^T panel)
+  const int krow = rowperm16(l32);
 
   int tile_id = blockIdx.x;
   if (tile_id < total_tiles) load_tile(tile_id);
@@ -120,7 +131,7 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
       const int pos = wave * (TP / NW) + it * PPI + ln_pp;
-      tile[buf][tile_slot<NCH, KSH>(pos, ln_chunk)] = layer_norm_chunk<C>(raw[it], lw, lb);
+      tile[buf][proj_slot<NCH>(pos, ln_chunk)] = layer_norm_chunk<C>(raw[it], lw, lb);
       if (ln_chunk == 0) {
         const int j = j0 + pos;
         float mb = -__builtin_inff();
@@ -137,13 +148,13 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
 
     // ---- projection phase
     const size_t bi = (size_t)b * N + i;
-    float vres[TPW][16];  // v job only
 #pragma unroll
     for (int tt = 0; tt < TPW; ++tt) {
-      // the B operand (this lane's position, k-step s) is re-read from LDS by every job: cheaper
-      // than holding it in 32 registers across the jobs
-      auto bop = [&](int s) { return tile[buf][tile_slot<NCH, KSH>(pos0 + tt, 2 * s + lh)]; };
-      const int j = j0 + pos0 + tt;
+      // the activation operand (this lane's position, k-step s) is re-read from LDS by every
+      // job: cheaper than holding it in 32 registers across the jobs
+      const int pos = 32 * tt + l32;
+      auto bop = [&](int s) { return tile[buf][proj_slot<NCH>(pos, 2 * s + lh)]; };
+      const int j = j0 + pos;
 
       if (has_jobs) {
 #pragma unroll
@@ -151,12 +162,27 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
           if (!job_live(jj)) continue;  // wave-uniform
           const int m = job_matrix(jj);
           f32x16_t acc = zero16();
-#pragma unroll
-          for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wj[jj][s], bop(s), acc);
           if (m == 2) {
+            // V^T panel of this position tile: rows = keys (A), columns = channels (B)
+            const int kpos = 32 * tt + krow;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) vres[tt][v] = acc[v];
+            for (int s = 0; s < KS; ++s)
+              acc = mfma_32x32x16(tile[buf][proj_slot<NCH>(kpos, 2 * s + lh)], wj[jj][s], acc);
+            // lane: channel 32*ot + l32 = head*D + d, keys 16*lh + (0..15) of the panel
+            const int ch = 32 * ot + l32;
+            const int head = ch / D, d = ch % D;
+            u32x4_t o0, o1;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              o0[q] = pack_bf16(acc[2 * q], acc[2 * q + 1]);
+              o1[q] = pack_bf16(acc[8 + 2 * q], acc[8 + 2 * q + 1]);
+            }
+            bf16_t* dst = p.vt + (bi * H + head) * D * Jp + (size_t)((j0 >> 5) + tt) * (D * 32) + d * 32 + 16 * lh;
+            *reinterpret_cast<u32x4_t*>(dst) = o0;
+            *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
           } else {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wj[jj][s], bop(s), acc);
             // lane owns channels 32*ot + 16*lh + v  ->  head, d0 .. d0+15
             const int ch0 = 32 * ot + 16 * lh;
             const int head = ch0 / D, d0 = ch0 % D;
@@ -186,25 +212,6 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
         if (lh == 0) {
 #pragma unroll
           for (int h = 0; h < H; ++h) p.tbias[(((size_t)b * H + h) * N + i) * Jp + j] = (j < N) ? acc[h] * kLog2e : 0.f;
-        }
-      }
-    }
-
-    // ---- v stores: register v is channel 32*ot + 8*(v/4) + 4*lh + v%4 = head*D + d;
-    // key-panel layout [b][i][h][key / 32][d][key % 32]
-    const bool v_job = WIDE ? wave >= 4 : (wave / 2) == 2;
-    if (has_jobs && v_job) {
-      const int j = j0 + pos0;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int ch = 32 * ot + 8 * (v >> 2) + 4 * lh + (v & 3);
-        const int head = ch / D, d = ch % D;
-        bf16_t* dst = p.vt + (bi * H + head) * D * Jp + (size_t)(j >> 5) * (D * 32) + d * 32 + (j & 31);
-        if (TPW == 4) {
-          u32x2_t w2 = {pack_bf16(vres[0][v], vres[1][v]), pack_bf16(vres[2 % TPW][v], vres[3 % TPW][v])};
-          *reinterpret_cast<u32x2_t*>(dst) = w2;
-        } else {
-          *reinterpret_cast<uint32_t*>(dst) = pack_bf16(vres[0][v], vres[1][v]);
         }
       }
     }
