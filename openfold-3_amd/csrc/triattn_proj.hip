@@ -47,7 +47,6 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
   //   carries the same MFMA load.
   // else (H*D = 64): waves 0..5 own one (matrix, tile) job, waves 6 and 7 do the bias of two
   //   position tiles each.
-  constexpr int NJ = WIDE ? 2 : 1;     // q/k/v jobs per wave (the second one only on waves 0..3)
   constexpr int TPW = 4;               // every wave visits all four position tiles
   static_assert(NT == 4 || NT == 2, "H*D must be 128 or 64");
 
@@ -63,26 +62,6 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
   load_affine8(p.ln_w, ln_chunk, lw);
   load_affine8(p.ln_b, ln_chunk, lb);
 
-  const bool has_jobs = WIDE || wave < 6;
-  // 0 q, 1 k, 2 v
-  auto job_matrix = [&](int jj) { return WIDE ? (wave < 4 ? jj : 2) : wave / 2; };
-  auto job_live = [&](int jj) { return WIDE ? (jj == 0 || wave < 4) : wave < 6; };
-  const int ot = WIDE ? wave % 4 : wave % 2;
-
-  u32x4_t wj[NJ][KS];
-#pragma unroll
-  for (int jj = 0; jj < NJ; ++jj) {
-    const int m = job_matrix(jj);
-    const bf16_t* W = (m == 0) ? p.w_q : (m == 1 ? p.w_k : p.w_v);
-    // q, k (A operands): lane owns 16 consecutive channels (rowperm16); v (B operand): natural rows
-    const int row = 32 * ot + ((m == 2) ? l32 : rowperm16(l32));
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      u32x4_t w = {0u, 0u, 0u, 0u};
-      if (job_live(jj)) w = *reinterpret_cast<const u32x4_t*>(W + row * C + 16 * s + 8 * lh);
-      wj[jj][s] = w;
-    }
-  }
   if (wave == 0) {
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
@@ -97,72 +76,107 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
   const int tiles_per_batch = N * tiles_per_row;
 
   u32x4_t raw[LN_ITERS];
+  float mraw[LN_ITERS];  // mask of the same positions (used by the lane with ln_chunk == 0)
   auto load_tile = [&](int tile_id) {
     const int b = tile_id / tiles_per_batch;
     const int rem = tile_id - b * tiles_per_batch;
     const int i = rem / tiles_per_row;
     const int j0 = (rem - i * tiles_per_row) * TP;
     const bf16_t* xrow = p.x + b * p.x_view.stride_b + i * p.x_view.stride_r;
+    const float* mrow = p.mask ? p.mask + b * p.mask_view.stride_b + i * p.mask_view.stride_r : nullptr;
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
       const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
       u32x4_t v = {0u, 0u, 0u, 0u};
-      if (j < N) v = *reinterpret_cast<const u32x4_t*>(xrow + j * p.x_view.stride_k + 8 * ln_chunk);
+      float m = 1.f;
+      if (j < N) {
+        v = *reinterpret_cast<const u32x4_t*>(xrow + j * p.x_view.stride_k + 8 * ln_chunk);
+        if (mrow && ln_chunk == 0) m = mrow[j * p.mask_view.stride_k];
+      }
       raw[it] = v;
+      mraw[it] = m;
     }
   };
 
-  // every job takes the positions in natural order: position 32*tt + l32 is column l32 of
+  // Every job takes the positions in natural order: position 32*tt + l32 is column l32 of
   // position tile tt (q, k, bias: activations are the MFMA B operand) or, for v, row
   // rowperm16(l32) of it (activations are the A operand, so that a lane ends up with 16
-  // consecutive keys of one channel: 32 contiguous bytes of the V^T panel)
+  // consecutive keys of one channel: 32 contiguous bytes of the V^T panel).
   const int krow = rowperm16(l32);
 
-  int tile_id = blockIdx.x;
-  if (tile_id < total_tiles) load_tile(tile_id);
+  // A wave's role is fixed for the kernel, and each role runs its own copy of the tile loop:
+  //   role 0  q and k of output tile w (H*D = 128), or one of them (H*D = 64: waves 0..3)
+  //   role 1  v of output tile w-4 plus the bias of position tile w-4 (H*D = 128), or v alone
+  //   role 2  bias of two position tiles (H*D = 64: waves 6, 7)
+  // Inside a role every tile issues the same sequence of loads and stores.  Together with the
+  // peeled first tile this lets the wait for the values loaded one tile ahead leave the
+  // previous tile's stores in flight (the compiler counts them; it cannot when the number
+  // depends on a branch).
+  auto run = [&](auto role_tag) {
+    constexpr int ROLE = decltype(role_tag)::value;
+    constexpr int NJ = (ROLE == 0 && WIDE) ? 2 : (ROLE == 2 ? 0 : 1);
+    const int ot = WIDE ? wave % 4 : wave % 2;
+    const int m0 = ROLE == 1 ? 2 : (WIDE ? 0 : wave / 2);  // matrix of job 0: 0 q, 1 k, 2 v
 
-  for (int buf = 0; tile_id < total_tiles; tile_id += gridDim.x, buf ^= 1) {
-    const int b = tile_id / tiles_per_batch;
-    const int rem = tile_id - b * tiles_per_batch;
-    const int i = rem / tiles_per_row;
-    const int j0 = (rem - i * tiles_per_row) * TP;
-
-    // ---- LayerNorm phase (+ mask bias, one lane per position)
+    u32x4_t wj[NJ > 0 ? NJ : 1][KS];
 #pragma unroll
-    for (int it = 0; it < LN_ITERS; ++it) {
-      const int pos = wave * (TP / NW) + it * PPI + ln_pp;
-      tile[buf][proj_slot<NCH>(pos, ln_chunk)] = layer_norm_chunk<C>(raw[it], lw, lb);
-      if (ln_chunk == 0) {
-        const int j = j0 + pos;
-        float mb = -__builtin_inff();
-        if (j < N) {
-          float m = 1.f;
-          if (p.mask) m = p.mask[b * p.mask_view.stride_b + i * p.mask_view.stride_r + j * p.mask_view.stride_k];
-          mb = kLog2e * (p.inf * (m - 1.f));
-        }
-        p.mbias[((size_t)b * N + i) * Jp + j] = mb;
-      }
+    for (int jj = 0; jj < NJ; ++jj) {
+      const int m = m0 + jj;
+      const bf16_t* W = (m == 0) ? p.w_q : (m == 1 ? p.w_k : p.w_v);
+      // q, k (A operands): lane owns 16 consecutive channels (rowperm16); v (B operand): natural rows
+      const int row = 32 * ot + ((ROLE == 1) ? l32 : rowperm16(l32));
+#pragma unroll
+      for (int s = 0; s < KS; ++s) wj[jj][s] = *reinterpret_cast<const u32x4_t*>(W + row * C + 16 * s + 8 * lh);
     }
-    if (tile_id + (int)gridDim.x < total_tiles) load_tile(tile_id + gridDim.x);
-    __syncthreads();  // the only barrier per tile (the LDS tile is double buffered)
 
-    // ---- projection phase
-    const size_t bi = (size_t)b * N + i;
+    auto do_tile = [&](int tile_id, int buf) {
+      const int b = tile_id / tiles_per_batch;
+      const int rem = tile_id - b * tiles_per_batch;
+      const int i = rem / tiles_per_row;
+      const int j0 = (rem - i * tiles_per_row) * TP;
+
+      // ---- LayerNorm phase (+ mask bias, one lane per position)
 #pragma unroll
-    for (int tt = 0; tt < TPW; ++tt) {
-      // the activation operand (this lane's position, k-step s) is re-read from LDS by every
-      // job: cheaper than holding it in 32 registers across the jobs
-      const int pos = 32 * tt + l32;
-      auto bop = [&](int s) { return tile[buf][proj_slot<NCH>(pos, 2 * s + lh)]; };
-      const int j = j0 + pos;
+      for (int it = 0; it < LN_ITERS; ++it) {
+        const int pos = wave * (TP / NW) + it * PPI + ln_pp;
+        tile[buf][proj_slot<NCH>(pos, ln_chunk)] = layer_norm_chunk<C>(raw[it], lw, lb);
+        if (ln_chunk == 0) {
+          const int j = j0 + pos;
+          float mb = -__builtin_inff();
+          if (j < N) mb = kLog2e * (p.inf * (mraw[it] - 1.f));
+          p.mbias[((size_t)b * N + i) * Jp + j] = mb;
+        }
+      }
+      if (tile_id + (int)gridDim.x < total_tiles) load_tile(tile_id + gridDim.x);
+      __syncthreads();  // the only barrier per tile (the LDS tile is double buffered)
 
-      if (has_jobs) {
+      // ---- projection phase
+      const size_t bi = (size_t)b * N + i;
+      auto bias_tile = [&](int tt) {  // triangle bias of position tile tt (wave-uniform, may be a run-time value)
+        const int pos = 32 * tt + l32, j = j0 + pos;
+        f32x16_t acc = zero16();
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+          acc = mfma_32x32x16(wb_lds[s * 64 + lane], tile[buf][proj_slot<NCH>(pos, 2 * s + lh)], acc);
+        // rows 0..3 of the result sit in registers 0..3 of lanes 0..31
+        if (lh == 0) {
+#pragma unroll
+          for (int h = 0; h < H; ++h) p.tbias[(((size_t)b * H + h) * N + i) * Jp + j] = (j < N) ? acc[h] * kLog2e : 0.f;
+        }
+      };
+      if (ROLE == 2) {
+        bias_tile(2 * (wave - 6));
+        bias_tile(2 * (wave - 6) + 1);
+        return;
+      }
+#pragma unroll
+      for (int tt = 0; tt < TPW; ++tt) {
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj) {
-          if (!job_live(jj)) continue;  // wave-uniform
-          const int m = job_matrix(jj);
           f32x16_t acc = zero16();
-          if (m == 2) {
+          u32x4_t o0, o1;
+          bf16_t* dst;
+          if (ROLE == 1) {
             // V^T panel of this position tile: rows = keys (A), columns = channels (B)
             const int kpos = 32 * tt + krow;
 #pragma unroll
@@ -171,50 +185,56 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
             // lane: channel 32*ot + l32 = head*D + d, keys 16*lh + (0..15) of the panel
             const int ch = 32 * ot + l32;
             const int head = ch / D, d = ch % D;
-            u32x4_t o0, o1;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               o0[q] = pack_bf16(acc[2 * q], acc[2 * q + 1]);
               o1[q] = pack_bf16(acc[8 + 2 * q], acc[8 + 2 * q + 1]);
             }
-            bf16_t* dst = p.vt + (bi * H + head) * D * Jp + (size_t)((j0 >> 5) + tt) * (D * 32) + d * 32 + 16 * lh;
-            *reinterpret_cast<u32x4_t*>(dst) = o0;
-            *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
+            dst = p.vt + (bi * H + head) * D * Jp + (size_t)((j0 >> 5) + tt) * (D * 32) + d * 32 + 16 * lh;
           } else {
+            // the activation operand is re-read from LDS by every job: cheaper than holding it in
+            // 32 registers across the jobs
+            const int pos = 32 * tt + l32;
 #pragma unroll
-            for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wj[jj][s], bop(s), acc);
+            for (int s = 0; s < KS; ++s)
+              acc = mfma_32x32x16(wj[jj][s], tile[buf][proj_slot<NCH>(pos, 2 * s + lh)], acc);
             // lane owns channels 32*ot + 16*lh + v  ->  head, d0 .. d0+15
             const int ch0 = 32 * ot + 16 * lh;
             const int head = ch0 / D, d0 = ch0 % D;
-            const float sc = (m == 0) ? qscale : 1.f;
-            u32x4_t o0, o1;
+            const bool is_q = (m0 + jj) == 0;
+            const float sc = is_q ? qscale : 1.f;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               o0[q] = pack_bf16(acc[2 * q] * sc, acc[2 * q + 1] * sc);
               o1[q] = pack_bf16(acc[8 + 2 * q] * sc, acc[8 + 2 * q + 1] * sc);
             }
-            bf16_t* base = (m == 0) ? p.q : p.k;
-            bf16_t* dst = base + ((bi * H + head) * Jp + j) * D + d0;
-            *reinterpret_cast<u32x4_t*>(dst) = o0;
-            *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
+            dst = (is_q ? p.q : p.k) + ((bi * H + head) * Jp + j0 + pos) * D + d0;
           }
+          *reinterpret_cast<u32x4_t*>(dst) = o0;
+          *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
         }
       }
+      if (ROLE == 1 && WIDE) bias_tile(wave - 4);
+    };
 
-      // triangle bias: WIDE -> wave 4+tt does position tile tt; else waves 6, 7 take position
-      // tiles {0,1} and {2,3}
-      const bool bias_here = WIDE ? (wave == 4 + tt) : (wave >= 6 && (tt >> 1) == (wave - 6));
-      if (bias_here) {
-        f32x16_t acc = zero16();
-#pragma unroll
-        for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wb_lds[s * 64 + lane], bop(s), acc);
-        // rows 0..3 of the result sit in registers 0..3 of lanes 0..31
-        if (lh == 0) {
-#pragma unroll
-          for (int h = 0; h < H; ++h) p.tbias[(((size_t)b * H + h) * N + i) * Jp + j] = (j < N) ? acc[h] * kLog2e : 0.f;
-        }
-      }
+    int tile_id = blockIdx.x;
+    int buf = 0;
+    if (tile_id < total_tiles) {
+      load_tile(tile_id);
+      do_tile(tile_id, buf);
+      tile_id += gridDim.x;
+      buf ^= 1;
     }
+    for (; tile_id < total_tiles; tile_id += gridDim.x, buf ^= 1) do_tile(tile_id, buf);
+  };
+
+  if (WIDE) {
+    if (wave < 4) run(std::integral_constant<int, 0>{});
+    else run(std::integral_constant<int, 1>{});
+  } else {
+    if (wave < 4) run(std::integral_constant<int, 0>{});
+    else if (wave < 6) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, 2>{});
   }
 }
 
