@@ -1,0 +1,93 @@
+"""Edge cases of the HIP path: smallest and ragged sizes, strided and sliced inputs, mask dtypes,
+other streams, run-to-run determinism.  Same oracle and tolerances as tests/test_gpu_parity.py."""
+import pytest
+import torch
+
+from gpu_util import lib  # noqa: F401
+from oracle import pairstack_oracle as orc
+from test_gpu_parity import _check, _load, _round_params, DEV
+
+import of3pair
+
+pytestmark = pytest.mark.gpu
+
+
+def _block(c, d, seed=0):
+    p = _round_params(orc.make_block_params(seed, c, c, d, 4))
+    return _load(of3pair.PairStack(c, c, d, 4), p), p
+
+
+@pytest.mark.parametrize("n", [1, 2, 31, 33, 129, 200])
+def test_block_small_and_ragged_sizes(n):
+    """N = 1 (a single token), N below, at and just above the 32-key and 128-position tile sizes."""
+    lib()
+    m, p = _block(128, 32, seed=30 + n)
+    gen = torch.Generator().manual_seed(n)
+    z = orc.round_bf16(torch.randn(2, n, n, 128, generator=gen))
+    mask = (torch.rand(2, n, n, generator=gen) > 0.15).float()
+    mask[0] = 1.0
+    print("ragged block n =", n, flush=True)
+    got = m(z.to(DEV).to(torch.bfloat16), mask.to(DEV))
+    want = orc.pair_stack_block(z, mask, p, 4)
+    _check("block n=%d" % n, got, want, rms_rel=1.2e-2)
+
+
+def test_fully_masked_input():
+    """mask == 0 everywhere: trimul contributes (LN_out.bias Wz^T)*gate, attention averages v uniformly."""
+    lib()
+    n = 48
+    m, p = _block(64, 16, seed=41)
+    z = orc.round_bf16(orc.make_pair_input(42, (1,), n, 64))
+    mask = torch.zeros(1, n, n)
+    got = m(z.to(DEV).to(torch.bfloat16), mask.to(DEV))
+    _check("all masked", got, orc.pair_stack_block(z, mask, p, 4), rms_rel=1.2e-2)
+
+
+def test_strided_batch_and_sliced_inputs():
+    """A batch taken as every other element of a larger tensor and a square window of a larger pair
+    tensor: the kernels follow the strides, nothing is copied for the batch case."""
+    lib()
+    n = 40
+    gen = torch.Generator().manual_seed(50)
+    p = _round_params(orc.make_trimul_params(gen, 128, 128))
+    m = _load(of3pair.TriangleMultiplicationIncoming(128, 128), p)
+    big = orc.round_bf16(torch.randn(4, n, n, 128, generator=gen))
+    bg = big.to(DEV).to(torch.bfloat16)
+    got = m(bg[::2])                                    # batch stride 2*N*N*C
+    _check("strided batch", got, orc.trimul_update(big[::2], None, p, False))
+    win = bg[1, 4:36, 4:36, :]                          # row stride N*C, 32 x 32 window
+    got = m(win)
+    _check("window", got, orc.trimul_update(big[1, 4:36, 4:36, :], None, p, False))
+    pa = _round_params(orc.make_triattn_params(gen, 128, 32, 4))
+    a = _load(of3pair.TriangleAttention(128, 32, 4, starting=False), pa)
+    got = a(win, mask=torch.ones(32, 32, device=DEV))
+    _check("window attention", got, orc.triattn_update(big[1, 4:36, 4:36, :], None, pa, 4, starting=False), rms_rel=6e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bool, torch.int32, torch.bfloat16, torch.float64])
+def test_mask_dtypes(dtype):
+    """The reference accepts 0/1 masks of any dtype (tmu.py:485, tri_att.py:134)."""
+    lib()
+    n = 36
+    m, p = _block(128, 32, seed=60)
+    gen = torch.Generator().manual_seed(61)
+    z = orc.round_bf16(torch.randn(1, n, n, 128, generator=gen))
+    mask = (torch.rand(1, n, n, generator=gen) > 0.3)
+    got = m(z.to(DEV).to(torch.bfloat16), mask.to(dtype).to(DEV))
+    _check("mask " + str(dtype), got, orc.pair_stack_block(z, mask.float(), p, 4), rms_rel=1.2e-2)
+
+
+def test_runs_on_the_current_stream_and_is_deterministic():
+    lib()
+    n = 96
+    m, p = _block(128, 32, seed=70)
+    z = orc.round_bf16(orc.make_pair_input(71, (1,), n, 128)).to(DEV).to(torch.bfloat16)
+    mask = orc.tail_padding_mask((1,), n, 7).to(DEV)
+    ref = m(z, mask)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        outs = [m(z, mask) for _ in range(3)]
+    side.synchronize()
+    for o in outs:
+        assert torch.equal(o, ref), "results differ between runs / streams"
