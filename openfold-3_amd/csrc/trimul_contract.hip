@@ -330,12 +330,6 @@ hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, i
       return launch_contract<128, 4>(a, b, x, planes, Np, stream);
     case 3:
       return launch_contract<256, 4>(a, b, x, planes, Np, stream);
-    case 4:
-      return launch_contract<128, 5>(a, b, x, planes, Np, stream);
-    case 5:
-      return launch_contract<128, 3>(a, b, x, planes, Np, stream);
-    case 6:
-      return launch_contract<192, 3>(a, b, x, planes, Np, stream);
     default:
       return hipErrorInvalidValue;
   }
