@@ -23,8 +23,13 @@
  *       :625-672  _cueq_triangle_attn (q,k,v [B,I,H,J,c], triangle bias, boolean mask,
  *                 scale) / :94-135 _attention                   -> of3_triattn_flash
  *       :288-302  Attention._wrap_up (gate, linear_o)           -> of3_triattn_out
+ *   openfold3/core/model/layers/transition.py
+ *       :225-271  SwiGLUTransition.forward (LayerNorm, SwiGLU of
+ *                 openfold3/core/model/primitives/activations.py:33-61,
+ *                 linear_out, mask)                             -> of3_transition_fwd
  *   openfold3/core/model/latent/base_blocks.py
  *       :329-335  "z = z + update" after each module            -> add_residual = 1
+ *       :470-478  "z = z + pair_transition(z, mask)"            -> of3_transition_fwd, add_residual = 1
  *
  * Shapes: B batch (templates are folded into B), N tokens, C = c_z, CH = c_hidden of the
  * triangle multiplication, H heads of per-head width D.  Supported: (C, CH) in
@@ -39,8 +44,8 @@
  * own element strides; a null mask means all ones (tmu.py:482-483, tri_att.py:120-124).
  *
  * dtype: OF3_DTYPE_BF16 selects the MFMA kernels described above.  OF3_DTYPE_F32 (the
- * reference's default inference precision) is served by of3_trimul_fwd / of3_triattn_fwd
- * only: every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
+ * reference's default inference precision) is served by of3_trimul_fwd / of3_triattn_fwd /
+ * of3_transition_fwd only: every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
  * element counts, any N, C and CH <= 256, H*D <= 256 with D in {16, 32, 64}; plain fp32
  * arithmetic in the reference's order of operations (no MFMA, not the fast path).  The
  * stage entry points are bf16 only.
@@ -134,6 +139,19 @@ int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask
                     const void* w_v, const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C,
                     int64_t H, int64_t D, float inf, int add_residual, void* workspace, int64_t workspace_bytes,
                     int dtype, void* stream);
+
+/* ---- pair transition ------------------------------------------------------------------ */
+
+/* out = [x +] ((silu(LN(x) Wa^T) * (LN(x) Wb^T)) Wout^T) * mask, position-wise; out uses x's
+ * strides and may alias x (every position is read before it is written, by the same wave).
+ * w_a, w_b: [HID][C] (SwiGLU linear_a, the half passed through SiLU, and linear_b);
+ * w_out: [C][HID]; HID = n*C.  No bias terms (the reference's Linear(bias=False)), no
+ * workspace.  bf16: C in {64, 128}, HID a multiple of 32 and >= 128, a row's extent
+ * (N-1)*stride_j elements below 2^31.  fp32: C <= 256, HID <= 1024. */
+int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
+                       const void* ln_w, const void* ln_b, const void* w_a, const void* w_b, const void* w_out,
+                       void* out, int64_t B, int64_t N, int64_t C, int64_t HID, int add_residual, int dtype,
+                       void* stream);
 
 #ifdef __cplusplus
 }

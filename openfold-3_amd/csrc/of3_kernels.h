@@ -85,6 +85,19 @@ struct TriattnOutArgs {
 };
 hipError_t triattn_out_launch(const TriattnOutArgs& args, int C, int HD, hipStream_t stream);
 
+struct TransitionArgs {
+  const bf16_t* x;    // pair tensor, x_view addressing
+  const float* mask;  // may be null (all ones)
+  PairView x_view, mask_view;
+  const bf16_t *ln_w, *ln_b;  // [C]
+  const bf16_t *w_a, *w_b;    // [HID][C]  (SwiGLU linear_a: the gated half, linear_b)
+  const bf16_t *w_out;        // [C][HID]
+  bf16_t* out;                // x_view addressing
+  int B, N, HID;
+  int add_residual;
+};
+hipError_t transition_launch(const TransitionArgs& args, int C, hipStream_t stream);
+
 // ---- fp32 path (pair_f32.hip): whole updates, any N, C and C_hidden <= 256, head width 16/32/64
 struct TrimulF32Args {
   const float* z;
@@ -112,5 +125,15 @@ struct TriattnF32Args {
   float inf;
 };
 hipError_t triattn_fwd_f32(const TriattnF32Args& args, hipStream_t stream);
+
+struct TransitionF32Args {
+  const float* x;
+  const float* mask;  // may be null
+  PairView x_view, mask_view;
+  const float *ln_w, *ln_b, *w_a, *w_b, *w_out;  // [C], [C], [HID][C], [HID][C], [C][HID]
+  float* out;
+  int B, N, C, HID, add_residual;
+};
+hipError_t transition_fwd_f32(const TransitionF32Args& args, hipStream_t stream);
 
 }  // namespace of3

@@ -401,4 +401,62 @@ int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask
   return of3_triattn_out(o, x, x_strides, out, ln_w, ln_b, w_g, w_o, B, N, C, H, D, add_residual, stream);
 }
 
+int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
+                       const void* ln_w, const void* ln_b, const void* w_a, const void* w_b, const void* w_out,
+                       void* out, int64_t B, int64_t N, int64_t C, int64_t HID, int add_residual, int dtype,
+                       void* stream) {
+  const void* ptrs[] = {x, ln_w, ln_b, w_a, w_b, w_out, out};
+  if (B < 1 || N < 1 || N > (1 << 20) || !mask_ok(mask, mask_strides)) return OF3_EINVAL;
+  if (dtype == OF3_DTYPE_F32) {
+    if (N > (1 << 16) || C < 1 || C > 256 || HID < 1 || HID > 1024 || !f32_strides_ok(x_strides)) return OF3_EINVAL;
+    for (const void* p : ptrs)
+      if (!p || !aligned4(p)) return OF3_EINVAL;
+    auto f = [](const void* p) { return static_cast<const float*>(p); };
+    of3::TransitionF32Args a;
+    a.x = f(x);
+    a.mask = mask;
+    a.x_view = view(x_strides, false);
+    a.mask_view = mask_view(mask, mask_strides, false);
+    a.ln_w = f(ln_w);
+    a.ln_b = f(ln_b);
+    a.w_a = f(w_a);
+    a.w_b = f(w_b);
+    a.w_out = f(w_out);
+    a.out = static_cast<float*>(out);
+    a.B = (int)B;
+    a.N = (int)N;
+    a.C = (int)C;
+    a.HID = (int)HID;
+    a.add_residual = add_residual ? 1 : 0;
+    hipError_t e = of3::transition_fwd_f32(a, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? OF3_OK : fail_hip(e);
+  }
+  if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
+  if (!(C == 128 || C == 64) || HID < 128 || HID % 32 != 0 || HID > (1 << 16) || !strides_ok(x_strides))
+    return OF3_EINVAL;
+  // positions along a row are addressed with 32-bit byte offsets
+  if ((N - 1) * x_strides[2] * 2 + 2 * C > 0xffffffffll) return OF3_EINVAL;
+  if (mask && (N - 1) * mask_strides[2] * 4 + 4 > 0xffffffffll) return OF3_EINVAL;
+  if (B * N * ((N + 255) / 256) > 0x7fffffffll) return OF3_EINVAL;
+  for (const void* p : ptrs)
+    if (!p || !aligned16(p)) return OF3_EINVAL;
+  of3::TransitionArgs args;
+  args.x = bf(x);
+  args.mask = mask;
+  args.x_view = view(x_strides, false);
+  args.mask_view = mask_view(mask, mask_strides, false);
+  args.ln_w = bf(ln_w);
+  args.ln_b = bf(ln_b);
+  args.w_a = bf(w_a);
+  args.w_b = bf(w_b);
+  args.w_out = bf(w_out);
+  args.out = bf(out);
+  args.B = (int)B;
+  args.N = (int)N;
+  args.HID = (int)HID;
+  args.add_residual = add_residual ? 1 : 0;
+  hipError_t e = of3::transition_launch(args, (int)C, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
 }  // extern "C"

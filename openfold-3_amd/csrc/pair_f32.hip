@@ -3,6 +3,7 @@
 // operations as the reference's stock PyTorch path:
 //   triangle multiplication   triangular_multiplicative_update.py:482-503, :71-97
 //   triangle attention        triangular_attention.py:102-167, attention.py:94-135,265-302
+//   pair transition           transition.py:225-271, activations.py:33-61
 // These kernels are written for exactness and generality (any N, C, C_hidden <= 256, head
 // width <= 64), with plain fp32 FMA arithmetic, full-precision expf and no MFMA; they are the
 // precision reference of the library on the GPU, not its fast path (that is the bf16 path).
@@ -304,6 +305,49 @@ __global__ __launch_bounds__(kThreads) void triattn_out_f32(TriattnF32 p, int gr
   }
 }
 
+// ---- pair transition -------------------------------------------------------------------------
+constexpr int kMaxHid = 1024;
+
+struct TransitionF32 {
+  const float *x, *mask;
+  PairView xv, mv;
+  const float *ln_w, *ln_b, *w_a, *w_b, *w_out;
+  float* out;
+  int B, N, C, HID, add_residual;
+};
+
+// out = [x +] ((silu(xn Wa^T) * (xn Wb^T)) Wout^T) * mask for kP positions of one row
+__global__ __launch_bounds__(kThreads) void transition_f32(TransitionF32 p, int groups) {
+  __shared__ float xn[kP][kMaxC];
+  __shared__ float hid[kP][kMaxHid];
+  const int N = p.N, C = p.C, HID = p.HID;
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kP;
+  layer_norm_rows(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+      },
+      p.ln_w, p.ln_b, C, xn);
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * HID; idx += kThreads) {
+    const int pos = idx / HID, hd = idx % HID;
+    const float a = dot_row(xn[pos], p.w_a + (size_t)hd * C, C);
+    const float bb = dot_row(xn[pos], p.w_b + (size_t)hd * C, C);
+    hid[pos][hd] = (a * sigmoid_f32(a)) * bb;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * C; idx += kThreads) {
+    const int pos = idx / C, co = idx % C, j = j0 + pos;
+    if (j >= N) continue;
+    float res = dot_row(hid[pos], p.w_out + (size_t)co * HID, HID);
+    if (p.mask) res *= p.mask[b * p.mv.stride_b + i * p.mv.stride_r + j * p.mv.stride_k];
+    const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
+    if (p.add_residual) res = p.x[o] + res;
+    p.out[o] = res;
+  }
+}
+
 }  // namespace
 
 hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
@@ -385,6 +429,30 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   else
     return hipErrorInvalidValue;
   hipLaunchKernelGGL(triattn_out_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  return hipGetLastError();
+}
+
+hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
+  if (a.C > kMaxC || a.HID > kMaxHid) return hipErrorInvalidValue;
+  TransitionF32 p;
+  p.x = a.x;
+  p.mask = a.mask;
+  p.xv = a.x_view;
+  p.mv = a.mask_view;
+  p.ln_w = a.ln_w;
+  p.ln_b = a.ln_b;
+  p.w_a = a.w_a;
+  p.w_b = a.w_b;
+  p.w_out = a.w_out;
+  p.out = a.out;
+  p.B = a.B;
+  p.N = a.N;
+  p.C = a.C;
+  p.HID = a.HID;
+  p.add_residual = a.add_residual;
+  const int groups = (a.N + kP - 1) / kP;
+  const long blocks = (long)a.B * a.N * groups;
+  hipLaunchKernelGGL(transition_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
   return hipGetLastError();
 }
 

@@ -37,6 +37,8 @@ SIGNATURES = {
     "of3_triattn_out": (c_int, [c_void_p, c_void_p, _I64x3] + [c_void_p] * 5 + [c_int64] * 5 + [c_int, c_void_p]),
     "of3_triattn_fwd": (c_int, [c_void_p, _I64x3, c_void_p, _I64x3] + [c_void_p] * 9 + [c_int64] * 5
                         + [c_float, c_int, c_void_p, c_int64, c_int, c_void_p]),
+    "of3_transition_fwd": (c_int, [c_void_p, _I64x3, c_void_p, _I64x3] + [c_void_p] * 6 + [c_int64] * 4
+                           + [c_int, c_int, c_void_p]),
 }
 
 _lib = None

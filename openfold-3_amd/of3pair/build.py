@@ -26,6 +26,7 @@ SOURCES = [
     "triattn_proj.hip",
     "triattn_flash.hip",
     "triattn_out.hip",
+    "transition.hip",
     "pair_f32.hip",
 ]
 

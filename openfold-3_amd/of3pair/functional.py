@@ -160,3 +160,30 @@ def triangle_attention(x, mask, norm_weight, norm_bias, bias_weight, q_weight, k
                                  int(bool(add_residual)), ws.data_ptr(), ws.numel(), code, _stream(x))
     _lib.check(st, "of3_triattn_fwd")
     return _finish(x, x4, out4, lead, inplace)
+
+
+def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_weight, add_residual: bool = False,
+                      inplace: bool = False):
+    """Update of transition.py:256-268 (LayerNorm, SwiGLU, linear_out, mask), or x + update when
+    add_residual.  x [*, N, N, C], mask [*, N, N] or None; a_weight / b_weight [n*C, C] are
+    SwiGLU's linear_a (through SiLU) and linear_b, out_weight [C, n*C]."""
+    code = _require_gpu(x, "x")
+    lib = _lib.load()
+    x4, lead = _flatten_pair(x)
+    B, N, _, C = x4.shape
+    HID = a_weight.shape[0]
+    if tuple(a_weight.shape) != (HID, C) or tuple(b_weight.shape) != (HID, C) or tuple(out_weight.shape) != (C, HID):
+        raise ValueError("transition weights must be [n*C, C], [n*C, C] and [C, n*C]")
+    keep = [_w(t, x.dtype) for t in (norm_weight, norm_bias, a_weight, b_weight, out_weight)]
+    m3, mptr, mstr = _mask_arg(mask, lead, B, N, x.device)
+    out4 = x4 if inplace else _out_like(x4)
+    with torch.cuda.device(x.device):
+        st = lib.of3_transition_fwd(x4.data_ptr(), _lib.strides3(x4.stride()[:3]), mptr, mstr,
+                                    *[k.data_ptr() for k in keep], out4.data_ptr(), B, N, C, HID,
+                                    int(bool(add_residual)), code, _stream(x))
+    if st == _lib.OF3_EINVAL:
+        raise ValueError("pair transition: bf16 supports c_in 64 or 128 with a hidden width n*c_in that is a multiple "
+                         "of 32 and at least 128, fp32 c_in <= 256 and n*c_in <= 1024; got c_in=%d hidden=%d in %s"
+                         % (C, HID, x.dtype))
+    _lib.check(st, "of3_transition_fwd")
+    return _finish(x, x4, out4, lead, inplace)

@@ -3,6 +3,7 @@
 Constructor arguments, parameter names (state-dict keys) and forward signatures follow
   openfold3/core/model/layers/triangular_multiplicative_update.py:119-152, :421-429, :506-519
   openfold3/core/model/layers/triangular_attention.py:31-69, :102-111, :171-179
+  openfold3/core/model/layers/transition.py:225-255, :90-110 (SwiGLUTransition)
 so that a PairBlock (openfold3/core/model/latent/base_blocks.py:268-288) can hold these
 modules instead and load the same checkpoints.  The arithmetic runs in libof3pair (HIP);
 there is one implementation, so the reference's kernel-selection and chunking keyword
@@ -35,6 +36,8 @@ def _truncated_normal_(weight: torch.Tensor, scale: float = 1.0):
 def _init_linear(lin: nn.Linear, how: str):
     if how == "default":
         _truncated_normal_(lin.weight)
+    elif how in ("relu", "he_normal"):  # He initialisation, truncated normal (initialization.py:66-67)
+        _truncated_normal_(lin.weight, scale=2.0)
     elif how in ("final", "gating"):
         with torch.no_grad():
             lin.weight.zero_()
@@ -53,6 +56,10 @@ TRI_ATT_INIT = {
     "mha": {"linear_q": "default", "linear_k": "default", "linear_v": "default", "linear_g": "gating",
             "linear_o": "final"},
 }
+
+
+# default_linear_init_config.py:29-34, :157-162
+SWIGLU_TRANSITION_INIT = {"swiglu": {"linear_a": "relu", "linear_b": "relu"}, "linear_out": "final"}
 
 
 def _init_name(spec, key, default):
@@ -187,3 +194,46 @@ class TriangleAttentionEndingNode(TriangleAttention):
     """AF3 Algorithm 15."""
 
     __init__ = partialmethod(TriangleAttention.__init__, starting=False)
+
+
+class _SwiGLUParams(nn.Module):
+    """Parameter holder with the names of the reference's SwiGLU (activations.py:33-55)."""
+
+    def __init__(self, c_in, c_out, init):
+        super().__init__()
+        self.c_in = c_in
+        self.c_out = c_out
+        self.linear_a = nn.Linear(c_in, c_out, bias=False)
+        self.linear_b = nn.Linear(c_in, c_out, bias=False)
+        for name, default in SWIGLU_TRANSITION_INIT["swiglu"].items():
+            _init_linear(getattr(self, name), _init_name(init, name, default))
+
+
+class SwiGLUTransition(nn.Module):
+    """AF3 Algorithm 11 as the pair stack uses it (transition.py:225-271): LayerNorm, SwiGLU,
+    linear_out, mask.  State-dict keys: layer_norm.{weight,bias}, swiglu.linear_{a,b}.weight,
+    linear_out.weight.  Pair tensors only: x [*, N, N, C_in], mask [*, N, N]."""
+
+    def __init__(self, c_in, n, linear_init_params=None):
+        super().__init__()
+        self.c_in = c_in
+        self.n = n
+        self.layer_norm = nn.LayerNorm(c_in, eps=1e-5)
+        sw = None
+        if linear_init_params is not None:
+            sw = linear_init_params["swiglu"] if "swiglu" in linear_init_params else None
+        self.swiglu = _SwiGLUParams(c_in, n * c_in, sw)
+        self.linear_out = nn.Linear(n * c_in, c_in, bias=False)
+        _init_linear(self.linear_out, _init_name(linear_init_params, "linear_out", SWIGLU_TRANSITION_INIT["linear_out"]))
+
+    @torch.no_grad()
+    def forward(self, x, mask=None, chunk_size=None, ckpt_chunk_size=None, _add_residual=False, _inplace=False):
+        """x [*, N, N, C_in], mask [*, N, N] or None (all ones, transition.py:106-107) -> the
+        update.  chunk_size / ckpt_chunk_size of the reference are accepted and ignored: the
+        hidden activations never leave the registers, so there is nothing to chunk.
+        _add_residual / _inplace (not in the reference) return x + update from the kernel and
+        overwrite x; the pair-stack runner uses them for the add of base_blocks.py:470-478."""
+        return F3.swiglu_transition(
+            x, mask, self.layer_norm.weight, self.layer_norm.bias, self.swiglu.linear_a.weight,
+            self.swiglu.linear_b.weight, self.linear_out.weight, add_residual=bool(_add_residual),
+            inplace=bool(_inplace))

@@ -13,15 +13,16 @@ import torch
 import torch.nn as nn
 
 from . import functional as F3
-from .layers import (TriangleAttention, TriangleMultiplicationIncoming, TriangleMultiplicationOutgoing)
+from .layers import (SwiGLUTransition, TriangleAttention, TriangleMultiplicationIncoming,
+                     TriangleMultiplicationOutgoing)
 
 
 class PairStack(nn.Module):
     """tri_mul_out -> tri_mul_in -> tri_att_start -> tri_att_end, each followed by its
     residual add (dropout is the identity in eval mode, dropout.py:57-58).  Sub-module names
     match PairBlock's, so `pair_stack.<name>.<param>` checkpoint keys load unchanged.  The
-    pair transition that follows in PairBlock.forward (base_blocks.py:470-478) is not part of
-    this module."""
+    pair transition that follows in PairBlock.forward (base_blocks.py:470-478) is added by the
+    PairBlock subclass below."""
 
     def __init__(self, c_z: int, c_hidden_mul: int, c_hidden_pair_att: int, no_heads_pair: int,
                  inf: float = 1e9, linear_init_params=None):
@@ -82,3 +83,37 @@ class PairStack(nn.Module):
         z = self.tri_mul_out_in(z, pair_mask, inplace_safe=inplace_safe)
         # z is now a tensor this module owns (or the caller allowed overwriting)
         return self.tri_att_start_end(z, pair_mask, inplace_safe=True)
+
+
+class PairBlock(PairStack):
+    """The reference's PairBlock (base_blocks.py:218-480): the four triangle updates, then
+    z + pair_transition(z, mask).  Same constructor arguments and sub-module names
+    (tri_mul_out, tri_mul_in, tri_att_start, tri_att_end, pair_transition).  Only what the
+    AF3 configuration uses is implemented: the SwiGLU transition and un-fused projection
+    weights; pair_dropout is accepted for signature parity (inference: identity)."""
+
+    def __init__(self, c_z: int, c_hidden_mul: int, c_hidden_pair_att: int, no_heads_pair: int,
+                 transition_type: str = "swiglu", transition_n: int = 4, pair_dropout: float = 0.0,
+                 fuse_projection_weights: bool = False, inf: float = 1e9, linear_init_params=None):
+        if transition_type != "swiglu":
+            raise ValueError("Transition type %s is not available (the kernels implement 'swiglu')" % transition_type)
+        if fuse_projection_weights:
+            raise ValueError("fused projection weights are not implemented")
+        super().__init__(c_z, c_hidden_mul, c_hidden_pair_att, no_heads_pair, inf=inf,
+                         linear_init_params=linear_init_params)
+        pt = None
+        if linear_init_params is not None and "pair_transition" in linear_init_params:
+            pt = linear_init_params["pair_transition"]
+            pt = pt["swiglu"] if "swiglu" in pt else pt
+        self.pair_transition = SwiGLUTransition(c_z, transition_n, linear_init_params=pt)
+        self.pair_dropout = pair_dropout
+
+    @torch.no_grad()
+    def forward(self, z, pair_mask, chunk_size=None, use_deepspeed_evo_attention=False,
+                use_cueq_triangle_kernels=False, use_lma=False, inplace_safe: bool = False,
+                _mask_trans: bool = True, _attn_chunk_size=None):
+        """base_blocks.py:408-480.  _mask_trans=False runs the transition unmasked
+        (base_blocks.py:445-448)."""
+        z = super().forward(z, pair_mask, inplace_safe=inplace_safe)
+        # z is owned by this call (or may be overwritten): the transition updates it in place
+        return self.pair_transition(z, mask=pair_mask if _mask_trans else None, _add_residual=True, _inplace=True)

@@ -121,3 +121,26 @@ def triattn_update(x, mask, p, no_heads, starting=True, inf=1e9):
                 o[h * c:(h + 1) * c] = w @ vals
             out[i, j] = Wo @ (o * gv)
     return out
+
+
+def transition_update(x, mask, p):
+    """(silu(LN(x) Wa^T) * (LN(x) Wb^T)) Wout^T * mask, one position at a time
+    (transition.py:261-271, activations.py:60-61); silu(t) = t / (1 + exp(-t))."""
+    x = _f64(x)
+    shape = x.shape
+    c = shape[-1]
+    xf = x.reshape(-1, c)
+    mf = np.ones(xf.shape[0]) if mask is None else _f64(mask).reshape(-1)
+    lw, lb = _f64(p["layer_norm.weight"]), _f64(p["layer_norm.bias"])
+    wa, wb, wo = _f64(p["swiglu.linear_a.weight"]), _f64(p["swiglu.linear_b.weight"]), _f64(p["linear_out.weight"])
+    out = np.zeros_like(xf)
+    for r in range(xf.shape[0]):
+        xn = _ln(xf[r], lw, lb)
+        h = np.zeros(wa.shape[0])
+        for j in range(wa.shape[0]):
+            ta = float(np.dot(wa[j], xn))
+            tb = float(np.dot(wb[j], xn))
+            h[j] = ta / (1.0 + math.exp(-ta)) * tb
+        for co in range(c):
+            out[r, co] = float(np.dot(wo[co], h)) * mf[r]
+    return out.reshape(shape)

@@ -162,6 +162,46 @@ def triattn_update(x, mask, p, no_heads: int, starting: bool = True, inf: float 
 
 
 # --------------------------------------------------------------------------
+# pair transition (the step that follows the pair stack in every PairBlock)
+# --------------------------------------------------------------------------
+def transition_update(x, mask, p):
+    """SwiGLUTransition.forward (transition.py:96-128, :261-271) with SwiGLU of
+    activations.py:60-61: LayerNorm, silu(x Wa^T) * (x Wb^T), linear_out, times mask.
+    x: [*, C]; mask: x.shape[:-1] or None (ones, transition.py:113-114).  Returns the update
+    only; the caller adds it to z (base_blocks.py:470-478).  Parameter names as in the
+    reference: layer_norm.{weight,bias}, swiglu.linear_a.weight, swiglu.linear_b.weight [n*C, C],
+    linear_out.weight [C, n*C]."""
+    if mask is None:
+        mask = x.new_ones(x.shape[:-1])
+    xn = layer_norm(x, p["layer_norm.weight"], p["layer_norm.bias"])
+    a = linear(xn, p["swiglu.linear_a.weight"])
+    b = linear(xn, p["swiglu.linear_b.weight"])
+    h = torch.nn.functional.silu(a) * b
+    return linear(h, p["linear_out.weight"]) * mask.to(x.dtype).unsqueeze(-1)
+
+
+def pair_block(z, pair_mask, p, no_heads: int, row_chunk: int | None = None, mask_trans: bool = True):
+    """PairBlock.forward in eval mode (base_blocks.py:408-480): the pair stack, then
+    z + pair_transition(z, mask = pair_mask if _mask_trans else None).  ``p`` also holds the
+    transition under the prefix pair_transition."""
+    z = pair_stack_block(z, pair_mask, p, no_heads, row_chunk=row_chunk)
+    return z + transition_update(z, pair_mask if mask_trans else None, _sub(p, "pair_transition."))
+
+
+def make_transition_params(gen, c_in: int, n: int):
+    def lin(o, i):
+        return torch.randn(o, i, generator=gen) / math.sqrt(i)
+
+    return {
+        "layer_norm.weight": 1.0 + 0.1 * torch.randn(c_in, generator=gen),
+        "layer_norm.bias": 0.1 * torch.randn(c_in, generator=gen),
+        "swiglu.linear_a.weight": lin(n * c_in, c_in),
+        "swiglu.linear_b.weight": lin(n * c_in, c_in),
+        "linear_out.weight": lin(c_in, n * c_in),
+    }
+
+
+# --------------------------------------------------------------------------
 # the same two updates restricted to a few output positions (for sizes at which
 # the full fp32 evaluation does not finish in seconds); 3-D inputs only
 # --------------------------------------------------------------------------

@@ -1,0 +1,148 @@
+"""Parity of the pair-transition kernel (SwiGLUTransition module -> C ABI -> HIP) and of the
+whole PairBlock with the CPU oracle, on the same seeded inputs and weights.
+
+bf16: the three checks of test_gpu_parity.py (max-norm 2e-2, rms 5e-3, at most 1.5x the rms
+error of the oracle's own operations executed in bfloat16).  fp32: max-abs 1e-4."""
+import pytest
+import torch
+
+from gpu_util import lib, report  # noqa: F401
+from oracle import pairstack_oracle as orc
+
+import of3pair
+from of3pair import functional as F3
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+REL = 2e-2
+
+
+def _check(name, got, want, rms_rel=5e-3, bf16_ref=None):
+    got = got.float().cpu()
+    want = want.float()
+    rms = float(want.pow(2).mean().sqrt())
+    report(name, got, want, atol=REL * float(want.abs().max()), rtol=0.0)
+    erms = float((got - want).pow(2).mean().sqrt())
+    assert erms <= rms_rel * rms, "%s: rms error %.3g vs rms %.3g" % (name, erms, rms)
+    if bf16_ref is not None:
+        floor = float((bf16_ref.float() - want).pow(2).mean().sqrt())
+        assert erms <= 1.5 * floor, "%s: rms error %.3g above the bf16 reference path's %.3g" % (name, erms, floor)
+
+
+def _round(p):
+    return {k: orc.round_bf16(v) for k, v in p.items()}
+
+
+def _bf16(p):
+    return {k: v.to(torch.bfloat16) for k, v in p.items()}
+
+
+def _module(c, n_mult, p, dtype):
+    m = of3pair.SwiGLUTransition(c, n_mult)
+    m.load_state_dict(p, strict=True)
+    return m.to(DEV).to(dtype).eval()
+
+
+# N covers: one partial wave (5), partial tile with idle waves (100), exactly one tile (256),
+# one full + one ragged tile (300), several tiles per work-group at B*N*tiles > 256 CUs (40 x 2)
+@pytest.mark.parametrize("c,n_mult,n,batch", [
+    (128, 4, 5, ()), (128, 4, 100, (2,)), (128, 4, 256, ()), (128, 4, 300, ()), (128, 2, 64, (1, 3)),
+    (64, 2, 96, ()), (64, 4, 40, (2,)), (128, 4, 40, (2, 4)),
+])
+def test_transition_module(c, n_mult, n, batch):
+    lib()
+    gen = torch.Generator().manual_seed(300 + n + c)
+    p = _round(orc.make_transition_params(gen, c, n_mult))
+    x = orc.round_bf16(orc.make_pair_input(11, batch, n, c))
+    mask = (torch.rand(*batch, n, n, generator=gen) > 0.2).float()
+    m = _module(c, n_mult, p, torch.bfloat16)
+    print("transition module", c, n_mult, n, batch, flush=True)
+    xg = x.to(DEV).to(torch.bfloat16)
+    got = m(xg, mask=mask.to(DEV), chunk_size=4)
+    want = orc.transition_update(x, mask, p)
+    floor = orc.transition_update(x.to(torch.bfloat16), mask.to(torch.bfloat16), _bf16(p))
+    _check("transition update", got, want, bf16_ref=floor)
+    assert torch.equal(xg.float().cpu(), x), "out-of-place call must not touch x"
+    masked = got.float().cpu()[mask == 0]
+    assert masked.numel() == 0 or float(masked.abs().max()) == 0.0, "masked positions must be exactly zero"
+    # x + update, in place
+    res = m(xg, mask=mask.to(DEV), _add_residual=True, _inplace=True)
+    assert res.data_ptr() == xg.data_ptr()
+    _check("transition x+update", res, x + want, rms_rel=4e-3)
+
+
+def test_transition_no_mask_and_transposed_view():
+    lib()
+    gen = torch.Generator().manual_seed(17)
+    p = _round(orc.make_transition_params(gen, 128, 4))
+    x = orc.round_bf16(orc.make_pair_input(12, (2,), 72, 128))
+    m = _module(128, 4, p, torch.bfloat16)
+    xg = x.to(DEV).to(torch.bfloat16)
+    want = orc.transition_update(x, None, p)
+    _check("transition maskless", m(xg), want)
+    got_t = m(xg.transpose(-2, -3))
+    _check("transition on transposed view", got_t.transpose(-2, -3), want)
+    assert got_t.stride() == xg.transpose(-2, -3).stride()
+
+
+def test_transition_deterministic_and_side_stream():
+    lib()
+    gen = torch.Generator().manual_seed(18)
+    p = _round(orc.make_transition_params(gen, 128, 4))
+    x = orc.round_bf16(orc.make_pair_input(13, (), 130, 128)).to(DEV).to(torch.bfloat16)
+    m = _module(128, 4, p, torch.bfloat16)
+    a = m(x)
+    b = m(x)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        c = m(x)
+    s.synchronize()
+    torch.cuda.synchronize()
+    assert torch.equal(a, b) and torch.equal(a, c)
+
+
+@pytest.mark.parametrize("c,n_mult,n,batch", [(128, 4, 33, ()), (96, 2, 20, (2,)), (64, 4, 50, ())])
+def test_transition_fp32(c, n_mult, n, batch):
+    lib()
+    gen = torch.Generator().manual_seed(400 + n)
+    p = orc.make_transition_params(gen, c, n_mult)
+    x = orc.make_pair_input(14, batch, n, c)
+    mask = (torch.rand(*batch, n, n, generator=gen) > 0.2).float()
+    m = _module(c, n_mult, p, torch.float32)
+    got = m(x.to(DEV), mask=mask.to(DEV))
+    want = orc.transition_update(x, mask, p)
+    report("transition fp32", got.cpu(), want, atol=1e-4, rtol=0.0)
+    res = m(x.to(DEV), mask=None, _add_residual=True)
+    report("transition fp32 x+update", res.cpu(), x + orc.transition_update(x, None, p), atol=1e-4, rtol=0.0)
+
+
+def test_transition_rejects_unsupported():
+    lib()
+    x = torch.zeros(1, 8, 8, 32, device=DEV, dtype=torch.bfloat16)  # c_in = 32 has no bf16 kernel
+    w = torch.zeros(128, 32, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        F3.swiglu_transition(x, None, torch.ones(32, device=DEV), torch.zeros(32, device=DEV), w, w,
+                             torch.zeros(32, 128, device=DEV))
+
+
+@pytest.mark.parametrize("mask_trans", [True, False])
+def test_pair_block_with_transition(mask_trans):
+    """PairBlock = pair stack + z + pair_transition(z) against the oracle's pair_block."""
+    lib()
+    c, n = 128, 72
+    gen = torch.Generator().manual_seed(500)
+    p = _round(orc.make_block_params(501, c, c, 32, 4))
+    p.update({"pair_transition." + k: v for k, v in _round(orc.make_transition_params(gen, c, 4)).items()})
+    z = orc.round_bf16(orc.make_pair_input(15, (1,), n, c))
+    mask = orc.tail_padding_mask((1,), n, 9)
+    blk = of3pair.PairBlock(c, c, 32, 4, "swiglu", 4, 0.25, False, 1e9)
+    blk.load_state_dict(p, strict=True)
+    blk = blk.to(DEV).to(torch.bfloat16).eval()
+    zg = z.to(DEV).to(torch.bfloat16)
+    got = blk(zg, mask.to(DEV), chunk_size=None, inplace_safe=False, _mask_trans=mask_trans)
+    want = orc.pair_block(z, mask, p, 4, mask_trans=mask_trans)
+    _check("pair block", got, want, rms_rel=1e-2)
+    assert torch.equal(zg.float().cpu(), z), "inplace_safe=False must leave z intact"
+    got2 = blk(zg, mask.to(DEV), inplace_safe=True, _mask_trans=mask_trans)
+    assert torch.equal(got2, got)

@@ -197,3 +197,42 @@ def test_triattn_update_rows_equals_full(starting):
     part = orc.triattn_update_rows(x, mask, p, heads, rows, starting=starting)
     want = full[rows] if starting else full[:, rows].transpose(0, 1)
     assert (part - want).abs().max() < 1e-5
+
+
+# ---- pair transition ---------------------------------------------------------------------------
+def test_transition_matches_bruteforce():
+    gen = torch.Generator().manual_seed(31)
+    n, c, mult = 5, 8, 4
+    x = torch.randn(n, n, c, generator=gen)
+    mask = (torch.rand(n, n, generator=gen) > 0.3).float()
+    p = orc.make_transition_params(gen, c, mult)
+    got = orc.transition_update(x, mask, p).double().numpy()
+    assert np.abs(got - bf.transition_update(x, mask, p)).max() < FP32_TOL
+    got = orc.transition_update(x, None, p).double().numpy()
+    assert np.abs(got - bf.transition_update(x, None, p)).max() < FP32_TOL
+
+
+def test_transition_invariants():
+    gen = torch.Generator().manual_seed(32)
+    c, mult = 16, 2
+    x = torch.randn(3, 7, 7, c, generator=gen)
+    mask = (torch.rand(3, 7, 7, generator=gen) > 0.5).float()
+    p = orc.make_transition_params(gen, c, mult)
+    out = orc.transition_update(x, mask, p)
+    assert out.shape == x.shape
+    assert (out[mask == 0] == 0).all()                      # masked positions give exactly 0
+    q = dict(p)
+    q["linear_out.weight"] = torch.zeros_like(p["linear_out.weight"])   # the shipped "final" init
+    assert orc.transition_update(x, mask, q).abs().max() == 0
+    q = dict(p)
+    q["swiglu.linear_a.weight"] = torch.zeros_like(p["swiglu.linear_a.weight"])  # silu(0) = 0
+    assert orc.transition_update(x, mask, q).abs().max() == 0
+    # position-wise: permuting positions permutes the result
+    perm = torch.randperm(7, generator=gen)
+    assert torch.allclose(orc.transition_update(x[:, perm], mask[:, perm], p), out[:, perm], atol=1e-6)
+    # swiglu against the library's own gated form: silu(a) * b == a * sigmoid(a) * b
+    xn = orc.layer_norm(x, p["layer_norm.weight"], p["layer_norm.bias"])
+    a = orc.linear(xn, p["swiglu.linear_a.weight"])
+    b = orc.linear(xn, p["swiglu.linear_b.weight"])
+    want = orc.linear(a * torch.sigmoid(a) * b, p["linear_out.weight"]) * mask.unsqueeze(-1)
+    assert torch.allclose(out, want, atol=1e-6)
