@@ -10,13 +10,18 @@
 //    and then held in registers as MFMA B operands for the whole tile.
 //  * the hidden dimension is walked in tiles of 32 channels.  The weights of a hidden tile (32
 //    rows of Wa and of Wb, 32 columns of Wout) are shared by all waves and travel
-//    L2 -> LDS with direct-to-LDS loads through a 3-deep ring, two hidden tiles ahead (one
-//    vmcnt wait + one barrier per hidden tile); the ring runs on across tiles, the sequence of
-//    hidden tiles simply repeats.
+//    L2 -> LDS with direct-to-LDS loads, two hidden tiles ahead (one vmcnt wait + one barrier
+//    per hidden tile), through a 3-deep ring for Wa/Wb and a 4-deep one for Wout; the rings
+//    run on across tiles, the sequence of hidden tiles simply repeats.
 //  * per hidden tile: a^T, b^T = W{a,b}[32 x C] * xn^T (A from LDS, B from registers), then
 //    h = silu(a) * b in fp32, rounded to bf16, is already laid out as the B operand of the
 //    second product (a lane holds 16 consecutive hidden channels of its position), so
 //    out^T += Wout[C x 32] * h^T needs no data movement between the two GEMMs.
+//  * software pipeline: the SiLU arithmetic of hidden tile t-1 (vector ALU, two
+//    transcendentals per element) is interleaved, element by element, with the first
+//    product's MFMAs of tile t, and the second product of tile t-1 follows; a wave issues in
+//    order, so without this its matrix and vector phases (about equally long) add up instead
+//    of overlapping.  That is why Wout stays one step longer in LDS than Wa/Wb.
 //  * epilogue: mask and residual (the activations as loaded wait in the wave's LDS tile during
 //    the hidden loop) in the accumulator layout, transposed through that tile, whole rows
 //    stored, next tile's loads issued.
@@ -36,8 +41,9 @@ namespace {
 #define OF3_LDS_AS __attribute__((address_space(3)))
 
 constexpr int kWaves = 8;
-constexpr int kStages = 3;
-constexpr int kPD = kStages - 1;  // prefetch distance in hidden tiles
+constexpr int kStagesW = 3;  // Wa/Wb ring: a stage is read in its own step
+constexpr int kStagesO = 4;  // Wout ring: a stage is read in the step after its own
+constexpr int kPD = 2;       // prefetch distance in hidden tiles
 
 __device__ __forceinline__ void compiler_fence() { __asm__ volatile("" ::: "memory"); }
 template <int N>
@@ -46,8 +52,18 @@ __device__ __forceinline__ void wait_vmcnt() {  // vmcnt(N) only (gfx9 encoding,
   __builtin_amdgcn_s_waitcnt((N & 15) | 0x70 | 0xF00 | ((N >> 4) << 14));
 }
 
-// swizzle keys (see the reader patterns at their uses)
-__device__ __forceinline__ int key_w(int row) { return (row & 3) | ((row >> 2) & 4); }  // Wa / Wb tile rows
+// Swizzle keys.  A ds_read_b128 is served 16 lanes (256 bytes, all 64 banks) per cycle; the 16
+// lanes of an MFMA A-operand read hold rows {0..7, 16..23} or {8..15, 24..31} of a tile
+// (rowperm16) at one chunk index, so the key must spread those rows over one 256-byte window.
+template <int NCH>
+__device__ __forceinline__ int key_w(int row) {  // Wa / Wb tile rows of NCH chunks
+  return NCH == 16 ? (row & 7) | ((row >> 1) & 8)            // one row per window: 16 distinct keys
+                   : ((row >> 1) & 3) | ((row >> 2) & 4);    // two rows per window: 8 keys per row parity
+}
+template <int NCH>
+__device__ __forceinline__ int key_x(int pos) {  // wave-private activation tile, 32 positions of NCH chunks
+  return NCH == 16 ? pos & 15 : (pos >> 1) & 7;  // B-operand reads: 16 consecutive positions at one chunk index
+}
 __device__ __forceinline__ int key_o(int row) {                                         // Wout tile rows (64 B)
   return ((((row >> 4) ^ (row >> 1)) & 1) << 1) | (((row >> 2) ^ (row >> 1)) & 1);
 }
@@ -69,8 +85,9 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
   static_assert(LPT + NLD + ITERS < 64, "vmcnt budget");
 
   extern __shared__ u32x4_t lds[];
-  u32x4_t* ring = lds;                                         // [kStages][STAGE]
-  u32x4_t* mine = lds + kStages * STAGE + (threadIdx.x >> 6) * (ROWS * NCH);  // wave-private [32 pos][NCH]
+  u32x4_t* ring_w = lds;                                   // [kStagesW][2 * WSLOTS]
+  u32x4_t* ring_o = lds + kStagesW * 2 * WSLOTS;           // [kStagesO][OSLOTS]
+  u32x4_t* mine = ring_o + kStagesO * OSLOTS + (threadIdx.x >> 6) * (ROWS * NCH);  // wave-private [32 pos][NCH]
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -83,18 +100,20 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
   u32x4_t lb_pk = *reinterpret_cast<const u32x4_t*>(p.ln_b + 8 * rw_chunk);
 
   // ---- direct-to-LDS sources of this wave's LPT instructions (byte offsets inside hidden tile 0;
-  // a hidden tile further on adds a wave-uniform offset).  Instruction q covers ring slots
-  // 64q .. 64q+63 of the stage: first the Wa tile, then Wb, then Wout.
+  // a hidden tile further on adds a wave-uniform offset).  Instruction q covers slots
+  // 64q .. 64q+63 of the stage: first the Wa tile, then Wb (one ring), then Wout (the other).
   uint32_t dma_off[LPT];
   const char* dma_base[LPT];  // wave-uniform
   int dma_step[LPT], dma_slot[LPT];
+  bool dma_out[LPT];
 #pragma unroll
   for (int n = 0; n < LPT; ++n) {
     const int q = (LPT * wave + n) % DMA_TOTAL;
     const int t = 64 * q + lane;
-    dma_slot[n] = 64 * q;
-    if (64 * q < 2 * WSLOTS) {  // Wa or Wb: slot (row, c') holds chunk c' ^ key_w(row) of row `row` of the tile
-      const int tt = t % WSLOTS, row = tt / NCH, chunk = (tt % NCH) ^ key_w(row);
+    dma_out[n] = 64 * q >= 2 * WSLOTS;
+    dma_slot[n] = dma_out[n] ? 64 * q - 2 * WSLOTS : 64 * q;
+    if (!dma_out[n]) {  // Wa or Wb: slot (row, c') holds chunk c' ^ key_w(row) of row `row` of the tile
+      const int tt = t % WSLOTS, row = tt / NCH, chunk = (tt % NCH) ^ key_w<NCH>(row);
       dma_base[n] = reinterpret_cast<const char*>(64 * q < WSLOTS ? p.w_a : p.w_b);
       dma_step[n] = 32 * C * (int)sizeof(bf16_t);
       dma_off[n] = (uint32_t)((row * C + 8 * chunk) * sizeof(bf16_t));
@@ -105,27 +124,26 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
       dma_off[n] = (uint32_t)((row * p.HID + 8 * chunk) * sizeof(bf16_t));
     }
   }
-  auto issue_stage = [&](int ht, int buf) {
-    u32x4_t* dst = ring + buf * STAGE;
+  auto issue_stage = [&](int ht, int buf_w, int buf_o) {
 #pragma unroll
     for (int n = 0; n < LPT; ++n) {
       const char* src = dma_base[n] + (size_t)ht * dma_step[n] + dma_off[n];
-      __builtin_amdgcn_global_load_lds((const void OF3_GLOBAL_AS*)src, (void OF3_LDS_AS*)(dst + dma_slot[n]), 16, 0, 0);
+      u32x4_t* dst = (dma_out[n] ? ring_o + buf_o * OSLOTS : ring_w + buf_w * 2 * WSLOTS) + dma_slot[n];
+      __builtin_amdgcn_global_load_lds((const void OF3_GLOBAL_AS*)src, (void OF3_LDS_AS*)dst, 16, 0, 0);
     }
   };
 
   // ---- operand read slots
   const int arow = rowperm16(l32);  // A rows are dealt so that a lane ends with 16 consecutive output rows
-  // W{a,b}: chunk 2s+lh of row arow.  The key is below 8, so it permutes k-steps only inside
-  // groups of four: four slot registers, the group is a constant offset.
-  int wa_rd4[4];
+  // W{a,b}: chunk 2s+lh of row arow
+  int wa_rd[KS];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) wa_rd4[s] = arow * NCH + ((2 * s + lh) ^ key_w(arow));
+  for (int s = 0; s < KS; ++s) wa_rd[s] = arow * NCH + ((2 * s + lh) ^ key_w<NCH>(arow));
   // Wout: k-step s, lane-half lh <-> hidden 16*lh + 8*s + (0..7) = chunk 2*lh + s of row
   // 32*ct + arow; the key does not depend on ct.
   int wo_rd2[2];
 #pragma unroll
-  for (int s = 0; s < 2; ++s) wo_rd2[s] = 2 * WSLOTS + arow * 4 + ((2 * lh + s) ^ key_o(arow));
+  for (int s = 0; s < 2; ++s) wo_rd2[s] = arow * 4 + ((2 * lh + s) ^ key_o(arow));
 
   // ---- tile bookkeeping
   const int tiles_per_batch = N * tiles_per_row;
@@ -171,11 +189,12 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
   // land in buffers nobody reads again): the number of memory instructions between any two
   // points of the program is then fixed, which is what the waits below rely on.
   int issue_ht = 0;  // hidden tile of the next stage to request
-  int issue_buf = 0;
+  int issue_w = 0, issue_o = 0;
   auto issue_next = [&]() {
-    issue_stage(issue_ht, issue_buf);
+    issue_stage(issue_ht, issue_w, issue_o);
     issue_ht = issue_ht + 1 == NHT ? 0 : issue_ht + 1;
-    issue_buf = issue_buf + 1 == kStages ? 0 : issue_buf + 1;
+    issue_w = issue_w + 1 == kStagesW ? 0 : issue_w + 1;
+    issue_o = issue_o + 1 == kStagesO ? 0 : issue_o + 1;
   };
 #pragma unroll
   for (int s = 0; s < kPD; ++s) issue_next();
@@ -199,21 +218,21 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int pos = it * PPI + t_pp;
-      mine[pos * NCH + (t_chunk ^ (pos & 7 & (NCH - 1)))] = layer_norm_chunk<C>(raw[it], lw, lb);
+      mine[pos * NCH + (t_chunk ^ key_x<NCH>(pos))] = layer_norm_chunk<C>(raw[it], lw, lb);
     }
 #pragma unroll
-    for (int s = 0; s < KS; ++s) xb[s] = mine[t_l32 * NCH + ((2 * s + t_lh) ^ (t_l32 & 7 & (NCH - 1)))];
+    for (int s = 0; s < KS; ++s) xb[s] = mine[t_l32 * NCH + ((2 * s + t_lh) ^ key_x<NCH>(t_l32))];
     // the tile then keeps the activations as loaded: the residual of the epilogue
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int pos = it * PPI + t_pp;
-      mine[pos * NCH + (t_chunk ^ (pos & 7 & (NCH - 1)))] = raw[it];
+      mine[pos * NCH + (t_chunk ^ key_x<NCH>(pos))] = raw[it];
     }
     mtile = p.mask ? mval : 1.f;
   };
   prepare_tile();
 
-  int buf = 0;
+  int buf_w = 0, buf_o = 0;  // buffers of the stage the next step consumes
   for (int tl = 0; tl < my_tiles; ++tl) {
     const int tile_id = blockIdx.x + tl * gridDim.x;
     int j0;
@@ -222,86 +241,90 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
     f32x16_t oacc[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) oacc[ct] = zero16();
+    f32x16_t pa, pb;  // a^T, b^T of the previous hidden tile, waiting for their SiLU and second product
+    u32x4_t hb[2];    // h of that tile as bf16: lane-half lh, register v = hidden 16*lh + v
 
-    // One hidden tile.  KIND 0: any but the last two of a tile; 1: the last but one, which also
-    // issues the next tile's loads; 2: the last.
-    auto hidden_step = [&](int ht, auto kind_tag) {
-      constexpr int KIND = decltype(kind_tag)::value;
-      // Stage `step` must have landed.  Memory operations retire in issue order, so "at most
-      // n outstanding" means everything older than the newest n is complete.  Younger than
-      // the stage: the next stage and whatever else was issued since
-      // the request two steps ago: the next tile's NLD loads (issued in the last step but one
-      // of every tile) and the ITERS stores of the previous tile's epilogue.
-      if (KIND == 2) wait_vmcnt<LPT + NLD>();
-      else if (KIND == 0 && tl > 0 && ht == 0) wait_vmcnt<LPT + NLD + ITERS>();
-      else if (KIND == 0 && tl > 0 && ht == 1) wait_vmcnt<LPT + ITERS>();
-      else wait_vmcnt<LPT>();
-      __builtin_amdgcn_s_barrier();  // everybody's part of the stage is visible; stage step-1 is free
-      compiler_fence();
-      issue_next();                  // stage step+2 goes into the buffer of stage step-1
-      // next tile's activations, early enough to arrive under the last two hidden tiles (a
-      // dummy reload of this tile after the last one keeps the instruction count per tile fixed)
-      if (KIND == 1) load_tile(tl + 1 < my_tiles ? tile_id + gridDim.x : tile_id);
-      const u32x4_t* st = ring + buf * STAGE;
-      buf = buf + 1 == kStages ? 0 : buf + 1;
-
-      // ---- a^T, b^T: 32 hidden rows x this wave's 32 positions.  The 16 A operands (Wa k-steps
-      // 0..7, then Wb) pass through a four-deep register ring, four reads ahead of their MFMA;
-      // the source order below is the issue order (scheduling fences between the groups).
-      auto w_op = [&](int i) -> u32x4_t {
-        return st[(i < KS ? 0 : WSLOTS) + wa_rd4[i & 3] + 8 * ((i % KS) >> 2)];
-      };
-      auto o_op = [&](int i) -> u32x4_t { return st[wo_rd2[i / CT] + 128 * (i % CT)]; };  // s-major
-      f32x16_t acca = zero16(), accb = zero16();
-      u32x4_t aq[4];  // one ring for all 2*KS + 2*CT operands of the step
+    // element e of h = silu(a) * b from the previous hidden tile's a, b
+    auto silu_elem = [&](int e) {
+      const float h = pa[e] * fast_rcp(1.f + fast_exp2(-kLog2e * pa[e])) * pb[e];
+      pa[e] = h;
+      if (e & 1) hb[e >> 3][(e & 7) >> 1] = pack_bf16(pa[e - 1], h);
+    };
+    // out^T += Wout[:, previous hidden tile] * h^T, Wout from ring buffer `bo`
+    auto second_product = [&](const u32x4_t* so) {
+      u32x4_t oq[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) aq[i] = w_op(i);
-      __builtin_amdgcn_sched_barrier(0);
-      // silu(a) of one register quad, in place (needs a only: runs under the Wb MFMAs)
-      auto silu4 = [&](int g) {
-#pragma unroll
-        for (int v = 4 * g; v < 4 * g + 4; ++v) acca[v] = acca[v] * fast_rcp(1.f + fast_exp2(-kLog2e * acca[v]));
-      };
-#pragma unroll
-      for (int i = 0; i < 2 * KS; ++i) {
-        if (i < KS) acca = mfma_32x32x16(aq[i & 3], xb[i], acca);
-        else accb = mfma_32x32x16(aq[i & 3], xb[i - KS], accb);
-        if (i + 4 < 2 * KS) aq[i & 3] = w_op(i + 4);
-        else aq[i & 3] = o_op(i + 4 - 2 * KS);
-        // quads of silu(a) once a is final and two Wb MFMAs cover its latency
-        const int g = i - (KS + 2);
-        if (g >= 0 && g < 4) silu4(g);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if (KS + 2 + 4 > 2 * KS) {  // narrow channel counts: the quads that did not fit above
-#pragma unroll
-        for (int g = 2 * KS - (KS + 2); g < 4; ++g) silu4(g);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      // ---- h = silu(a) * b, rounded to bf16: lane-half lh, register v = hidden 16*lh + v; the
-      // second half is computed under the first four MFMAs of out^T += Wout[:, hidden tile] * h^T
-      u32x4_t hb[2];
-      auto make_h = [&](int s2) {
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          const int v = 8 * s2 + 2 * w;
-          hb[s2][w] = pack_bf16(acca[v] * accb[v], acca[v + 1] * accb[v + 1]);
-        }
-      };
-      make_h(0);
+      for (int i = 0; i < 4 && i < 2 * CT; ++i) oq[i] = so[wo_rd2[i / CT] + 128 * (i % CT)];
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < 2 * CT; ++i) {
-        const int ct = i % CT, s2 = i / CT;
-        oacc[ct] = mfma_32x32x16(aq[(2 * KS + i) & 3], hb[s2], oacc[ct]);
-        if (i + 4 < 2 * CT) aq[(2 * KS + i) & 3] = o_op(i + 4);
-        if (i == 0) make_h(1);
+        oacc[i % CT] = mfma_32x32x16(oq[i & 3], hb[i / CT], oacc[i % CT]);
+        if (i + 4 < 2 * CT) oq[i & 3] = so[wo_rd2[(i + 4) / CT] + 128 * ((i + 4) % CT)];
         __builtin_amdgcn_sched_barrier(0);
       }
     };
-    for (int ht = 0; ht < NHT - 2; ++ht) hidden_step(ht, std::integral_constant<int, 0>{});
-    hidden_step(NHT - 2, std::integral_constant<int, 1>{});
-    hidden_step(NHT - 1, std::integral_constant<int, 2>{});
+
+    // One hidden tile.  KIND 0: the first of a tile (nothing to finish from the previous
+    // one); 1: any other but the last two; 2: the last but one, which also issues the next
+    // tile's loads; 3: the last.
+    auto hidden_step = [&](int ht, auto kind_tag) {
+      constexpr int KIND = decltype(kind_tag)::value;
+      // Stage `ht` must have landed.  Memory operations retire in issue order, so "at most
+      // n outstanding" means everything older than the newest n is complete.  Younger than
+      // the stage: the next stage and whatever else was issued since the request two steps
+      // ago: the next tile's NLD loads (issued in the last step but one of every tile) and
+      // the ITERS stores of the previous tile's epilogue.
+      if (KIND == 3) wait_vmcnt<LPT + NLD>();
+      else if (KIND == 0 && tl > 0) wait_vmcnt<LPT + NLD + ITERS>();
+      else if (KIND == 1 && tl > 0 && ht == 1) wait_vmcnt<LPT + ITERS>();
+      else wait_vmcnt<LPT>();
+      __builtin_amdgcn_s_barrier();  // everybody's part of the stage is visible; the buffers that
+      compiler_fence();              // the stage two ahead goes into are no longer read
+      issue_next();
+      // next tile's activations, early enough to arrive under the last two hidden tiles (a
+      // dummy reload of this tile after the last one keeps the instruction count per tile fixed)
+      if (KIND == 2) load_tile(tl + 1 < my_tiles ? tile_id + gridDim.x : tile_id);
+      const u32x4_t* sw = ring_w + buf_w * 2 * WSLOTS;
+      const u32x4_t* so_prev = ring_o + (buf_o == 0 ? kStagesO - 1 : buf_o - 1) * OSLOTS;
+      buf_w = buf_w + 1 == kStagesW ? 0 : buf_w + 1;
+      buf_o = buf_o + 1 == kStagesO ? 0 : buf_o + 1;
+
+      // ---- a^T, b^T of this hidden tile (32 hidden rows x this wave's 32 positions): the
+      // 2*KS A operands (Wa k-steps, then Wb) pass through a four-deep register ring, four
+      // reads ahead of their MFMA; each MFMA is followed by the SiLU arithmetic of 16/(2*KS)
+      // elements of the previous tile.  The source order is the issue order (scheduling fences).
+      constexpr int EPS = 16 / (2 * KS);
+      auto w_op = [&](int i) -> u32x4_t {
+        return sw[(i < KS ? 0 : WSLOTS) + wa_rd[i % KS]];
+      };
+      f32x16_t ca = zero16(), cb = zero16();
+      u32x4_t aq[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) aq[i] = w_op(i);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 2 * KS; ++i) {
+        if (i < KS) ca = mfma_32x32x16(aq[i & 3], xb[i], ca);
+        else cb = mfma_32x32x16(aq[i & 3], xb[i - KS], cb);
+        if (i + 4 < 2 * KS) aq[i & 3] = w_op(i + 4);
+        if (KIND != 0) {
+#pragma unroll
+          for (int e = EPS * i; e < EPS * (i + 1); ++e) silu_elem(e);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (KIND != 0) second_product(so_prev);
+      pa = ca;
+      pb = cb;
+    };
+    hidden_step(0, std::integral_constant<int, 0>{});
+    for (int ht = 1; ht < NHT - 2; ++ht) hidden_step(ht, std::integral_constant<int, 1>{});
+    hidden_step(NHT - 2, std::integral_constant<int, 2>{});
+    hidden_step(NHT - 1, std::integral_constant<int, 3>{});
+    // the last hidden tile's SiLU and second product (its Wout stays valid until two barriers on)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) silu_elem(e);
+    second_product(ring_o + (buf_o == 0 ? kStagesO - 1 : buf_o - 1) * OSLOTS);
 
     char* orow = reinterpret_cast<char*>(p.out + row_off);
     // ---- epilogue: mask, residual (read from the wave's LDS tile in the accumulator layout and
@@ -312,8 +335,8 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
       const int chunk = 4 * ct + 2 * e_lh;  // channels 32*ct + 16*lh + (0..15)
-      const int s0 = e_l32 * NCH + (chunk ^ (e_l32 & 7 & (NCH - 1)));
-      const int s1 = e_l32 * NCH + ((chunk + 1) ^ (e_l32 & 7 & (NCH - 1)));
+      const int s0 = e_l32 * NCH + (chunk ^ key_x<NCH>(e_l32));
+      const int s1 = e_l32 * NCH + ((chunk + 1) ^ key_x<NCH>(e_l32));
       float r0[8], r1[8];
       unpack8(mine[s0], r0);
       unpack8(mine[s1], r1);
@@ -333,7 +356,7 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int pos = it * PPI + e_pp;
-      outv[it] = mine[pos * NCH + (e_chunk ^ (pos & 7 & (NCH - 1)))];
+      outv[it] = mine[pos * NCH + (e_chunk ^ key_x<NCH>(pos))];
     }
     // The next tile is prepared before this tile's stores are issued: direct-to-LDS loads in
     // flight make the compiler wait for every outstanding memory operation at the first use
@@ -354,8 +377,7 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
 template <int C>
 hipError_t launch(const TransitionArgs& a, hipStream_t stream) {
   auto kern = transition_kernel<C>;
-  constexpr int stage = 2 * 32 * (C / 8) + C * 4;
-  constexpr int smem = (kStages * stage + kWaves * 32 * (C / 8)) * 16;
+  constexpr int smem = (kStagesW * 2 * 32 * (C / 8) + kStagesO * C * 4 + kWaves * 32 * (C / 8)) * 16;
   static int cus = 0;
   if (cus == 0) {
     int dev = 0, n = 0;
