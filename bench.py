@@ -16,6 +16,8 @@ Besides the whole-block time the line carries
                 bounds it (MFMA for the contraction and the attention core, HBM for the
                 LayerNorm/projection passes; algorithmic bytes per launch are listed in
                 KERNEL_MODEL below);
+                the entry "pair_transition" is the SwiGLU transition that follows the block in
+                every PairBlock: timed right after the block's kernels, not part of `value`;
   cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path)
                 timed once on the host cores for the same workload.
 """
@@ -43,6 +45,8 @@ CAL_BYTES = 256 << 20      # size of the calibration copy
 # profiles/.  None for any other workload.
 MEASURED_TRAFFIC = {("trimul_contract", 768): 539774737}
 
+TRANSITION_N = 4           # hidden width factor of the pair transition (AF3 configuration)
+
 METRIC = "ms per Pairformer pair-stack block at N=768 bf16; % of MFMA peak & HBM GB/s"
 
 
@@ -63,6 +67,8 @@ def kernel_model(B, N, C, CH, H, D):
         "triattn_flash": {"bound": "mfma", "flops": 4 * B * N ** 3 * H * D},
         # reads o and x, writes out
         "triattn_out": {"bound": "hbm", "bytes": B * N * N * hd * 2 + 2 * U},
+        # the transition after the block (n = 4): three C x 4C products per position
+        "pair_transition": {"bound": "mfma", "flops": 6 * B * N * N * C * (TRANSITION_N * C)},
     }
 
 
@@ -178,8 +184,14 @@ def main():
                 w("mha.linear_o.weight"), B, N, C, H, D, 1, s))),
         ]
 
+    tgen = torch.Generator().manual_seed(7)
+    tp = {k_: v.to(dev).to(bf).contiguous() for k_, v in orc.make_transition_params(tgen, C, TRANSITION_N).items()}
+    transition = [("pair_transition", lambda: ck(lib.of3_transition_fwd(
+        P(zz), z_fwd, P(mask), m_fwd, P(tp["layer_norm.weight"]), P(tp["layer_norm.bias"]),
+        P(tp["swiglu.linear_a.weight"]), P(tp["swiglu.linear_b.weight"]), P(tp["linear_out.weight"]), P(zz),
+        B, N, C, TRANSITION_N * C, 1, _lib.OF3_DTYPE_BF16, s)))]
     launches = (trimul("tri_mul_out.", 1) + trimul("tri_mul_in.", 0)
-                + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr))
+                + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr) + transition)
     for _ in range(max(args.warmup, 1)):
         for _, fn in launches:
             fn()

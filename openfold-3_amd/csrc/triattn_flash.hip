@@ -118,13 +118,13 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
 
   // ---- direct-to-LDS sources.  LDS slot of an instruction = its base + lane.
   // bias slice: instruction n of wave w fills slots 64*(2w+n)..+63; slot t holds chunk
-  // (t & 7) ^ (q & 7) of query q = t >> 3 (128-byte rows of 32 keys)
+  // (t & 7) ^ ((q >> 1) & 7) of query q = t >> 3 (128-byte rows of 32 keys)
   // (byte offsets from wave-uniform bases, so that the loads use scalar base + 32-bit lane offset)
   uint32_t tb_off[kTbLoads];
 #pragma unroll
   for (int n = 0; n < kTbLoads; ++n) {
     const int t = 64 * (kTbLoads * wave + n) + lane;
-    const int qloc = t >> 3, chunk = (t & 7) ^ (qloc & 7);
+    const int qloc = t >> 3, chunk = (t & 7) ^ ((qloc >> 1) & 7);
     int qrow = q0 + qloc;
     qrow = qrow < N ? qrow : N - 1;
     tb_off[n] = (uint32_t)(((size_t)qrow * Jp + 4 * chunk) * sizeof(float));
@@ -177,10 +177,12 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
     const int vr = krow & (D - 1);
     v_rd[s2] = KSLOTS + vr * 4 + ((2 * lh + s2) ^ key4(vr));
   }
-  // bias slot this lane reads for tile rq, chunk c: rq*256 + l32*8 + ((4*lh + c) ^ (l32 & 7))
+  // bias slot this lane reads for tile rq, chunk c: rq*256 + l32*8 + ((4*lh + c) ^ key), key =
+  // (l32 >> 1) & 7: the 16 lanes of one read phase hold 16 consecutive queries, two 128-byte
+  // rows per 256-byte bank window, so queries of equal parity need distinct keys
   int tb_rd[4];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) tb_rd[c] = l32 * 8 + ((4 * lh + c) ^ (l32 & 7));
+  for (int c = 0; c < 4; ++c) tb_rd[c] = l32 * 8 + ((4 * lh + c) ^ ((l32 >> 1) & 7));
 
   float m_run[kRQ], l_run[kRQ];
   f32x16_t oacc[kRQ];

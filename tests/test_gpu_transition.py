@@ -117,6 +117,30 @@ def test_transition_fp32(c, n_mult, n, batch):
     report("transition fp32 x+update", res.cpu(), x + orc.transition_update(x, None, p), atol=1e-4, rtol=0.0)
 
 
+@pytest.mark.parametrize("n,rows", [(768, [0, 1, 383, 767]), (2048, [0, 1023, 2047])])
+def test_transition_full_size_at_sampled_rows(n, rows):
+    """BASELINE sizes (N = 768 and 2048, c_z = 128, n = 4): the update is position-wise, so the
+    oracle evaluates whole rows of the same input; the rest of the output is checked through
+    a size-independent property (masked positions exactly zero, unmasked ones finite)."""
+    lib()
+    gen = torch.Generator().manual_seed(600 + n)
+    p = _round(orc.make_transition_params(gen, 128, 4))
+    m = _module(128, 4, p, torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(n)
+    xg = torch.randn(1, n, n, 128, device=DEV, generator=g).to(torch.bfloat16)
+    mask = (torch.rand(1, n, n, device=DEV, generator=g) > 0.1).float()
+    print("transition full size", n, flush=True)
+    got = m(xg, mask=mask)
+    assert torch.isfinite(got).all()
+    assert float(got[mask == 0].float().abs().max()) == 0.0
+    x_rows = xg[0, rows].float().cpu()
+    want = orc.transition_update(x_rows, mask[0, rows].cpu(), p)
+    _check("transition rows at N=%d" % n, got[0, rows], want)
+    res = m(xg, mask=mask, _add_residual=True, _inplace=True)
+    assert res.data_ptr() == xg.data_ptr()
+    _check("transition x+update rows at N=%d" % n, res[0, rows], x_rows + want, rms_rel=4e-3)
+
+
 def test_transition_rejects_unsupported():
     lib()
     x = torch.zeros(1, 8, 8, 32, device=DEV, dtype=torch.bfloat16)  # c_in = 32 has no bf16 kernel
