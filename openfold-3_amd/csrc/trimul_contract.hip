@@ -220,8 +220,19 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
   for (int t_local = 0; t_local < my_tiles; ++t_local) {
     for (int kb = 0; kb < nk; ++kb) {
       const u32x4_t* cur = lds + cur_buf * STAGE;
+      // The second k-step's fragments are requested right after the first MFMA: that MFMA
+      // carries the wait for a0/b0 (with direct-to-LDS loads in flight every LDS wait the
+      // compiler emits is a wait for all outstanding reads), so the new reads travel under the
+      // remaining MFMAs instead of being waited for at once.
+      acc[0][0] = mfma_32x32x16(a0[0], b0[0], acc[0][0]);
+      __builtin_amdgcn_sched_barrier(0);
       fetch(cur, 1, a1, b1);
-      mma(a0, b0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < TN; ++nt)
+          if (mt + nt > 0) acc[mt][nt] = mfma_32x32x16(a0[mt], b0[nt], acc[mt][nt]);
       __builtin_amdgcn_sched_barrier(0);
 
       // This wave holds all of stage s in registers.  Stages s+1..s+3 are in flight and
