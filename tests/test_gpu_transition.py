@@ -170,3 +170,46 @@ def test_pair_block_with_transition(mask_trans):
     assert torch.equal(zg.float().cpu(), z), "inplace_safe=False must leave z intact"
     got2 = blk(zg, mask.to(DEV), inplace_safe=True, _mask_trans=mask_trans)
     assert torch.equal(got2, got)
+
+
+def test_template_pair_blocks_with_transition():
+    """Template stack shape (c_t = 64, 4 heads x 16, transition n = 2, template_module.py:96-116):
+    two full PairBlocks over 3 templates folded into the batch, each template with its own
+    padded tail."""
+    lib()
+    n, t, c = 200, 3, 64
+    gen = torch.Generator().manual_seed(31)
+    plist = []
+    for seed in (20, 21):
+        p = _round(orc.make_block_params(seed, c, c, 16, 4))
+        p.update({"pair_transition." + k: v for k, v in _round(orc.make_transition_params(gen, c, 2)).items()})
+        plist.append(p)
+    z = orc.round_bf16(orc.make_pair_input(16, (t,), n, c))
+    mask = orc.tail_padding_mask((t,), n, torch.tensor([0, 13, 40]))
+    zg = z.to(DEV).to(torch.bfloat16)
+    want = z
+    for p in plist:
+        blk = of3pair.PairBlock(c, c, 16, 4, "swiglu", 2, 0.25, False, 1e9)
+        blk.load_state_dict(p, strict=True)
+        blk = blk.to(DEV).to(torch.bfloat16).eval()
+        zg = blk(zg, mask.to(DEV), inplace_safe=True)
+        want = orc.pair_block(want, mask, p, 4, row_chunk=64)
+    _check("template pair blocks", zg, want, rms_rel=1.5e-2)
+
+
+def test_pair_block_config2_n384_padded():
+    """BASELINE config 2 shape through the whole PairBlock (pair stack + transition, n = 4)."""
+    lib()
+    import math
+    n, c = 384, 128
+    gen = torch.Generator().manual_seed(41)
+    p = _round(orc.make_block_params(0, c, c, 32, 4))
+    p.update({"pair_transition." + k: v for k, v in _round(orc.make_transition_params(gen, c, 4)).items()})
+    z = orc.round_bf16(orc.make_pair_input(1, (1,), n, c))
+    mask = orc.tail_padding_mask((1,), n, n - math.ceil(0.9 * n))
+    blk = of3pair.PairBlock(c, c, 32, 4, "swiglu", 4, 0.25, False, 1e9)
+    blk.load_state_dict(p, strict=True)
+    blk = blk.to(DEV).to(torch.bfloat16).eval()
+    got = blk(z.to(DEV).to(torch.bfloat16), mask.to(DEV))
+    want = orc.pair_block(z, mask, p, 4, row_chunk=64)
+    _check("pair block n=384", got, want, rms_rel=1e-2)
