@@ -43,7 +43,7 @@ CAL_BYTES = 256 << 20      # size of the calibration copy
 # counter passes of this command (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE), each
 # scaled by what the same counter reads for the calibration copy; the summaries are kept in
 # profiles/.  None for any other workload.
-MEASURED_TRAFFIC = {("trimul_contract", 768): 539774737}
+MEASURED_TRAFFIC = {("trimul_contract", 768): 539701909}
 
 TRANSITION_N = 4           # hidden width factor of the pair transition (AF3 configuration)
 
