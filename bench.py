@@ -16,8 +16,10 @@ Besides the whole-block time the line carries
                 bounds it (MFMA for the contraction and the attention core, HBM for the
                 LayerNorm/projection passes; algorithmic bytes per launch are listed in
                 KERNEL_MODEL below);
-                the entry "pair_transition" is the SwiGLU transition that follows the block in
-                every PairBlock: timed right after the block's kernels, not part of `value`;
+                the entries "pair_transition" (the SwiGLU transition that follows the block in
+                every PairBlock) and "pair_bias_proj" (the 16-head pair bias the single-representation
+                attention of a PairFormerBlock takes from z) are timed right after the block's
+                kernels and are not part of `value`;
   cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path)
                 timed once on the host cores for the same workload.
 """
@@ -46,6 +48,7 @@ CAL_BYTES = 256 << 20      # size of the calibration copy
 MEASURED_TRAFFIC = {("trimul_contract", 768): 539701909}
 
 TRANSITION_N = 4           # hidden width factor of the pair transition (AF3 configuration)
+PAIR_BIAS_HEADS = 16       # heads of the pairformer's single-representation attention
 
 METRIC = "ms per Pairformer pair-stack block at N=768 bf16; % of MFMA peak & HBM GB/s"
 
@@ -69,6 +72,8 @@ def kernel_model(B, N, C, CH, H, D):
         "triattn_out": {"bound": "hbm", "bytes": B * N * N * hd * 2 + 2 * U},
         # the transition after the block (n = 4): three C x 4C products per position
         "pair_transition": {"bound": "mfma", "flops": 6 * B * N * N * C * (TRANSITION_N * C)},
+        # reads z, writes the [PAIR_BIAS_HEADS, N, N] bias
+        "pair_bias_proj": {"bound": "hbm", "bytes": U + B * PAIR_BIAS_HEADS * N * N * 2},
     }
 
 
@@ -190,8 +195,14 @@ def main():
         P(zz), z_fwd, P(mask), m_fwd, P(tp["layer_norm.weight"]), P(tp["layer_norm.bias"]),
         P(tp["swiglu.linear_a.weight"]), P(tp["swiglu.linear_b.weight"]), P(tp["linear_out.weight"]), P(zz),
         B, N, C, TRANSITION_N * C, 1, _lib.OF3_DTYPE_BF16, s)))]
+    bp = {k_: v.to(dev).to(bf).contiguous() for k_, v in orc.make_pair_bias_params(tgen, C, PAIR_BIAS_HEADS).items()}
+    bias_out = torch.empty(B, PAIR_BIAS_HEADS, N, N, dtype=bf, device=dev)
+    pair_bias = [("pair_bias_proj", lambda: ck(lib.of3_pair_bias_fwd(
+        P(zz), z_fwd, P(bp["layer_norm_z.weight"]), P(bp["layer_norm_z.bias"]), P(bp["linear_z.weight"]),
+        P(bias_out), B, N, C, PAIR_BIAS_HEADS, _lib.OF3_DTYPE_BF16, s)))]
     launches = (trimul("tri_mul_out.", 1) + trimul("tri_mul_in.", 0)
-                + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr) + transition)
+                + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr) + transition
+                + pair_bias)
     for _ in range(max(args.warmup, 1)):
         for _, fn in launches:
             fn()

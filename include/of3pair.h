@@ -27,6 +27,8 @@
  *       :225-271  SwiGLUTransition.forward (LayerNorm, SwiGLU of
  *                 openfold3/core/model/primitives/activations.py:33-61,
  *                 linear_out, mask)                             -> of3_transition_fwd
+ *   openfold3/core/model/layers/attention_pair_bias.py
+ *       :151-161  _prep_bias: layer_norm_z, linear_z, permute   -> of3_pair_bias_fwd
  *   openfold3/core/model/latent/base_blocks.py
  *       :329-335  "z = z + update" after each module            -> add_residual = 1
  *       :470-478  "z = z + pair_transition(z, mask)"            -> of3_transition_fwd, add_residual = 1
@@ -45,7 +47,7 @@
  *
  * dtype: OF3_DTYPE_BF16 selects the MFMA kernels described above.  OF3_DTYPE_F32 (the
  * reference's default inference precision) is served by of3_trimul_fwd / of3_triattn_fwd /
- * of3_transition_fwd only: every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
+ * of3_transition_fwd / of3_pair_bias_fwd only: every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
  * element counts, any N, C and CH <= 256, H*D <= 256 with D in {16, 32, 64}; plain fp32
  * arithmetic in the reference's order of operations (no MFMA, not the fast path).  The
  * stage entry points are bf16 only.
@@ -152,6 +154,15 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
                        const void* ln_w, const void* ln_b, const void* w_a, const void* w_b, const void* w_out,
                        void* out, int64_t B, int64_t N, int64_t C, int64_t HID, int add_residual, int dtype,
                        void* stream);
+
+/* ---- pair-bias projection ------------------------------------------------------------- */
+
+/* out[b][h][i][j] = sum_c LN(z[b,i,j,:])[c] * w[h][c]: the pair bias the single-representation
+ * attention adds to its logits (layer_norm_z, linear_z without bias, permute_final_dims(z, [2,0,1])).
+ * out is contiguous [B][H][N][N] in z's dtype; ln_b may be null (a LayerNorm created without
+ * offset); w is [H][C].  No workspace.  bf16: C in {64, 128}, H <= 32; fp32: C <= 256, H <= 64. */
+int of3_pair_bias_fwd(const void* z, const int64_t z_strides[3], const void* ln_w, const void* ln_b, const void* w,
+                      void* out, int64_t B, int64_t N, int64_t C, int64_t H, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -98,6 +98,16 @@ struct TransitionArgs {
 };
 hipError_t transition_launch(const TransitionArgs& args, int C, hipStream_t stream);
 
+struct PairBiasArgs {
+  const bf16_t* z;            // pair tensor, z_view addressing
+  PairView z_view;
+  const bf16_t *ln_w, *ln_b;  // [C]; ln_b may be null (LayerNorm without offset)
+  const bf16_t* w;            // [H][C]
+  bf16_t* out;                // [B][H][N][N] contiguous
+  int B, N, H;
+};
+hipError_t pair_bias_launch(const PairBiasArgs& args, int C, hipStream_t stream);
+
 // ---- fp32 path (pair_f32.hip): whole updates, any N, C and C_hidden <= 256, head width 16/32/64
 struct TrimulF32Args {
   const float* z;
@@ -135,5 +145,14 @@ struct TransitionF32Args {
   int B, N, C, HID, add_residual;
 };
 hipError_t transition_fwd_f32(const TransitionF32Args& args, hipStream_t stream);
+
+struct PairBiasF32Args {
+  const float* z;
+  PairView z_view;
+  const float *ln_w, *ln_b, *w;  // ln_b may be null
+  float* out;                    // [B][H][N][N]
+  int B, N, C, H;
+};
+hipError_t pair_bias_fwd_f32(const PairBiasF32Args& args, hipStream_t stream);
 
 }  // namespace of3

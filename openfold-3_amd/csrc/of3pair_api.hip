@@ -459,4 +459,42 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
   return e == hipSuccess ? OF3_OK : fail_hip(e);
 }
 
+int of3_pair_bias_fwd(const void* z, const int64_t z_strides[3], const void* ln_w, const void* ln_b, const void* w,
+                      void* out, int64_t B, int64_t N, int64_t C, int64_t H, int dtype, void* stream) {
+  if (B < 1 || N < 1 || N > (1 << 16) || H < 1 || !z || !ln_w || !w || !out) return OF3_EINVAL;
+  if (B * N * ((N + 7) / 8) > 0x7fffffffll) return OF3_EINVAL;
+  if (dtype == OF3_DTYPE_F32) {
+    if (C < 1 || C > 256 || H > 64 || !f32_strides_ok(z_strides)) return OF3_EINVAL;
+    if (!aligned4(z) || !aligned4(ln_w) || !aligned4(ln_b) || !aligned4(w) || !aligned4(out)) return OF3_EINVAL;
+    of3::PairBiasF32Args a;
+    a.z = static_cast<const float*>(z);
+    a.z_view = view(z_strides, false);
+    a.ln_w = static_cast<const float*>(ln_w);
+    a.ln_b = static_cast<const float*>(ln_b);
+    a.w = static_cast<const float*>(w);
+    a.out = static_cast<float*>(out);
+    a.B = (int)B;
+    a.N = (int)N;
+    a.C = (int)C;
+    a.H = (int)H;
+    hipError_t e = of3::pair_bias_fwd_f32(a, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? OF3_OK : fail_hip(e);
+  }
+  if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
+  if (!(C == 128 || C == 64) || H > 32 || !strides_ok(z_strides)) return OF3_EINVAL;
+  if (!aligned16(z) || !aligned16(ln_w) || !aligned16(ln_b) || !aligned16(w) || !aligned16(out)) return OF3_EINVAL;
+  of3::PairBiasArgs a;
+  a.z = bf(z);
+  a.z_view = view(z_strides, false);
+  a.ln_w = bf(ln_w);
+  a.ln_b = bf(ln_b);
+  a.w = bf(w);
+  a.out = bf(out);
+  a.B = (int)B;
+  a.N = (int)N;
+  a.H = (int)H;
+  hipError_t e = of3::pair_bias_launch(a, (int)C, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
 }  // extern "C"

@@ -4,6 +4,7 @@
 //   triangle multiplication   triangular_multiplicative_update.py:482-503, :71-97
 //   triangle attention        triangular_attention.py:102-167, attention.py:94-135,265-302
 //   pair transition           transition.py:225-271, activations.py:33-61
+//   pair-bias projection      attention_pair_bias.py:151-161
 // These kernels are written for exactness and generality (any N, C, C_hidden <= 256, head
 // width <= 64), with plain fp32 FMA arithmetic, full-precision expf and no MFMA; they are the
 // precision reference of the library on the GPU, not its fast path (that is the bf16 path).
@@ -348,6 +349,41 @@ __global__ __launch_bounds__(kThreads) void transition_f32(TransitionF32 p, int 
   }
 }
 
+// ---- pair-bias projection ---------------------------------------------------------------------
+struct PairBiasF32 {
+  const float* z;
+  PairView zv;
+  const float *ln_w, *ln_b, *w;
+  float* out;
+  int B, N, C, H;
+};
+
+// out[b][h][i][j] = LN(z[b,i,j,:]) . w[h,:] for kP positions of one row
+__global__ __launch_bounds__(kThreads) void pair_bias_f32(PairBiasF32 p, int groups) {
+  __shared__ float xn[kP][kMaxC];
+  __shared__ float zero_bias[kMaxC];
+  const int N = p.N, C = p.C, H = p.H;
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kP;
+  const float* lb = p.ln_b;
+  if (!lb) {
+    for (int c = threadIdx.x; c < C; c += kThreads) zero_bias[c] = 0.f;
+    __syncthreads();
+    lb = zero_bias;
+  }
+  layer_norm_rows(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.z + b * p.zv.stride_b + i * p.zv.stride_r + j * p.zv.stride_k : nullptr;
+      },
+      p.ln_w, lb, C, xn);
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * H; idx += kThreads) {
+    const int pos = idx % kP, h = idx / kP, j = j0 + pos;
+    if (j < N) p.out[(((size_t)b * H + h) * N + i) * N + j] = dot_row(xn[pos], p.w + (size_t)h * C, C);
+  }
+}
+
 }  // namespace
 
 hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
@@ -453,6 +489,25 @@ hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
   const int groups = (a.N + kP - 1) / kP;
   const long blocks = (long)a.B * a.N * groups;
   hipLaunchKernelGGL(transition_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  return hipGetLastError();
+}
+
+hipError_t pair_bias_fwd_f32(const PairBiasF32Args& a, hipStream_t stream) {
+  if (a.C > kMaxC) return hipErrorInvalidValue;
+  PairBiasF32 p;
+  p.z = a.z;
+  p.zv = a.z_view;
+  p.ln_w = a.ln_w;
+  p.ln_b = a.ln_b;
+  p.w = a.w;
+  p.out = a.out;
+  p.B = a.B;
+  p.N = a.N;
+  p.C = a.C;
+  p.H = a.H;
+  const int groups = (a.N + kP - 1) / kP;
+  const long blocks = (long)a.B * a.N * groups;
+  hipLaunchKernelGGL(pair_bias_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
   return hipGetLastError();
 }
 

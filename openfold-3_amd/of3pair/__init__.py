@@ -1,12 +1,12 @@
 """of3pair: MI355X-native kernels for the OpenFold3 Pairformer pair stack (triangle
 multiplicative updates, triangle attention and the pair transition) behind the reference's layer-module API."""
-from .layers import (SwiGLUTransition, TriangleAttention, TriangleAttentionEndingNode, TriangleAttentionStartingNode,
+from .layers import (PairBiasProjection, SwiGLUTransition, TriangleAttention, TriangleAttentionEndingNode, TriangleAttentionStartingNode,
                      TriangleMultiplicationIncoming, TriangleMultiplicationOutgoing,
                      TriangleMultiplicativeUpdate)
 from .pair_stack import PairBlock, PairStack
 
 __all__ = [
     "TriangleMultiplicativeUpdate", "TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming",
-    "TriangleAttention", "TriangleAttentionStartingNode", "TriangleAttentionEndingNode", "SwiGLUTransition",
+    "TriangleAttention", "TriangleAttentionStartingNode", "TriangleAttentionEndingNode", "SwiGLUTransition", "PairBiasProjection",
     "PairStack", "PairBlock",
 ]

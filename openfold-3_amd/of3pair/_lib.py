@@ -39,6 +39,7 @@ SIGNATURES = {
                         + [c_float, c_int, c_void_p, c_int64, c_int, c_void_p]),
     "of3_transition_fwd": (c_int, [c_void_p, _I64x3, c_void_p, _I64x3] + [c_void_p] * 6 + [c_int64] * 4
                            + [c_int, c_int, c_void_p]),
+    "of3_pair_bias_fwd": (c_int, [c_void_p, _I64x3] + [c_void_p] * 4 + [c_int64] * 4 + [c_int, c_void_p]),
 }
 
 _lib = None

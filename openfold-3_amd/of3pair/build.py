@@ -27,6 +27,7 @@ SOURCES = [
     "triattn_flash.hip",
     "triattn_out.hip",
     "transition.hip",
+    "pair_bias.hip",
     "pair_f32.hip",
 ]
 

@@ -187,3 +187,28 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
                          % (C, HID, x.dtype))
     _lib.check(st, "of3_transition_fwd")
     return _finish(x, x4, out4, lead, inplace)
+
+
+def pair_bias(z, norm_weight, norm_bias, weight):
+    """Pair bias of AttentionPairBias._prep_bias (attention_pair_bias.py:151-161):
+    permute_final_dims(linear_z(layer_norm_z(z)), [2, 0, 1]).  z [*, N, N, C] -> [*, H, N, N] in
+    z's dtype; norm_bias may be None (a LayerNorm created without offset); weight is [H, C]."""
+    code = _require_gpu(z, "z")
+    lib = _lib.load()
+    z4, lead = _flatten_pair(z)
+    B, N, _, C = z4.shape
+    H = weight.shape[0]
+    if tuple(weight.shape) != (H, C):
+        raise ValueError("pair-bias weight must be [no_heads, c_z]")
+    nw, w = _w(norm_weight, z.dtype), _w(weight, z.dtype)
+    nb = None if norm_bias is None else _w(norm_bias, z.dtype)
+    out = torch.empty(B, H, N, N, dtype=z.dtype, device=z.device)
+    with torch.cuda.device(z.device):
+        st = lib.of3_pair_bias_fwd(z4.data_ptr(), _lib.strides3(z4.stride()[:3]), nw.data_ptr(),
+                                   None if nb is None else nb.data_ptr(), w.data_ptr(), out.data_ptr(), B, N, C, H,
+                                   code, _stream(z))
+    if st == _lib.OF3_EINVAL:
+        raise ValueError("pair bias: bf16 supports c_z 64 or 128 and up to 32 heads, fp32 c_z <= 256 and up to 64 "
+                         "heads; got c_z=%d heads=%d in %s" % (C, H, z.dtype))
+    _lib.check(st, "of3_pair_bias_fwd")
+    return out.view(*lead, H, N, N) if len(lead) != 1 else out

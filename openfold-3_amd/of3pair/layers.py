@@ -237,3 +237,22 @@ class SwiGLUTransition(nn.Module):
             x, mask, self.layer_norm.weight, self.layer_norm.bias, self.swiglu.linear_a.weight,
             self.swiglu.linear_b.weight, self.linear_out.weight, add_residual=bool(_add_residual),
             inplace=bool(_inplace))
+
+
+class PairBiasProjection(nn.Module):
+    """The pair-bias half of the reference's AttentionPairBias (attention_pair_bias.py:106-107,
+    :151-161): layer_norm_z and linear_z under the same parameter names, so the matching slice
+    of an AttentionPairBias state dict loads unchanged.  forward(z) returns the [*, H, N, N]
+    bias that _prep_bias appends to its list."""
+
+    def __init__(self, c_z, no_heads, create_offset=True, linear_init="default"):
+        super().__init__()
+        self.c_z = c_z
+        self.no_heads = no_heads
+        self.layer_norm_z = nn.LayerNorm(c_z, eps=1e-5, bias=create_offset)
+        self.linear_z = nn.Linear(c_z, no_heads, bias=False)
+        _init_linear(self.linear_z, linear_init)
+
+    @torch.no_grad()
+    def forward(self, z):
+        return F3.pair_bias(z, self.layer_norm_z.weight, self.layer_norm_z.bias, self.linear_z.weight)

@@ -144,3 +144,22 @@ def transition_update(x, mask, p):
         for co in range(c):
             out[r, co] = float(np.dot(wo[co], h)) * mf[r]
     return out.reshape(shape)
+
+
+def pair_bias(z, p):
+    """float64 loops: out[h, i, j] = sum_c LN(z[i, j, :])[c] * W[h, c] for z [N, N, C]."""
+    z = np.asarray(z, dtype=np.float64)
+    w = np.asarray(p["linear_z.weight"], dtype=np.float64)
+    g = np.asarray(p["layer_norm_z.weight"], dtype=np.float64)
+    b = np.asarray(p["layer_norm_z.bias"], dtype=np.float64) if "layer_norm_z.bias" in p else np.zeros_like(g)
+    n, _, c = z.shape
+    out = np.zeros((w.shape[0], n, n))
+    for i in range(n):
+        for j in range(n):
+            x = z[i, j]
+            mu = x.sum() / c
+            var = ((x - mu) ** 2).sum() / c
+            xn = (x - mu) / np.sqrt(var + 1e-5) * g + b
+            for h in range(w.shape[0]):
+                out[h, i, j] = (xn * w[h]).sum()
+    return out

@@ -188,6 +188,29 @@ def pair_block(z, pair_mask, p, no_heads: int, row_chunk: int | None = None, mas
     return z + transition_update(z, pair_mask if mask_trans else None, _sub(p, "pair_transition."))
 
 
+def pair_bias(z, p):
+    """AttentionPairBias._prep_bias, pair part (attention_pair_bias.py:151-161): layer_norm_z,
+    linear_z (no bias), permute_final_dims(z, [2, 0, 1]).  z [*, N, N, C] -> [*, H, N, N].
+    Parameters: layer_norm_z.weight, layer_norm_z.bias (optional: LayerNorm without offset),
+    linear_z.weight [H, C]."""
+    bias = p.get("layer_norm_z.bias")
+    if bias is None:
+        bias = torch.zeros_like(p["layer_norm_z.weight"])
+    zn = layer_norm(z, p["layer_norm_z.weight"], bias)
+    out = linear(zn, p["linear_z.weight"])
+    return out.movedim(-1, -3)
+
+
+def make_pair_bias_params(gen, c_z: int, no_heads: int, offset: bool = True):
+    p = {
+        "layer_norm_z.weight": 1.0 + 0.1 * torch.randn(c_z, generator=gen),
+        "linear_z.weight": torch.randn(no_heads, c_z, generator=gen) / math.sqrt(c_z),
+    }
+    if offset:
+        p["layer_norm_z.bias"] = 0.1 * torch.randn(c_z, generator=gen)
+    return p
+
+
 def make_transition_params(gen, c_in: int, n: int):
     def lin(o, i):
         return torch.randn(o, i, generator=gen) / math.sqrt(i)

@@ -236,3 +236,36 @@ def test_transition_invariants():
     b = orc.linear(xn, p["swiglu.linear_b.weight"])
     want = orc.linear(a * torch.sigmoid(a) * b, p["linear_out.weight"]) * mask.unsqueeze(-1)
     assert torch.allclose(out, want, atol=1e-6)
+
+
+# ---- pair-bias projection ----------------------------------------------------------------------
+def test_pair_bias_matches_bruteforce_and_library_routines():
+    gen = torch.Generator().manual_seed(41)
+    n, c, h = 6, 16, 5
+    z = torch.randn(n, n, c, generator=gen)
+    for offset in (True, False):
+        p = orc.make_pair_bias_params(gen, c, h, offset=offset)
+        got = orc.pair_bias(z, p)
+        assert got.shape == (h, n, n)
+        assert np.abs(got.double().numpy() - bf.pair_bias(z, p)).max() < FP32_TOL
+        zn = torch.nn.functional.layer_norm(z, (c,), p["layer_norm_z.weight"], p.get("layer_norm_z.bias"), 1e-5)
+        want = torch.nn.functional.linear(zn, p["linear_z.weight"]).permute(2, 0, 1)
+        assert (got - want).abs().max() < FP32_TOL
+
+
+def test_pair_bias_invariants():
+    gen = torch.Generator().manual_seed(42)
+    c, h = 32, 4
+    z = torch.randn(2, 9, 9, c, generator=gen)
+    p = orc.make_pair_bias_params(gen, c, h)
+    out = orc.pair_bias(z, p)
+    assert out.shape == (2, h, 9, 9)
+    # LayerNorm makes the result invariant to a per-position shift and positive scale of z
+    assert (orc.pair_bias(3.0 * z + 5.0, p) - out).abs().max() < 1e-4
+    # head h of the output only depends on row h of the weight; a transposed input gives the transposed bias
+    q = dict(p)
+    q["linear_z.weight"] = p["linear_z.weight"].clone()
+    q["linear_z.weight"][1] = 0
+    o2 = orc.pair_bias(z, q)
+    assert o2[:, 1].abs().max() == 0 and torch.equal(o2[:, 0], out[:, 0])
+    assert torch.equal(orc.pair_bias(z.transpose(-2, -3), p), out.transpose(-1, -2))
