@@ -201,7 +201,7 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
 
   // ---- LayerNorm -> wave-private LDS tile -> B operands in registers, for the tile whose
   // activations are in `raw`.  Runs before the first tile and at the end of every tile for
-  // the next one (there the wait for the loads is exact: straight-line code after the stores).
+  // the next one, before that tile's stores are issued (see there).
   u32x4_t xb[KS];
   float mtile;
   auto prepare_tile = [&]() {
