@@ -207,11 +207,14 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_f32(TriattnF32 p, int g
   }
 }
 
-// one thread per query of one (b, i, h); keys in chunks of 32 through LDS; online softmax
+// one thread per query of one (b, i, h); keys in chunks of 32 through LDS, and with them the
+// [128 queries x 32 keys] slice of the triangle bias (loaded row-wise, 128 contiguous bytes per
+// query, instead of one cache line per thread and key); online softmax
 template <int D>
 __global__ __launch_bounds__(128) void triattn_core_f32(TriattnF32 p, int qgroups) {
   constexpr int KC = 32;
   __shared__ float ks[KC][D], vs[KC][D], mbs[KC];
+  __shared__ float tbs[128][KC + 1];  // +1: the threads of a wave read one column
   const int N = p.N, H = p.H;
   const int qg = blockIdx.x % qgroups, h = (blockIdx.x / qgroups) % H, i = (blockIdx.x / (qgroups * H)) % N,
             b = blockIdx.x / (qgroups * H * N);
@@ -224,7 +227,7 @@ __global__ __launch_bounds__(128) void triattn_core_f32(TriattnF32 p, int qgroup
     qv[d] = active ? p.q[(bih + qi) * D + d] : 0.f;
     ov[d] = 0.f;
   }
-  const float* tbrow = p.tb + (((size_t)b * H + h) * N + (active ? qi : 0)) * N;
+  const float* tbq = p.tb + (((size_t)b * H + h) * N + (size_t)qg * 128) * N;  // row of query qg*128
   float m = -__builtin_inff(), l = 0.f;
   for (int k0 = 0; k0 < N; k0 += KC) {
     __syncthreads();
@@ -233,6 +236,10 @@ __global__ __launch_bounds__(128) void triattn_core_f32(TriattnF32 p, int qgroup
       const bool in = k0 + kk < N;
       ks[kk][d] = in ? p.k[(bih + k0 + kk) * D + d] : 0.f;
       vs[kk][d] = in ? p.v[(bih + k0 + kk) * D + d] : 0.f;
+    }
+    for (int e = threadIdx.x; e < 128 * KC; e += 128) {
+      const int r = e / KC, c = e % KC;
+      tbs[r][c] = (qg * 128 + r < N && k0 + c < N) ? tbq[(size_t)r * N + k0 + c] : 0.f;
     }
     if (threadIdx.x < KC) {
       const int kx = k0 + threadIdx.x;
@@ -251,7 +258,7 @@ __global__ __launch_bounds__(128) void triattn_core_f32(TriattnF32 p, int qgroup
       for (int d = 0; d < D; ++d) acc = fmaf(qv[d], ks[kk][d], acc);
       // logits in the reference's order: q.k, then the mask bias, then the triangle bias
       acc = acc + mbs[kk];
-      acc = acc + (kk < kn ? tbrow[k0 + kk] : 0.f);
+      acc = acc + tbs[threadIdx.x][kk];
       s[kk] = kk < kn ? acc : -__builtin_inff();
       cmax = fmaxf(cmax, s[kk]);
     }
