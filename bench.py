@@ -18,8 +18,10 @@ Besides the whole-block time the line carries
                 KERNEL_MODEL below);
                 the entries "pair_transition" (the SwiGLU transition that follows the block in
                 every PairBlock) and "pair_bias_proj" (the 16-head pair bias the single-representation
-                attention of a PairFormerBlock takes from z) are timed right after the block's
-                kernels and are not part of `value`;
+                attention of a PairFormerBlock takes from z) and "template_tail" (closing LayerNorm
+                of the template stack, mean over 4 templates, ReLU and linear_t, c_t = 64 -> c_z
+                = 128, at the same N) are timed right after the block's kernels and are not part
+                of `value`;
   cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path)
                 timed once on the host cores for the same workload.
 """
@@ -49,6 +51,7 @@ MEASURED_TRAFFIC = {("trimul_contract", 768): 539701909}
 
 TRANSITION_N = 4           # hidden width factor of the pair transition (AF3 configuration)
 PAIR_BIAS_HEADS = 16       # heads of the pairformer's single-representation attention
+TEMPLATES, C_T = 4, 64     # templates and template channels of the AF3 configuration
 
 METRIC = "ms per Pairformer pair-stack block at N=768 bf16; % of MFMA peak & HBM GB/s"
 
@@ -74,6 +77,8 @@ def kernel_model(B, N, C, CH, H, D):
         "pair_transition": {"bound": "mfma", "flops": 6 * B * N * N * C * (TRANSITION_N * C)},
         # reads z, writes the [PAIR_BIAS_HEADS, N, N] bias
         "pair_bias_proj": {"bound": "hbm", "bytes": U + B * PAIR_BIAS_HEADS * N * N * 2},
+        # reads the TEMPLATES planes of c_t channels, writes one c_z plane
+        "template_tail": {"bound": "hbm", "bytes": B * N * N * 2 * (TEMPLATES * C_T + C)},
     }
 
 
@@ -200,9 +205,15 @@ def main():
     pair_bias = [("pair_bias_proj", lambda: ck(lib.of3_pair_bias_fwd(
         P(zz), z_fwd, P(bp["layer_norm_z.weight"]), P(bp["layer_norm_z.bias"]), P(bp["linear_z.weight"]),
         P(bias_out), B, N, C, PAIR_BIAS_HEADS, _lib.OF3_DTYPE_BF16, s)))]
+    ttp = {k_: v.to(dev).to(bf).contiguous() for k_, v in orc.make_template_tail_params(tgen, C_T, C).items()}
+    t_in = torch.randn(B, TEMPLATES, N, N, C_T, device=dev).to(bf)
+    t_out = torch.empty(B, N, N, C, dtype=bf, device=dev)
+    template_tail = [("template_tail", lambda: ck(lib.of3_template_tail_fwd(
+        P(t_in), P(ttp["template_pair_stack.layer_norm.weight"]), P(ttp["template_pair_stack.layer_norm.bias"]),
+        P(ttp["linear_t.weight"]), P(t_out), B, TEMPLATES, N * N, C_T, C, 1, _lib.OF3_DTYPE_BF16, s)))]
     launches = (trimul("tri_mul_out.", 1) + trimul("tri_mul_in.", 0)
                 + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr) + transition
-                + pair_bias)
+                + pair_bias + template_tail)
     for _ in range(max(args.warmup, 1)):
         for _, fn in launches:
             fn()

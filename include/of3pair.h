@@ -29,6 +29,11 @@
  *                 linear_out, mask)                             -> of3_transition_fwd
  *   openfold3/core/model/layers/attention_pair_bias.py
  *       :151-161  _prep_bias: layer_norm_z, linear_z, permute   -> of3_pair_bias_fwd
+ *   openfold3/core/model/latent/template_module.py
+ *       :376      TemplatePairStack's closing LayerNorm
+ *                 (openfold3/core/model/primitives/normalization.py:65-84) -> of3_layer_norm_fwd
+ *       :462-465  TemplateEmbedderAllAtom tail: mean over the
+ *                 templates, ReLU, linear_t                     -> of3_template_tail_fwd
  *   openfold3/core/model/latent/base_blocks.py
  *       :329-335  "z = z + update" after each module            -> add_residual = 1
  *       :470-478  "z = z + pair_transition(z, mask)"            -> of3_transition_fwd, add_residual = 1
@@ -47,7 +52,8 @@
  *
  * dtype: OF3_DTYPE_BF16 selects the MFMA kernels described above.  OF3_DTYPE_F32 (the
  * reference's default inference precision) is served by of3_trimul_fwd / of3_triattn_fwd /
- * of3_transition_fwd / of3_pair_bias_fwd only: every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
+ * of3_transition_fwd / of3_pair_bias_fwd / of3_layer_norm_fwd / of3_template_tail_fwd only:
+ * every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
  * element counts, any N, C and CH <= 256, H*D <= 256 with D in {16, 32, 64}; plain fp32
  * arithmetic in the reference's order of operations (no MFMA, not the fast path).  The
  * stage entry points are bf16 only.
@@ -163,6 +169,23 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
  * offset); w is [H][C].  No workspace.  bf16: C in {64, 128}, H <= 32; fp32: C <= 256, H <= 64. */
 int of3_pair_bias_fwd(const void* z, const int64_t z_strides[3], const void* ln_w, const void* ln_b, const void* w,
                       void* out, int64_t B, int64_t N, int64_t C, int64_t H, int dtype, void* stream);
+
+/* ---- template branch: closing LayerNorm and embedder tail ------------------------------ */
+
+/* out = LayerNorm(x) over the last dimension of a contiguous [rows][C] tensor (eps 1e-5, affine):
+ * the LayerNorm that ends TemplatePairStack.forward.  out may alias x.  bf16: C in {64, 128};
+ * fp32: C <= 256. */
+int of3_layer_norm_fwd(const void* x, const void* ln_w, const void* ln_b, void* out, int64_t rows, int64_t C,
+                       int dtype, void* stream);
+
+/* out[b][p][:] = W . relu((1/T) * sum_t u[b][t][p][:]) with u = LayerNorm(t) when apply_ln is
+ * non-zero (t is the output of the stack's last block and the closing LayerNorm is fused in) or
+ * u = t (t already normalised).  t: contiguous [B][T][P][C_t], P = N*N positions; w: linear_t,
+ * [C_z][C_t], no bias; out: contiguous [B][P][C_z].  The sum runs over the templates in order,
+ * its bf16 value, the division by T and the linear output are rounded where the reference's
+ * bf16 tensors are.  No workspace.  bf16: C_t = 64, C_z = 128; fp32: C_t <= 256. */
+int of3_template_tail_fwd(const void* t, const void* ln_w, const void* ln_b, const void* w, void* out, int64_t B,
+                          int64_t T, int64_t P, int64_t C_t, int64_t C_z, int apply_ln, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

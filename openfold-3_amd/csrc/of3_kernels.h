@@ -108,6 +108,30 @@ struct PairBiasArgs {
 };
 hipError_t pair_bias_launch(const PairBiasArgs& args, int C, hipStream_t stream);
 
+// ---- template branch (template_tail.hip): closing LayerNorm of the stack, and the fused
+// LayerNorm -> mean over templates -> ReLU -> linear_t tail
+struct TemplateTailArgs {
+  const bf16_t* t;            // [B][T][P][C_t] contiguous, P = N*N positions
+  const bf16_t *ln_w, *ln_b;  // [C_t]; used when apply_ln
+  const bf16_t* w;            // linear_t, [C_z][C_t]
+  bf16_t* out;                // [B][P][C_z] contiguous
+  long P;
+  int B, T, apply_ln;
+};
+hipError_t template_tail_launch(const TemplateTailArgs& args, int CT, int CZ, hipStream_t stream);
+hipError_t layer_norm_launch(const bf16_t* x, const bf16_t* w, const bf16_t* b, bf16_t* out, long rows, int C,
+                             hipStream_t stream);
+
+struct TemplateTailF32Args {
+  const float *t, *ln_w, *ln_b, *w;
+  float* out;
+  long P;
+  int B, T, CT, CZ, apply_ln;
+};
+hipError_t template_tail_fwd_f32(const TemplateTailF32Args& args, hipStream_t stream);
+hipError_t layer_norm_fwd_f32(const float* x, const float* w, const float* b, float* out, long rows, int C,
+                              hipStream_t stream);
+
 // ---- fp32 path (pair_f32.hip): whole updates, any N, C and C_hidden <= 256, head width 16/32/64
 struct TrimulF32Args {
   const float* z;

@@ -497,4 +497,63 @@ int of3_pair_bias_fwd(const void* z, const int64_t z_strides[3], const void* ln_
   return e == hipSuccess ? OF3_OK : fail_hip(e);
 }
 
+int of3_layer_norm_fwd(const void* x, const void* ln_w, const void* ln_b, void* out, int64_t rows, int64_t C,
+                       int dtype, void* stream) {
+  if (rows < 1 || !x || !ln_w || !ln_b || !out) return OF3_EINVAL;
+  if (dtype == OF3_DTYPE_F32) {
+    if (C < 1 || C > 256) return OF3_EINVAL;
+    if (!aligned4(x) || !aligned4(ln_w) || !aligned4(ln_b) || !aligned4(out)) return OF3_EINVAL;
+    hipError_t e = of3::layer_norm_fwd_f32(static_cast<const float*>(x), static_cast<const float*>(ln_w),
+                                           static_cast<const float*>(ln_b), static_cast<float*>(out), (long)rows,
+                                           (int)C, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? OF3_OK : fail_hip(e);
+  }
+  if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
+  if (!(C == 128 || C == 64)) return OF3_EINVAL;
+  if (!aligned16(x) || !aligned16(ln_w) || !aligned16(ln_b) || !aligned16(out)) return OF3_EINVAL;
+  hipError_t e = of3::layer_norm_launch(bf(x), bf(ln_w), bf(ln_b), bf(out), (long)rows, (int)C,
+                                        static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
+int of3_template_tail_fwd(const void* t, const void* ln_w, const void* ln_b, const void* w, void* out, int64_t B,
+                          int64_t T, int64_t P, int64_t C_t, int64_t C_z, int apply_ln, int dtype, void* stream) {
+  if (B < 1 || T < 1 || T > 1024 || P < 1 || !t || !w || !out) return OF3_EINVAL;
+  if (apply_ln && (!ln_w || !ln_b)) return OF3_EINVAL;
+  if (B > 0x7fffffffll || P > (1ll << 40)) return OF3_EINVAL;
+  if (dtype == OF3_DTYPE_F32) {
+    if (C_t < 1 || C_t > 256 || C_z < 1 || C_z > 4096) return OF3_EINVAL;
+    if (!aligned4(t) || !aligned4(ln_w) || !aligned4(ln_b) || !aligned4(w) || !aligned4(out)) return OF3_EINVAL;
+    of3::TemplateTailF32Args a;
+    a.t = static_cast<const float*>(t);
+    a.ln_w = static_cast<const float*>(ln_w);
+    a.ln_b = static_cast<const float*>(ln_b);
+    a.w = static_cast<const float*>(w);
+    a.out = static_cast<float*>(out);
+    a.P = (long)P;
+    a.B = (int)B;
+    a.T = (int)T;
+    a.CT = (int)C_t;
+    a.CZ = (int)C_z;
+    a.apply_ln = apply_ln ? 1 : 0;
+    hipError_t e = of3::template_tail_fwd_f32(a, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? OF3_OK : fail_hip(e);
+  }
+  if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
+  if (C_t != 64 || C_z != 128) return OF3_EINVAL;
+  if (!aligned16(t) || !aligned16(ln_w) || !aligned16(ln_b) || !aligned16(w) || !aligned16(out)) return OF3_EINVAL;
+  of3::TemplateTailArgs a;
+  a.t = bf(t);
+  a.ln_w = bf(ln_w);
+  a.ln_b = bf(ln_b);
+  a.w = bf(w);
+  a.out = bf(out);
+  a.P = (long)P;
+  a.B = (int)B;
+  a.T = (int)T;
+  a.apply_ln = apply_ln ? 1 : 0;
+  hipError_t e = of3::template_tail_launch(a, (int)C_t, (int)C_z, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
 }  // extern "C"

@@ -391,7 +391,95 @@ __global__ __launch_bounds__(kThreads) void pair_bias_f32(PairBiasF32 p, int gro
   }
 }
 
+// ---- template branch: closing LayerNorm of the stack and the mean / ReLU / linear_t tail -------
+struct TemplateTailF32 {
+  const float *t, *ln_w, *ln_b, *w;
+  float* out;
+  long P;
+  int B, T, CT, CZ, apply_ln;
+};
+
+// kP positions per work-group: per template LayerNorm into xn, summed into acc (template order,
+// like torch.sum), then / T, ReLU, and the C_z dot products
+__global__ __launch_bounds__(kThreads) void template_tail_f32(TemplateTailF32 p, long groups) {
+  __shared__ float xn[kP][kMaxC];
+  __shared__ float acc[kP][kMaxC];
+  const int CT = p.CT, CZ = p.CZ, T = p.T;
+  const long g = blockIdx.x % groups;
+  const int b = (int)(blockIdx.x / groups);
+  const long p0 = g * kP;
+  for (int idx = threadIdx.x; idx < kP * CT; idx += kThreads) acc[idx / CT][idx % CT] = 0.f;
+  __syncthreads();
+  for (int t = 0; t < T; ++t) {
+    const float* plane = p.t + ((size_t)b * T + t) * p.P * CT;
+    if (p.apply_ln) {
+      layer_norm_rows([&](int pos) -> const float* { return p0 + pos < p.P ? plane + (p0 + pos) * CT : nullptr; },
+                      p.ln_w, p.ln_b, CT, xn);
+      __syncthreads();
+      for (int idx = threadIdx.x; idx < kP * CT; idx += kThreads) acc[idx / CT][idx % CT] += xn[idx / CT][idx % CT];
+    } else {
+      for (int idx = threadIdx.x; idx < kP * CT; idx += kThreads) {
+        const int pos = idx / CT, c = idx % CT;
+        if (p0 + pos < p.P) acc[pos][c] += plane[(p0 + pos) * CT + c];
+      }
+    }
+    __syncthreads();
+  }
+  for (int idx = threadIdx.x; idx < kP * CT; idx += kThreads) {
+    const float m = acc[idx / CT][idx % CT] / (float)T;
+    xn[idx / CT][idx % CT] = m > 0.f ? m : 0.f;
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * CZ; idx += kThreads) {
+    const int pos = idx / CZ, o = idx % CZ;
+    if (p0 + pos < p.P) p.out[((size_t)b * p.P + p0 + pos) * CZ + o] = dot_row(xn[pos], p.w + (size_t)o * CT, CT);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void layer_norm_f32(const float* __restrict__ x, const float* __restrict__ w,
+                                                           const float* __restrict__ bsh, float* __restrict__ out,
+                                                           long rows, int C) {
+  __shared__ float xn[kP][kMaxC];
+  const long r0 = (long)blockIdx.x * kP;
+  layer_norm_rows([&](int pos) -> const float* { return r0 + pos < rows ? x + (r0 + pos) * C : nullptr; }, w, bsh, C, xn);
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < kP * C; idx += kThreads) {
+    const int pos = idx / C, c = idx % C;
+    if (r0 + pos < rows) out[(r0 + pos) * C + c] = xn[pos][c];
+  }
+}
+
 }  // namespace
+
+hipError_t template_tail_fwd_f32(const TemplateTailF32Args& a, hipStream_t stream) {
+  if (a.CT < 1 || a.CT > kMaxC || a.CZ < 1 || a.T < 1 || a.P < 1 || a.B < 1) return hipErrorInvalidValue;
+  TemplateTailF32 p;
+  p.t = a.t;
+  p.ln_w = a.ln_w;
+  p.ln_b = a.ln_b;
+  p.w = a.w;
+  p.out = a.out;
+  p.P = a.P;
+  p.B = a.B;
+  p.T = a.T;
+  p.CT = a.CT;
+  p.CZ = a.CZ;
+  p.apply_ln = a.apply_ln;
+  const long groups = (a.P + kP - 1) / kP;
+  const long blocks = groups * a.B;
+  if (blocks > 0x7fffffffl) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(template_tail_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  return hipGetLastError();
+}
+
+hipError_t layer_norm_fwd_f32(const float* x, const float* w, const float* b, float* out, long rows, int C,
+                              hipStream_t stream) {
+  if (rows < 1 || C < 1 || C > kMaxC) return hipErrorInvalidValue;
+  const long blocks = (rows + kP - 1) / kP;
+  if (blocks > 0x7fffffffl) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(layer_norm_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, w, b, out, rows, C);
+  return hipGetLastError();
+}
 
 hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   TrimulF32 p;

@@ -4,9 +4,11 @@ from .layers import (PairBiasProjection, SwiGLUTransition, TriangleAttention, Tr
                      TriangleMultiplicationIncoming, TriangleMultiplicationOutgoing,
                      TriangleMultiplicativeUpdate)
 from .pair_stack import PairBlock, PairStack
+from .template import TemplateEmbedderCore, TemplatePairBlock, TemplatePairStack
+from . import checkpoint
 
 __all__ = [
     "TriangleMultiplicativeUpdate", "TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming",
     "TriangleAttention", "TriangleAttentionStartingNode", "TriangleAttentionEndingNode", "SwiGLUTransition", "PairBiasProjection",
-    "PairStack", "PairBlock",
+    "PairStack", "PairBlock", "TemplatePairBlock", "TemplatePairStack", "TemplateEmbedderCore", "checkpoint",
 ]

@@ -28,6 +28,7 @@ SOURCES = [
     "triattn_out.hip",
     "transition.hip",
     "pair_bias.hip",
+    "template_tail.hip",
     "pair_f32.hip",
 ]
 

@@ -212,3 +212,56 @@ def pair_bias(z, norm_weight, norm_bias, weight):
                          "heads; got c_z=%d heads=%d in %s" % (C, H, z.dtype))
     _lib.check(st, "of3_pair_bias_fwd")
     return out.view(*lead, H, N, N) if len(lead) != 1 else out
+
+
+def layer_norm(x, weight, bias):
+    """LayerNorm over the last dimension (eps 1e-5), the closing step of TemplatePairStack.forward
+    (template_module.py:376).  Returns a new contiguous tensor of x's shape and dtype."""
+    code = _require_gpu(x, "x")
+    lib = _lib.load()
+    xc = x.contiguous()
+    C = xc.shape[-1]
+    rows = xc.numel() // C
+    out = torch.empty_like(xc)
+    w, b = _w(weight, x.dtype), _w(bias, x.dtype)
+    with torch.cuda.device(x.device):
+        st = lib.of3_layer_norm_fwd(xc.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(), rows, C, code,
+                                    _stream(x))
+    if st == _lib.OF3_EINVAL:
+        raise ValueError("layer norm: bf16 supports 64 or 128 channels, fp32 up to 256; got %d in %s" % (C, x.dtype))
+    _lib.check(st, "of3_layer_norm_fwd")
+    return out
+
+
+def template_tail(t, norm_weight, norm_bias, linear_t_weight, apply_layer_norm: bool = True):
+    """Tail of TemplateEmbedderAllAtom.forward (template_module.py:462-465), with the template
+    stack's closing LayerNorm (:376) fused in when apply_layer_norm is set:
+    linear_t(relu(sum_T LN(t) / T)).  t [*, T, N, N, C_t] -> [*, N, N, C_z] in t's dtype."""
+    code = _require_gpu(t, "t")
+    lib = _lib.load()
+    if t.dim() < 4:
+        raise ValueError("t must be [*, N_templ, N, N, C_t]")
+    tc = t.contiguous()
+    lead = tc.shape[:-4]
+    T, N, N2, CT = tc.shape[-4:]
+    if N != N2:
+        raise ValueError("t must be square in its two token dimensions")
+    B = 1
+    for d in lead:
+        B *= d
+    CZ = linear_t_weight.shape[0]
+    if tuple(linear_t_weight.shape) != (CZ, CT):
+        raise ValueError("linear_t weight must be [c_z, c_t]")
+    w = _w(linear_t_weight, t.dtype)
+    nw = _w(norm_weight, t.dtype) if apply_layer_norm else None
+    nb = _w(norm_bias, t.dtype) if apply_layer_norm else None
+    out = torch.empty(*lead, N, N, CZ, dtype=t.dtype, device=t.device)
+    with torch.cuda.device(t.device):
+        st = lib.of3_template_tail_fwd(tc.data_ptr(), None if nw is None else nw.data_ptr(),
+                                       None if nb is None else nb.data_ptr(), w.data_ptr(), out.data_ptr(), B, T,
+                                       N * N, CT, CZ, 1 if apply_layer_norm else 0, code, _stream(t))
+    if st == _lib.OF3_EINVAL:
+        raise ValueError("template tail: bf16 supports c_t = 64 with c_z = 128, fp32 c_t <= 256; got c_t=%d c_z=%d "
+                         "in %s" % (CT, CZ, t.dtype))
+    _lib.check(st, "of3_template_tail_fwd")
+    return out

@@ -163,3 +163,23 @@ def pair_bias(z, p):
             for h in range(w.shape[0]):
                 out[h, i, j] = (xn * w[h]).sum()
     return out
+
+
+def template_tail(t, ln_w, ln_b, w):
+    """float64 loops: out[i, j, :] = W @ relu(mean_T LN(t[T, i, j, :])) for t [T, N, N, C]
+    (template_module.py:376 and :462-465)."""
+    t = np.asarray(t, dtype=np.float64)
+    g = np.asarray(ln_w, dtype=np.float64)
+    b = np.asarray(ln_b, dtype=np.float64)
+    w = np.asarray(w, dtype=np.float64)
+    nt, n, _, c = t.shape
+    out = np.zeros((n, n, w.shape[0]))
+    for i in range(n):
+        for j in range(n):
+            acc = np.zeros(c)
+            for k in range(nt):
+                acc += _ln(t[k, i, j], g, b)
+            acc = np.maximum(acc / nt, 0.0)
+            for o in range(w.shape[0]):
+                out[i, j, o] = (w[o] * acc).sum()
+    return out

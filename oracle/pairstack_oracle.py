@@ -12,8 +12,9 @@ reference's stock (no alternative kernel) path through
       openfold3/core/model/primitives/attention.py:265-302, :94-135,
   * PairBlock.tri_mul_out_in / tri_att_start_end
       openfold3/core/model/latent/base_blocks.py:307-406,
-  * TemplatePairBlock.forward (per-template loop, tri_mul_first=True)
-      openfold3/core/model/latent/template_module.py:148-166.
+  * TemplatePairBlock.forward (per-template loop, tri_mul_first=True), TemplatePairStack.forward
+    with its final LayerNorm, and the mean / ReLU / linear_t tail of TemplateEmbedderAllAtom
+      openfold3/core/model/latent/template_module.py:148-193, :302-378, :462-465.
 
 It may be imported by tests/, by __graft_entry__.smoke() and by the
 cpu_baseline leg of bench.py, as the checker or the timed CPU baseline.
@@ -326,6 +327,42 @@ def template_pair_stack(t, mask, blocks, no_heads: int, row_chunk: int | None = 
             zt = pair_stack_block(zt, mt, p, no_heads, row_chunk=row_chunk)
         outs.append(zt.unsqueeze(-4))
     return torch.cat(outs, dim=-4)
+
+
+def template_stack(t, mask, blocks, ln_weight, ln_bias, no_heads: int, row_chunk: int | None = None,
+                   mask_trans: bool = True):
+    """TemplatePairStack.forward (template_module.py:302-378): every template runs through every
+    TemplatePairBlock (tri_mul_first=True: pair stack, then t + pair_transition(t),
+    template_module.py:148-193), then the stack's LayerNorm.  t: [*, T, N, N, C]; mask: [*, T, N, N]
+    or [*, 1, N, N] (expanded over the templates, template_module.py:326-329).  ``blocks`` holds one
+    parameter dict per block with the PairBlock prefixes (tri_mul_out. ... pair_transition.).
+    """
+    if mask.shape[-3] == 1:
+        mask = mask.expand(*mask.shape[:-3], t.shape[-4], *mask.shape[-2:])
+    outs = []
+    for ti in range(t.shape[-4]):
+        zt = t[..., ti, :, :, :]
+        mt = mask[..., ti, :, :]
+        for p in blocks:
+            zt = pair_block(zt, mt, p, no_heads, row_chunk=row_chunk, mask_trans=mask_trans)
+        outs.append(zt.unsqueeze(-4))
+    return layer_norm(torch.cat(outs, dim=-4), ln_weight, ln_bias)
+
+
+def template_tail(t, linear_t_weight):
+    """Tail of TemplateEmbedderAllAtom.forward (template_module.py:462-465): mean over the
+    templates, ReLU, bias-free linear_t.  t: [*, T, N, N, C_t] (the stack's output) ->
+    [*, N, N, C_z]."""
+    u = torch.sum(t, dim=-4) / t.shape[-4]
+    return linear(torch.relu(u), linear_t_weight)
+
+
+def make_template_tail_params(gen, c_t: int, c_z: int):
+    return {
+        "template_pair_stack.layer_norm.weight": 1 + 0.1 * torch.randn(c_t, generator=gen),
+        "template_pair_stack.layer_norm.bias": 0.1 * torch.randn(c_t, generator=gen),
+        "linear_t.weight": torch.randn(c_z, c_t, generator=gen) / math.sqrt(c_t),
+    }
 
 
 # --------------------------------------------------------------------------

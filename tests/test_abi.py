@@ -33,7 +33,8 @@ def test_header_declares_expected_entry_points():
                      "of3_triattn_fwd", "of3_triattn_proj", "of3_triattn_flash", "of3_triattn_out",
                      "of3_version", "of3_last_hip_error", "of3_status_string", "of3_padded_n",
                      "of3_trimul_workspace_bytes", "of3_triattn_workspace_bytes",
-                     "of3_trimul_workspace_bytes_for", "of3_triattn_workspace_bytes_for"):
+                     "of3_trimul_workspace_bytes_for", "of3_triattn_workspace_bytes_for",
+                     "of3_transition_fwd", "of3_pair_bias_fwd", "of3_layer_norm_fwd", "of3_template_tail_fwd"):
         assert required in names
 
 
@@ -149,3 +150,21 @@ def test_check_maps_status_to_exceptions(lib):
         _lib.check(_lib.OF3_EINVAL, "x")
     with pytest.raises(RuntimeError):
         _lib.check(_lib.OF3_ENOSPC, "x")
+
+
+def test_template_entry_points_validate(lib):
+    """Argument checks run before any device work: bad shapes and null pointers are refused."""
+    from of3pair import _lib as L
+
+    p = 256  # any non-null, 16-byte aligned value: it is never dereferenced on these paths
+    assert lib.of3_layer_norm_fwd(None, p, p, p, 8, 64, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_layer_norm_fwd(p, p, p, p, 0, 64, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_layer_norm_fwd(p, p, p, p, 8, 96, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_layer_norm_fwd(p, p, p, p, 8, 300, L.OF3_DTYPE_F32, None) == L.OF3_EINVAL
+    assert lib.of3_layer_norm_fwd(p + 2, p, p, p, 8, 64, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_template_tail_fwd(p, p, p, p, p, 1, 0, 16, 64, 128, 1, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_template_tail_fwd(p, p, p, p, p, 1, 2, 16, 32, 128, 1, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_template_tail_fwd(p, p, p, p, p, 1, 2, 16, 64, 64, 1, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_template_tail_fwd(p, None, p, p, p, 1, 2, 16, 64, 128, 1, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_template_tail_fwd(p, p, p, None, p, 1, 2, 16, 64, 128, 0, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+    assert lib.of3_template_tail_fwd(p, p, p, p, p, 1, 2, 16, 64, 128, 1, 7, None) == L.OF3_EINVAL

@@ -103,3 +103,104 @@ def test_package_does_not_import_the_oracle():
         if fn.endswith(".py"):
             text = open(os.path.join(src_dir, fn)).read()
             assert "oracle" not in text, "%s mentions the oracle" % fn
+
+
+TEMPLATE_STACK_CFG = dict(c_t=64, c_hidden_tri_att=16, c_hidden_tri_mul=64, no_blocks=2, no_heads=4,
+                          transition_type="swiglu", pair_transition_n=2, dropout_rate=0.25, tri_mul_first=True,
+                          fuse_projection_weights=False, blocks_per_ckpt=None, inf=1e9, use_reentrant=False,
+                          tune_chunk_size=False)
+
+
+def test_template_modules_take_the_reference_config_and_names():
+    """template_pair_stack of the reference's model config (model_config.py:212-230) constructs
+    the stack; parameter names are the reference's (blocks.<i>.<PairBlock names>, layer_norm)."""
+    stack = of3pair.TemplatePairStack(**TEMPLATE_STACK_CFG)
+    names = set(stack.state_dict())
+    assert len(stack.blocks) == 2 and stack.blocks[0].tri_mul_first is True
+    for i in (0, 1):
+        for k in ("tri_mul_out.linear_a_p.weight", "tri_mul_in.layer_norm_out.bias", "tri_att_start.mha.linear_q.weight",
+                  "tri_att_end.linear_z.weight", "pair_transition.layer_norm.weight",
+                  "pair_transition.swiglu.linear_a.weight", "pair_transition.linear_out.weight"):
+            assert "blocks.%d.%s" % (i, k) in names
+    assert {"layer_norm.weight", "layer_norm.bias"} <= names
+    assert tuple(stack.state_dict()["blocks.1.pair_transition.swiglu.linear_b.weight"].shape) == (128, 64)
+    core = of3pair.TemplateEmbedderCore(64, 128, TEMPLATE_STACK_CFG, {"linear_t": {"bias": False, "init": "default"}})
+    assert tuple(core.linear_t.weight.shape) == (128, 64) and core.linear_t.bias is None
+    assert all(k.startswith("template_pair_stack.") or k == "linear_t.weight" for k in core.state_dict())
+    sig = inspect.signature(of3pair.TemplatePairStack.forward)
+    for name in ("t", "mask", "chunk_size", "use_deepspeed_evo_attention", "use_cueq_triangle_kernels", "use_lma",
+                 "inplace_safe", "_mask_trans"):
+        assert name in sig.parameters
+    with pytest.raises(ValueError):
+        of3pair.TemplatePairStack(**dict(TEMPLATE_STACK_CFG, transition_type="relu"))
+
+
+def _fake_model_state_dict():
+    """Keys as a reference model's state dict spells them, random values."""
+    gen = torch.Generator().manual_seed(5)
+    sd = {}
+    for i in range(2):
+        blk = of3pair.PairBlock(128, 128, 32, 4, "swiglu", 4, 0.25, False, 1e9)
+        for k, v in blk.state_dict().items():
+            sd["pairformer_stack.blocks.%d.pair_stack.%s" % (i, k)] = torch.randn(v.shape, generator=gen)
+        sd["pairformer_stack.blocks.%d.attn_pair_bias.layer_norm_z.weight" % i] = torch.randn(128, generator=gen)
+        sd["pairformer_stack.blocks.%d.attn_pair_bias.layer_norm_z.bias" % i] = torch.randn(128, generator=gen)
+        sd["pairformer_stack.blocks.%d.attn_pair_bias.linear_z.weight" % i] = torch.randn(16, 128, generator=gen)
+        sd["pairformer_stack.blocks.%d.attn_pair_bias.mha.linear_q.weight" % i] = torch.randn(384, 384, generator=gen)
+    core = of3pair.TemplateEmbedderCore(64, 128, TEMPLATE_STACK_CFG)
+    for k, v in core.state_dict().items():
+        sd["template_embedder." + k] = torch.randn(v.shape, generator=gen)
+    sd["template_embedder.template_pair_embedder.linear_z.weight"] = torch.randn(64, 128, generator=gen)
+    return sd
+
+
+@pytest.mark.parametrize("container", ["pretrained", "lightning", "deepspeed", "ema"])
+def test_checkpoint_slices_load_into_the_modules(container):
+    from of3pair import checkpoint as ck
+
+    raw = _fake_model_state_dict()
+    if container == "pretrained":
+        ckpt = raw
+    elif container == "lightning":
+        ckpt = {"state_dict": {"model." + k: v for k, v in raw.items()}, "epoch": 3}
+    elif container == "deepspeed":
+        ckpt = {"module": {"model." + k: v for k, v in raw.items()}}
+    else:
+        ckpt = {"state_dict": {"model." + k: torch.zeros_like(v) for k, v in raw.items()}, "ema": {"params": raw}}
+    sd = ck.state_dict_from_checkpoint(ckpt, init_from_ema_weights=(container == "ema"))
+    assert all(k.startswith("model.") for k in sd)
+    assert ck.pairformer_block_count(sd) == 2
+    blocks = [of3pair.PairBlock(128, 128, 32, 4, "swiglu", 4, 0.25, False, 1e9) for _ in range(2)]
+    ck.load_pairformer_pair_blocks(blocks, sd)
+    assert torch.equal(blocks[1].tri_att_end.mha.linear_o.weight,
+                       raw["pairformer_stack.blocks.1.pair_stack.tri_att_end.mha.linear_o.weight"])
+    assert torch.equal(blocks[0].pair_transition.swiglu.linear_a.weight,
+                       raw["pairformer_stack.blocks.0.pair_stack.pair_transition.swiglu.linear_a.weight"])
+    core = ck.load_template_embedder(of3pair.TemplateEmbedderCore(64, 128, TEMPLATE_STACK_CFG), sd)
+    assert torch.equal(core.linear_t.weight, raw["template_embedder.linear_t.weight"])
+    assert torch.equal(core.template_pair_stack.layer_norm.bias, raw["template_embedder.template_pair_stack.layer_norm.bias"])
+    proj = ck.load_pair_bias_projection(of3pair.PairBiasProjection(128, 16), sd,
+                                        "model.pairformer_stack.blocks.1.attn_pair_bias.")
+    assert torch.equal(proj.linear_z.weight, raw["pairformer_stack.blocks.1.attn_pair_bias.linear_z.weight"])
+
+
+def test_checkpoint_loading_reports_missing_and_unexpected_keys(tmp_path):
+    from of3pair import checkpoint as ck
+
+    sd = {"model." + k: v for k, v in _fake_model_state_dict().items()}
+    blk = of3pair.PairBlock(128, 128, 32, 4, "swiglu", 4, 0.25, False, 1e9)
+    with pytest.raises(KeyError):
+        ck.load_pair_block(blk, sd, "model.pairformer_stack.blocks.7.pair_stack.")
+    broken = dict(sd)
+    del broken["model.pairformer_stack.blocks.0.pair_stack.tri_mul_in.linear_g.weight"]
+    with pytest.raises(KeyError, match="linear_g"):
+        ck.load_pair_block(blk, broken, "model.pairformer_stack.blocks.0.pair_stack.")
+    extra = dict(sd)
+    extra["model.template_embedder.linear_u.weight"] = torch.zeros(1)
+    with pytest.raises(KeyError, match="linear_u"):
+        ck.load_template_embedder(of3pair.TemplateEmbedderCore(64, 128, TEMPLATE_STACK_CFG), extra)
+    # files are read with the loader that executes nothing
+    path = tmp_path / "w.pt"
+    torch.save({k[len("model."):]: v for k, v in sd.items()}, path)
+    loaded = ck.state_dict_from_checkpoint(ck.load_checkpoint_file(path))
+    assert sorted(loaded) == sorted(sd)

@@ -269,3 +269,50 @@ def test_pair_bias_invariants():
     o2 = orc.pair_bias(z, q)
     assert o2[:, 1].abs().max() == 0 and torch.equal(o2[:, 0], out[:, 0])
     assert torch.equal(orc.pair_bias(z.transpose(-2, -3), p), out.transpose(-1, -2))
+
+
+def test_template_tail_matches_bruteforce_and_library_routines():
+    gen = torch.Generator().manual_seed(51)
+    nt, n, c_t, c_z = 3, 5, 16, 24
+    t = torch.randn(nt, n, n, c_t, generator=gen)
+    p = orc.make_template_tail_params(gen, c_t, c_z)
+    g, b, w = p["template_pair_stack.layer_norm.weight"], p["template_pair_stack.layer_norm.bias"], p["linear_t.weight"]
+    got = orc.template_tail(orc.layer_norm(t, g, b), w)
+    assert got.shape == (n, n, c_z)
+    assert np.abs(got.double().numpy() - bf.template_tail(t, g, b, w)).max() < FP32_TOL
+    tn = torch.nn.functional.layer_norm(t, (c_t,), g, b, 1e-5)
+    want = torch.nn.functional.linear(torch.relu(tn.mean(dim=0)), w)
+    assert (got - want).abs().max() < FP32_TOL
+    # a template whose normalised features are all negative contributes nothing after the ReLU
+    # only through the mean: one template alone equals relu(LN) @ W^T
+    one = orc.template_tail(orc.layer_norm(t[:1], g, b), w)
+    assert (one - torch.nn.functional.linear(torch.relu(tn[0]), w)).abs().max() < FP32_TOL
+    # permuting the templates changes nothing (a mean), up to summation order
+    assert (orc.template_tail(orc.layer_norm(t.flip(0), g, b), w) - got).abs().max() < 1e-5
+
+
+def test_template_stack_is_blocks_then_layer_norm():
+    """template_stack = per-template PairBlocks (already pinned) followed by LayerNorm; a mask
+    given once ([1, N, N]) is the same mask for every template."""
+    gen = torch.Generator().manual_seed(52)
+    nt, n, c = 2, 7, 16
+    blocks = []
+    for seed in (3, 4):
+        p = orc.make_block_params(seed, c, c, 4, 4)
+        p.update({"pair_transition." + k: v for k, v in orc.make_transition_params(gen, c, 2).items()})
+        blocks.append(p)
+    t = orc.make_pair_input(53, (nt,), n, c)
+    mask = orc.tail_padding_mask((nt,), n, torch.tensor([0, 2]))
+    g = 1 + 0.1 * torch.randn(c, generator=gen)
+    b = 0.1 * torch.randn(c, generator=gen)
+    got = orc.template_stack(t, mask, blocks, g, b, 4)
+    for ti in range(nt):
+        z = t[ti]
+        for p in blocks:
+            z = orc.pair_block(z, mask[ti], p, 4)
+        want = torch.nn.functional.layer_norm(z, (c,), g, b, 1e-5)
+        assert (got[ti] - want).abs().max() < FP32_TOL
+    shared = orc.tail_padding_mask((1,), n, 2)
+    a = orc.template_stack(t, shared, blocks, g, b, 4)
+    bb = orc.template_stack(t, shared.expand(nt, n, n), blocks, g, b, 4)
+    assert torch.equal(a, bb)
