@@ -18,7 +18,8 @@ Besides the whole-block time the line carries
                 KERNEL_MODEL below);
                 the entries "pair_transition" (the SwiGLU transition that follows the block in
                 every PairBlock) and "pair_bias_proj" (the 16-head pair bias the single-representation
-                attention of a PairFormerBlock takes from z) and "template_tail" (closing LayerNorm
+                attention of a PairFormerBlock takes from z), "attn_pair_bias" (that attention itself
+                over s [N, 384], 16 heads of 24: its three small kernels as one call) and "template_tail" (closing LayerNorm
                 of the template stack, mean over 4 templates, ReLU and linear_t, c_t = 64 -> c_z
                 = 128, at the same N) are timed right after the block's kernels and are not part
                 of `value`;
@@ -52,6 +53,7 @@ MEASURED_TRAFFIC = {("trimul_contract", 768): 539701909}
 TRANSITION_N = 4           # hidden width factor of the pair transition (AF3 configuration)
 PAIR_BIAS_HEADS = 16       # heads of the pairformer's single-representation attention
 TEMPLATES, C_T = 4, 64     # templates and template channels of the AF3 configuration
+C_S, C_HEAD_S = 384, 24    # single representation and head width of its attention
 
 METRIC = "ms per Pairformer pair-stack block at N=768 bf16; % of MFMA peak & HBM GB/s"
 
@@ -77,6 +79,8 @@ def kernel_model(B, N, C, CH, H, D):
         "pair_transition": {"bound": "mfma", "flops": 6 * B * N * N * C * (TRANSITION_N * C)},
         # reads z, writes the [PAIR_BIAS_HEADS, N, N] bias
         "pair_bias_proj": {"bound": "hbm", "bytes": U + B * PAIR_BIAS_HEADS * N * N * 2},
+        # LayerNorm + q, k, v, g projections, QK^T and PV over 16 heads of 24, output projection
+        "attn_pair_bias": {"bound": "mfma", "flops": 10 * B * N * C_S * C_S + 4 * B * N * N * C_S},
         # reads the TEMPLATES planes of c_t channels, writes one c_z plane
         "template_tail": {"bound": "hbm", "bytes": B * N * N * 2 * (TEMPLATES * C_T + C)},
     }
@@ -211,9 +215,20 @@ def main():
     template_tail = [("template_tail", lambda: ck(lib.of3_template_tail_fwd(
         P(t_in), P(ttp["template_pair_stack.layer_norm.weight"]), P(ttp["template_pair_stack.layer_norm.bias"]),
         P(ttp["linear_t.weight"]), P(t_out), B, TEMPLATES, N * N, C_T, C, 1, _lib.OF3_DTYPE_BF16, s)))]
+    sp = {k_: v.to(dev).to(bf).contiguous()
+          for k_, v in orc.make_attention_pair_bias_params(tgen, C_S, C, C_HEAD_S, PAIR_BIAS_HEADS).items()}
+    s_in = torch.randn(B, N, C_S, device=dev).to(bf)
+    s_out = torch.empty_like(s_in)
+    s_ws = torch.empty(int(lib.of3_attn_pair_bias_workspace_bytes(B, N, C_S, PAIR_BIAS_HEADS, C_HEAD_S)),
+                       dtype=torch.uint8, device=dev)
+    attn_pair_bias = [("attn_pair_bias", lambda: ck(lib.of3_attn_pair_bias_fwd(
+        P(s_in), P(bias_out), None, P(sp["layer_norm_a.weight"]), P(sp["layer_norm_a.bias"]),
+        P(sp["mha.linear_q.weight"]), P(sp["mha.linear_q.bias"]), P(sp["mha.linear_k.weight"]),
+        P(sp["mha.linear_v.weight"]), P(sp["mha.linear_g.weight"]), P(sp["mha.linear_o.weight"]), P(s_out),
+        B, N, C_S, PAIR_BIAS_HEADS, C_HEAD_S, 1e9, 0, P(s_ws), s_ws.numel(), _lib.OF3_DTYPE_BF16, s)))]
     launches = (trimul("tri_mul_out.", 1) + trimul("tri_mul_in.", 0)
                 + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr) + transition
-                + pair_bias + template_tail)
+                + pair_bias + attn_pair_bias + template_tail)
     for _ in range(max(args.warmup, 1)):
         for _, fn in launches:
             fn()

@@ -29,6 +29,8 @@
  *                 linear_out, mask)                             -> of3_transition_fwd
  *   openfold3/core/model/layers/attention_pair_bias.py
  *       :151-161  _prep_bias: layer_norm_z, linear_z, permute   -> of3_pair_bias_fwd
+ *       :189-244  AttentionPairBias.forward of the trunk (no AdaLN): layer_norm_a, mask bias,
+ *                 Attention (attention.py:265-302, :94-135)     -> of3_attn_pair_bias_fwd
  *   openfold3/core/model/latent/template_module.py
  *       :376      TemplatePairStack's closing LayerNorm
  *                 (openfold3/core/model/primitives/normalization.py:65-84) -> of3_layer_norm_fwd
@@ -169,6 +171,22 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
  * offset); w is [H][C].  No workspace.  bf16: C in {64, 128}, H <= 32; fp32: C <= 256, H <= 64. */
 int of3_pair_bias_fwd(const void* z, const int64_t z_strides[3], const void* ln_w, const void* ln_b, const void* w,
                       void* out, int64_t B, int64_t N, int64_t C, int64_t H, int dtype, void* stream);
+
+/* ---- single-representation attention with pair bias ------------------------------------ */
+
+/* out = [a +] (softmax_k(q k^T / sqrt(D) + inf*(mask[k]-1) + pair_bias[h][q][k]) v * sigmoid(an Wg^T)) Wo^T
+ * with an = LayerNorm(a), q = an Wq^T + bq, k = an Wk^T, v = an Wv^T split into H heads of width D.
+ * a, out: contiguous [B][N][C_s] (out may alias a); pair_bias: contiguous [B][H][N][N], what
+ * of3_pair_bias_fwd returns for this module's layer_norm_z / linear_z; mask: fp32 [B][N] or null
+ * (all ones); w_q, w_k, w_v, w_g: [H*D][C_s]; b_q: [H*D]; w_o: [C_s][H*D].  bf16 only, the AF3
+ * trunk shape: C_s = H*D = 384, D a multiple of 8 up to 32 (16 heads of 24).  The workspace holds
+ * q, k, v, the gate and the gated attention output. */
+int64_t of3_attn_pair_bias_workspace_bytes(int64_t B, int64_t N, int64_t C_s, int64_t H, int64_t D);
+int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* mask, const void* ln_w,
+                           const void* ln_b, const void* w_q, const void* b_q, const void* w_k, const void* w_v,
+                           const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C_s, int64_t H,
+                           int64_t D, float inf, int add_residual, void* workspace, int64_t workspace_bytes,
+                           int dtype, void* stream);
 
 /* ---- template branch: closing LayerNorm and embedder tail ------------------------------ */
 

@@ -132,6 +132,22 @@ hipError_t template_tail_fwd_f32(const TemplateTailF32Args& args, hipStream_t st
 hipError_t layer_norm_fwd_f32(const float* x, const float* w, const float* b, float* out, long rows, int C,
                               hipStream_t stream);
 
+// ---- single-representation attention with pair bias (single_attn.hip), bf16, c_s = H*D = 384
+struct SingleAttnArgs {
+  const bf16_t* a;            // [B][N][c_s]
+  const bf16_t* pair_bias;    // [B][H][N][N], the pair-bias projection of z
+  const float* mask;          // [B][N] or null
+  const bf16_t *ln_w, *ln_b;  // layer_norm_a
+  const bf16_t *wq, *bq, *wk, *wv, *wg, *wo;
+  bf16_t *q, *k;              // workspace, [B][H][Np][32] (head width padded with zeros)
+  bf16_t* vt;                 // workspace, [B][H][32][Np]
+  bf16_t *g, *og;             // workspace, [B][N][H*D]: gate after the sigmoid, gated attention output
+  bf16_t* out;                // [B][N][c_s]; may alias a
+  float inf;
+  int B, N, Np, H, D, add_residual;  // Np = N rounded up to a multiple of 32
+};
+hipError_t single_attn_launch(const SingleAttnArgs& args, hipStream_t stream);
+
 // ---- fp32 path (pair_f32.hip): whole updates, any N, C and C_hidden <= 256, head width 16/32/64
 struct TrimulF32Args {
   const float* z;

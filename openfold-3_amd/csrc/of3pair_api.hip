@@ -556,4 +556,56 @@ int of3_template_tail_fwd(const void* t, const void* ln_w, const void* ln_b, con
   return e == hipSuccess ? OF3_OK : fail_hip(e);
 }
 
+int64_t of3_attn_pair_bias_workspace_bytes(int64_t B, int64_t N, int64_t C_s, int64_t H, int64_t D) {
+  if (B < 1 || N < 1 || N > (1 << 16) || C_s != 384 || H < 1 || D < 8 || D > 32 || (D % 8) != 0 || H * D != C_s)
+    return OF3_EINVAL;
+  const int64_t Np = (N + 31) / 32 * 32;
+  return 3 * align256(B * H * Np * 32 * 2) + 2 * align256(B * N * H * D * 2);
+}
+
+int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* mask, const void* ln_w,
+                           const void* ln_b, const void* w_q, const void* b_q, const void* w_k, const void* w_v,
+                           const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C_s, int64_t H,
+                           int64_t D, float inf, int add_residual, void* workspace, int64_t workspace_bytes,
+                           int dtype, void* stream) {
+  if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
+  const int64_t need = of3_attn_pair_bias_workspace_bytes(B, N, C_s, H, D);
+  if (need < 0 || B > 65535) return OF3_EINVAL;
+  const void* ptrs[] = {a, pair_bias, ln_w, ln_b, w_q, b_q, w_k, w_v, w_g, w_o, out, workspace};
+  for (const void* p : ptrs)
+    if (!p || !aligned16(p)) return OF3_EINVAL;
+  if (mask && !aligned4(mask)) return OF3_EINVAL;
+  if (workspace_bytes < need) return OF3_ENOSPC;
+  const int64_t Np = (N + 31) / 32 * 32;
+  const int64_t qk = align256(B * H * Np * 32 * 2), go = align256(B * N * H * D * 2);
+  char* ws = static_cast<char*>(workspace);
+  of3::SingleAttnArgs s;
+  s.a = bf(a);
+  s.pair_bias = bf(pair_bias);
+  s.mask = mask;
+  s.ln_w = bf(ln_w);
+  s.ln_b = bf(ln_b);
+  s.wq = bf(w_q);
+  s.bq = bf(b_q);
+  s.wk = bf(w_k);
+  s.wv = bf(w_v);
+  s.wg = bf(w_g);
+  s.wo = bf(w_o);
+  s.q = reinterpret_cast<of3::bf16_t*>(ws);
+  s.k = reinterpret_cast<of3::bf16_t*>(ws + qk);
+  s.vt = reinterpret_cast<of3::bf16_t*>(ws + 2 * qk);
+  s.g = reinterpret_cast<of3::bf16_t*>(ws + 3 * qk);
+  s.og = reinterpret_cast<of3::bf16_t*>(ws + 3 * qk + go);
+  s.out = bf(out);
+  s.inf = inf;
+  s.B = (int)B;
+  s.N = (int)N;
+  s.Np = (int)Np;
+  s.H = (int)H;
+  s.D = (int)D;
+  s.add_residual = add_residual ? 1 : 0;
+  hipError_t e = of3::single_attn_launch(s, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
 }  // extern "C"

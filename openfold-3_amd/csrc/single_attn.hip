@@ -1,0 +1,350 @@
+// Single-representation attention with pair bias, the trunk's AttentionPairBias
+// (attention_pair_bias.py:189-244 with Attention._prep_qkv / _attention / _wrap_up,
+// attention.py:265-302, :94-135), once per PairFormerBlock (pairformer.py:189-201):
+//     an = LN(a);  q = (an Wq^T + bq) / sqrt(D), k = an Wk^T, v = an Wv^T      (H heads of width D)
+//     s[h][q][k] = q.k + inf * (mask[k] - 1) + pair_bias[h][q][k];  p = softmax_k(s);  o = p v
+//     out = [a +] (o * sigmoid(an Wg^T)) Wo^T
+// The pair bias [B][H][N][N] is the output of the pair-bias projection kernel.  With N tokens of
+// c_s = 384 channels the whole module is about 2 GFLOP at N = 768: three small kernels.
+//
+//  1. single_proj: a work-group normalises 32 positions into an LDS tile [position][channel]
+//     (bf16, 16-byte chunks XOR-swizzled by the position) and its waves compute 32-wide output
+//     tiles with K = c_s MFMA steps, the weights read straight from global memory (they stay in
+//     L2).  A tile is one head of one of q, k, v, g, padded from D = 24 to 32 channels with zero
+//     weight rows, so q and k come out as [B][H][Np][32] with zero padding.  For q, k and g the
+//     weights are the A operand (rows dealt by rowperm16: a lane ends up with 16 consecutive
+//     channels of one position); for v the positions are the A operand, so that a lane holds one
+//     channel of 4-position runs and V^T [B][H][32][Np] is written with 8-byte stores.
+//     q carries log2(e) / sqrt(D) (the softmax below uses exp2), g is stored after the sigmoid.
+//  2. single_attn: one wave per (batch, head, 32 queries), flash style over 32-key tiles:
+//     S^T = K Q^T with the accumulator initialised to (pair bias + mask bias) * log2(e), running
+//     maximum and sum in fp32, O^T = V^T P^T with P^T taken from the S^T registers; the result
+//     is divided by the sum, multiplied by the gate and written as [B][N][H*D].
+//  3. single_out: the same tiling as 1 without the LayerNorm: out = [a +] og Wo^T.
+#include "of3_device.h"
+#include "of3_kernels.h"
+
+namespace of3 {
+
+namespace {
+
+constexpr int kK = 384;          // c_s = H * D: reduction length of both linear stages
+constexpr int kChunks = kK / 8;  // 16-byte chunks per position
+constexpr int kDP = 32;          // head width padded to one MFMA tile
+
+__device__ __forceinline__ float xhalf(float v) { return __shfl_xor(v, 32, 64); }
+
+// LDS tile [32 positions][kChunks]: chunk index XOR position in its low four bits (the 16 lanes
+// of a read phase hold 16 consecutive positions at one chunk index and must hit 16 bank windows;
+// a row is 768 bytes = 3 windows of 256, so without the key they would all hit the same one)
+__device__ __forceinline__ int act_slot(int pos, int chunk) { return pos * kChunks + ((chunk & ~15) | ((chunk ^ pos) & 15)); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// rows pos0 .. pos0+31 of src [rows][kK] into the LDS tile; with LN, normalised (statistics in
+// fp32, result rounded to bf16 as the reference's LayerNorm output).  Wave w handles 8 rows, lanes
+// 0..47 one chunk each.  Rows past n_rows repeat the last one (never stored by the callers).
+template <bool LN>
+__device__ __forceinline__ void fill_tile(u32x4_t* act, const bf16_t* __restrict__ src, long pos0, long n_rows,
+                                          const bf16_t* __restrict__ ln_w, const bf16_t* __restrict__ ln_b, int wave,
+                                          int lane) {
+  const bool has = lane < kChunks;
+  float lw[8], lb[8];
+  if (LN && has) {
+    load_affine8(ln_w, lane, lw);
+    load_affine8(ln_b, lane, lb);
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const int pos = 8 * wave + r;
+    long row = pos0 + pos;
+    row = row < n_rows ? row : n_rows - 1;
+    u32x4_t raw = {0u, 0u, 0u, 0u};
+    if (has) raw = *reinterpret_cast<const u32x4_t*>(src + row * kK + 8 * lane);
+    if (LN) {
+      float x[8];
+      unpack8(raw, x);
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s += x[i];
+      const float mean = wave_sum(s) * (1.f / kK);
+      float q = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        x[i] = has ? x[i] - mean : 0.f;
+        q += x[i] * x[i];
+      }
+      const float rstd = __builtin_amdgcn_rsqf(wave_sum(q) * (1.f / kK) + kLnEps);
+      if (has) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = x[i] * rstd * lw[i] + lb[i];
+        raw = pack8(x);
+      }
+    }
+    if (has) act[act_slot(pos, lane)] = raw;
+  }
+}
+
+// 32 x 32 output tile with K = kK: `w_row` points at the weight row this lane feeds (or is null
+// for a zero row), positions come from the LDS tile.  WEIGHTS_ARE_A: result lane (position l32,
+// half lh) holds w-rows 16*lh + v (the caller dealt the rows by rowperm16); otherwise lane
+// (w-row l32, half lh) holds positions 8*(v/4) + 4*lh + (v%4).
+template <bool WEIGHTS_ARE_A>
+__device__ __forceinline__ f32x16_t tile_product(const u32x4_t* act, const bf16_t* __restrict__ w_row, int l32, int lh) {
+  f32x16_t acc = zero16();
+#pragma unroll 6
+  for (int s = 0; s < kK / 16; ++s) {
+    u32x4_t w = {0u, 0u, 0u, 0u};
+    if (w_row) w = *reinterpret_cast<const u32x4_t*>(w_row + 16 * s + 8 * lh);
+    const u32x4_t x = act[act_slot(l32, 2 * s + lh)];
+    acc = WEIGHTS_ARE_A ? mfma_32x32x16(w, x, acc) : mfma_32x32x16(x, w, acc);
+  }
+  return acc;
+}
+
+// ---- 1. LayerNorm + q, k, v, g ------------------------------------------------------------
+__global__ __launch_bounds__(256) void single_proj_kernel(SingleAttnArgs p) {
+  __shared__ u32x4_t act[32 * kChunks];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int N = p.N, Np = p.Np, H = p.H, D = p.D;
+  const int b = blockIdx.z;
+  const long pos0 = (long)blockIdx.x * 32;
+  fill_tile<true>(act, p.a + (size_t)b * N * kK, pos0, N, p.ln_w, p.ln_b, wave, lane);
+  __syncthreads();
+
+  const long pos = pos0 + l32;  // position of this lane in the weights-are-A tiles
+  const float q_scale = kLog2e * __builtin_amdgcn_rsqf((float)D);
+  for (int tile = blockIdx.y * 4 + wave; tile < 4 * H; tile += gridDim.y * 4) {
+    const int kind = tile / H, h = tile - kind * H;  // 0 q, 1 k, 2 v, 3 g
+    if (kind != 2) {
+      const bf16_t* W = kind == 0 ? p.wq : (kind == 1 ? p.wk : p.wg);
+      const int dch = rowperm16(l32);
+      const f32x16_t acc = tile_product<true>(act, dch < D ? W + (size_t)(h * D + dch) * kK : nullptr, l32, lh);
+      // lane (position, half lh): padded channels 16*lh + v
+      float f[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) f[v] = acc[v];
+      if (kind == 0) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int d = 16 * lh + v;
+          f[v] = d < D ? (f[v] + bf16_to_f32(p.bq[h * D + d])) * q_scale : 0.f;
+        }
+      } else if (kind == 3) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) f[v] = sigmoidf_fast(f[v]);
+      }
+      u32x4_t o0, o1;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        o0[w] = pack_bf16(f[2 * w], f[2 * w + 1]);
+        o1[w] = pack_bf16(f[8 + 2 * w], f[8 + 2 * w + 1]);
+      }
+      if (kind == 3) {
+        if (pos < N) {
+          bf16_t* dst = p.g + ((size_t)b * N + pos) * (H * D) + h * D + 16 * lh;
+          if (16 * lh < D) *reinterpret_cast<u32x4_t*>(dst) = o0;
+          if (16 * lh + 8 < D) *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
+        }
+      } else if (pos < Np) {
+        if (pos >= N) {  // padded key rows are read by the attention kernel: zeros
+          o0 = u32x4_t{0u, 0u, 0u, 0u};
+          o1 = o0;
+        }
+        bf16_t* dst = (kind == 0 ? p.q : p.k) + (((size_t)b * H + h) * Np + pos) * kDP + 16 * lh;
+        *reinterpret_cast<u32x4_t*>(dst) = o0;
+        *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
+      }
+    } else {
+      const f32x16_t acc = tile_product<false>(act, l32 < D ? p.wv + (size_t)(h * D + l32) * kK : nullptr, l32, lh);
+      // lane (padded channel l32, half lh): positions pos0 + 8*(v/4) + 4*lh + (v%4)
+      bf16_t* row = p.vt + (((size_t)b * H + h) * kDP + l32) * Np;
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const long pp = pos0 + 8 * g4 + 4 * lh;
+        if (pp < Np) {
+          float f[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) f[e] = pp + e < N ? acc[4 * g4 + e] : 0.f;  // padded keys: zeros
+          u32x2_t o = {pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3])};
+          *reinterpret_cast<u32x2_t*>(row + pp) = o;
+        }
+      }
+    }
+  }
+}
+
+// ---- 2. attention core -------------------------------------------------------------------
+// 16 consecutive bf16 / fp32 values starting at element `first` of a row of `n` valid elements,
+// as floats; elements at or past n give `fill`
+__device__ __forceinline__ void load16_bf16(const bf16_t* __restrict__ row, int first, int n, bool vec_ok, float fill,
+                                            float (&out)[16]) {
+  if (vec_ok && first + 16 <= n) {
+    float lo[8], hi[8];
+    unpack8(*reinterpret_cast<const u32x4_t*>(row + first), lo);
+    unpack8(*reinterpret_cast<const u32x4_t*>(row + first + 8), hi);
+#pragma unroll
+    for (int v = 0; v < 8; ++v) out[v] = lo[v], out[8 + v] = hi[v];
+  } else {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) out[v] = first + v < n ? bf16_to_f32(row[first + v]) : fill;
+  }
+}
+
+__global__ __launch_bounds__(256) void single_attn_kernel(SingleAttnArgs p, int q_tiles) {
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int N = p.N, Np = p.Np, H = p.H, D = p.D;
+  const int qt = blockIdx.x * 4 + wave;
+  if (qt >= q_tiles) return;  // whole wave; the kernel has no barrier
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int q0 = qt * 32;
+  int qrow = q0 + l32;
+  const bool q_valid = qrow < N;
+  qrow = q_valid ? qrow : N - 1;
+
+  const size_t bh = (size_t)b * H + h;
+  const bf16_t* Q = p.q + (bh * Np + qrow) * kDP;
+  const bf16_t* K = p.k + bh * Np * kDP;
+  const bf16_t* Vt = p.vt + bh * kDP * Np;
+  const bf16_t* pb_row = p.pair_bias + (bh * N + qrow) * N;
+  const float* mask = p.mask ? p.mask + (size_t)b * N : nullptr;
+  const bool vec_ok = (N % 8) == 0;  // 16-byte aligned runs of the bias rows
+  const float mscale = p.inf * kLog2e;
+
+  u32x4_t qop[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) qop[s] = *reinterpret_cast<const u32x4_t*>(Q + 16 * s + 8 * lh);
+  const int krow = rowperm16(l32);
+
+  float m_run = -__builtin_inff(), l_run = 0.f;
+  f32x16_t oacc = zero16();
+  const int nkt = (N + 31) / 32;
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int k0 = 32 * kt;
+    u32x4_t kc[2], vc[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) kc[s] = *reinterpret_cast<const u32x4_t*>(K + (size_t)(k0 + krow) * kDP + 16 * s + 8 * lh);
+    // V^T rows = padded channels dealt by rowperm16; lane-half lh, k-step s2 feeds keys 16*lh + 8*s2 .. +7,
+    // the keys that registers 8*s2 .. 8*s2+7 of the same lane-half hold in S^T
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) vc[s2] = *reinterpret_cast<const u32x4_t*>(Vt + (size_t)krow * Np + k0 + 16 * lh + 8 * s2);
+
+    // this lane's 16 keys of the tile: k0 + 16*lh + v
+    float bias[16];
+    load16_bf16(pb_row, k0 + 16 * lh, N, vec_ok, 0.f, bias);
+    f32x16_t s;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = k0 + 16 * lh + v;
+      float mb = 0.f;
+      if (key >= N) mb = -__builtin_inff();  // padded keys: weight exactly zero
+      else if (mask) mb = mscale * (mask[key] - 1.f);
+      s[v] = bias[v] * kLog2e + mb;
+    }
+    s = mfma_32x32x16(kc[0], qop[0], s);
+    s = mfma_32x32x16(kc[1], qop[1], s);
+
+    float mx = s[0];
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+    const float m_new = fmaxf(m_run, fmaxf(mx, xhalf(mx)));  // every tile holds at least one real key
+    const float alpha = fast_exp2(m_run - m_new);            // exp2(-inf) = 0 on the first tile
+    l_run *= alpha;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) oacc[v] *= alpha;
+    m_run = m_new;
+    u32x4_t pop[2];
+    float rs = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) {
+      const uint32_t pk = pack_bf16(fast_exp2(s[2 * w] - m_new), fast_exp2(s[2 * w + 1] - m_new));
+      rs += bf16_lo(pk) + bf16_hi(pk);  // the sum of the weights the P V product uses
+      pop[w >> 2][w & 3] = pk;
+    }
+    l_run += rs;
+    oacc = mfma_32x32x16(vc[0], pop[0], oacc);
+    oacc = mfma_32x32x16(vc[1], pop[1], oacc);
+  }
+
+  // lane (query l32, half lh) owns head channels 16*lh + v
+  const float inv = fast_rcp(l_run + xhalf(l_run));
+  if (q_valid && 16 * lh < D) {
+    const size_t off = ((size_t)b * N + qrow) * (H * D) + h * D + 16 * lh;
+    float gate[16];
+    load16_bf16(p.g + off, 0, D - 16 * lh, true, 0.f, gate);
+    u32x4_t o0, o1;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      o0[w] = pack_bf16(oacc[2 * w] * inv * gate[2 * w], oacc[2 * w + 1] * inv * gate[2 * w + 1]);
+      o1[w] = pack_bf16(oacc[8 + 2 * w] * inv * gate[8 + 2 * w], oacc[8 + 2 * w + 1] * inv * gate[8 + 2 * w + 1]);
+    }
+    bf16_t* dst = p.og + off;
+    *reinterpret_cast<u32x4_t*>(dst) = o0;
+    if (16 * lh + 8 < D) *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
+  }
+}
+
+// ---- 3. output projection ----------------------------------------------------------------
+__global__ __launch_bounds__(256) void single_out_kernel(SingleAttnArgs p) {
+  __shared__ u32x4_t act[32 * kChunks];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int N = p.N;
+  const int b = blockIdx.z;
+  const long pos0 = (long)blockIdx.x * 32;
+  fill_tile<false>(act, p.og + (size_t)b * N * kK, pos0, N, nullptr, nullptr, wave, lane);
+  __syncthreads();
+  const long pos = pos0 + l32;
+  for (int tile = blockIdx.y * 4 + wave; tile < kK / 32; tile += gridDim.y * 4) {
+    const f32x16_t acc = tile_product<true>(act, p.wo + (size_t)(32 * tile + rowperm16(l32)) * kK, l32, lh);
+    if (pos < N) {
+      const size_t off = ((size_t)b * N + pos) * kK + 32 * tile + 16 * lh;
+      float f[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) f[v] = acc[v];
+      if (p.add_residual) {
+        // the reference adds the module's bf16 output to s: round before the add
+        float r[16];
+        load16_bf16(p.a + off, 0, 16, true, 0.f, r);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) f[v] = bf16_to_f32(to_bf16(f[v])) + r[v];
+      }
+      u32x4_t o0, o1;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        o0[w] = pack_bf16(f[2 * w], f[2 * w + 1]);
+        o1[w] = pack_bf16(f[8 + 2 * w], f[8 + 2 * w + 1]);
+      }
+      *reinterpret_cast<u32x4_t*>(p.out + off) = o0;
+      *reinterpret_cast<u32x4_t*>(p.out + off + 8) = o1;
+    }
+  }
+}
+
+}  // namespace
+
+hipError_t single_attn_launch(const SingleAttnArgs& a, hipStream_t stream) {
+  if (a.H * a.D != kK || a.D > kDP || (a.D % 8) != 0 || a.H < 1 || a.N < 1 || a.B < 1 || a.B > 65535 || a.H > 65535)
+    return hipErrorInvalidValue;
+  if (a.Np != (a.N + 31) / 32 * 32) return hipErrorInvalidValue;
+  const int row_blocks = a.Np / 32;
+  hipLaunchKernelGGL(single_proj_kernel, dim3(row_blocks, 4, a.B), dim3(256), 0, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(single_attn_kernel, dim3((row_blocks + 3) / 4, a.H, a.B), dim3(256), 0, stream, a, row_blocks);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(single_out_kernel, dim3(row_blocks, 3, a.B), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+}  // namespace of3

@@ -1,6 +1,6 @@
 """of3pair: MI355X-native kernels for the OpenFold3 Pairformer pair stack (triangle
 multiplicative updates, triangle attention and the pair transition) behind the reference's layer-module API."""
-from .layers import (PairBiasProjection, SwiGLUTransition, TriangleAttention, TriangleAttentionEndingNode, TriangleAttentionStartingNode,
+from .layers import (AttentionPairBias, PairBiasProjection, SwiGLUTransition, TriangleAttention, TriangleAttentionEndingNode, TriangleAttentionStartingNode,
                      TriangleMultiplicationIncoming, TriangleMultiplicationOutgoing,
                      TriangleMultiplicativeUpdate)
 from .pair_stack import PairBlock, PairStack
@@ -9,6 +9,6 @@ from . import checkpoint
 
 __all__ = [
     "TriangleMultiplicativeUpdate", "TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming",
-    "TriangleAttention", "TriangleAttentionStartingNode", "TriangleAttentionEndingNode", "SwiGLUTransition", "PairBiasProjection",
+    "TriangleAttention", "TriangleAttentionStartingNode", "TriangleAttentionEndingNode", "SwiGLUTransition", "PairBiasProjection", "AttentionPairBias",
     "PairStack", "PairBlock", "TemplatePairBlock", "TemplatePairStack", "TemplateEmbedderCore", "checkpoint",
 ]

@@ -29,6 +29,7 @@ SOURCES = [
     "transition.hip",
     "pair_bias.hip",
     "template_tail.hip",
+    "single_attn.hip",
     "pair_f32.hip",
 ]
 

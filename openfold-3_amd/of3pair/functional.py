@@ -265,3 +265,46 @@ def template_tail(t, norm_weight, norm_bias, linear_t_weight, apply_layer_norm: 
                          "in %s" % (CT, CZ, t.dtype))
     _lib.check(st, "of3_template_tail_fwd")
     return out
+
+
+def attention_pair_bias(a, z, mask, norm_a_weight, norm_a_bias, norm_z_weight, norm_z_bias, z_weight, q_weight,
+                        q_bias, k_weight, v_weight, g_weight, o_weight, no_heads: int, inf: float = 1e9,
+                        add_residual: bool = False, inplace: bool = False):
+    """AttentionPairBias.forward of the trunk (attention_pair_bias.py:189-244): attention over
+    the single representation a [*, N, C_s] with the pair bias of z [*, N, N, C_z] and the key
+    mask [*, N].  Returns the update (or a + update with add_residual; inplace writes into a).
+    bf16 only, C_s = no_heads * head width = 384."""
+    code = _require_gpu(a, "a")
+    if a.dtype != torch.bfloat16:
+        raise ValueError("attention_pair_bias: the kernels are bf16 only, got %s" % a.dtype)
+    lib = _lib.load()
+    bias = pair_bias(z, norm_z_weight, norm_z_bias, z_weight)  # [*, H, N, N]
+    lead = a.shape[:-2]
+    N, CS = a.shape[-2:]
+    B = 1
+    for d in lead:
+        B *= d
+    H = no_heads
+    HD = q_weight.shape[0]
+    if HD % H or tuple(q_weight.shape) != (HD, CS) or tuple(o_weight.shape) != (CS, HD):
+        raise ValueError("attention_pair_bias: weights must be [H*c, C_s] and linear_o [C_s, H*c]")
+    D = HD // H
+    if tuple(bias.shape[-3:]) != (H, N, N) or bias.numel() != B * H * N * N:
+        raise ValueError("attention_pair_bias: z must be [*, N, N, C_z] with a's leading dimensions")
+    ac = a if a.is_contiguous() else a.contiguous()
+    out = ac if (inplace and ac is a) else torch.empty_like(ac)
+    m = None
+    if mask is not None:
+        m = mask.to(torch.float32).expand(*lead, N).contiguous()
+    need = lib.of3_attn_pair_bias_workspace_bytes(B, N, CS, H, D)
+    if need < 0:
+        raise ValueError("attention_pair_bias: supported shape is C_s = no_heads * c = 384 with c a multiple of 8 "
+                         "up to 32; got C_s=%d heads=%d c=%d" % (CS, H, D))
+    ws = _workspace(a.device, need)
+    w = [_w(t, a.dtype) for t in (norm_a_weight, norm_a_bias, q_weight, q_bias, k_weight, v_weight, g_weight, o_weight)]
+    with torch.cuda.device(a.device):
+        st = lib.of3_attn_pair_bias_fwd(ac.data_ptr(), bias.data_ptr(), None if m is None else m.data_ptr(),
+                                        *[t.data_ptr() for t in w], out.data_ptr(), B, N, CS, H, D, float(inf),
+                                        1 if add_residual else 0, ws.data_ptr(), ws.numel(), code, _stream(a))
+    _lib.check(st, "of3_attn_pair_bias_fwd")
+    return out

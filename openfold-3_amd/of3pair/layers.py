@@ -256,3 +256,66 @@ class PairBiasProjection(nn.Module):
     @torch.no_grad()
     def forward(self, z):
         return F3.pair_bias(z, self.layer_norm_z.weight, self.layer_norm_z.bias, self.linear_z.weight)
+
+
+class _PairBiasAttentionParams(nn.Module):
+    """Parameter holder with the names of the reference's Attention inside AttentionPairBias
+    (attention.py:236-258 with default_linear_init_config.py:56-64: linear_q carries a bias)."""
+
+    def __init__(self, c_q, c_hidden, no_heads, init):
+        super().__init__()
+        hc = c_hidden * no_heads
+        self.linear_q = nn.Linear(c_q, hc, bias=True)
+        self.linear_k = nn.Linear(c_q, hc, bias=False)
+        self.linear_v = nn.Linear(c_q, hc, bias=False)
+        self.linear_o = nn.Linear(hc, c_q, bias=False)
+        self.linear_g = nn.Linear(c_q, hc, bias=False)
+        for name, default in (("linear_q", "default"), ("linear_k", "default"), ("linear_v", "default"),
+                              ("linear_g", "gating"), ("linear_o", "final")):
+            spec = None if init is None else (init.get(name) if hasattr(init, "get") else init[name])
+            how = default if spec is None else (spec if isinstance(spec, str) else spec.get("init", default))
+            _init_linear(getattr(self, name), how)
+        with torch.no_grad():
+            self.linear_q.bias.zero_()
+
+
+class AttentionPairBias(nn.Module):
+    """The trunk's AttentionPairBias (attention_pair_bias.py:33-244, AF3 Algorithm 24 without
+    AdaLN): same constructor arguments, parameter names (layer_norm_a, layer_norm_z, linear_z,
+    mha.linear_q/k/v/g/o) and forward signature.  use_ada_layer_norm (the diffusion variant) and
+    ungated attention are not implemented."""
+
+    def __init__(self, c_q, c_k, c_v, c_s, c_z, c_hidden, no_heads, use_ada_layer_norm=False, gating=True, inf=1e9,
+                 linear_init_params=None):
+        super().__init__()
+        if use_ada_layer_norm or not gating:
+            raise ValueError("only the trunk variant (LayerNorm, gated) is implemented")
+        if not (c_q == c_k == c_v):
+            raise ValueError("self-attention over one representation: c_q = c_k = c_v")
+        self.c_q, self.c_s, self.c_z, self.inf, self.no_heads = c_q, c_s, c_z, inf, no_heads
+        self.use_ada_layer_norm = False
+        offset = True
+        mha_init = None
+        if linear_init_params is not None:
+            lz = linear_init_params.get("layer_norm_z") if hasattr(linear_init_params, "get") else None
+            if lz is not None:
+                offset = bool(lz.get("create_offset", True))
+            mha_init = linear_init_params.get("mha") if hasattr(linear_init_params, "get") else None
+        self.layer_norm_a = nn.LayerNorm(c_q, eps=1e-5)
+        self.layer_norm_z = nn.LayerNorm(c_z, eps=1e-5, bias=offset)
+        self.linear_z = nn.Linear(c_z, no_heads, bias=False)
+        _init_linear(self.linear_z, _init_name(linear_init_params, "linear_z", "default"))
+        self.mha = _PairBiasAttentionParams(c_q, c_hidden, no_heads, mha_init)
+
+    @torch.no_grad()
+    def forward(self, a, z, s=None, mask=None, use_deepspeed_evo_attention=False, use_cueq_triangle_kernels=False,
+                use_lma=False, use_high_precision_attention=False, _add_residual: bool = False,
+                _inplace: bool = False):
+        """a [*, N, C_q], z [*, N, N, C_z], mask [*, N] -> the update [*, N, C_q]
+        (a + update with _add_residual, written into a with _inplace)."""
+        m = self.mha
+        return F3.attention_pair_bias(
+            a, z, mask, self.layer_norm_a.weight, self.layer_norm_a.bias, self.layer_norm_z.weight,
+            self.layer_norm_z.bias, self.linear_z.weight, m.linear_q.weight, m.linear_q.bias, m.linear_k.weight,
+            m.linear_v.weight, m.linear_g.weight, m.linear_o.weight, no_heads=self.no_heads, inf=self.inf,
+            add_residual=_add_residual, inplace=_inplace)

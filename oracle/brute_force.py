@@ -183,3 +183,41 @@ def template_tail(t, ln_w, ln_b, w):
             for o in range(w.shape[0]):
                 out[i, j, o] = (w[o] * acc).sum()
     return out
+
+
+def attention_pair_bias(a, z, mask, p, no_heads, inf=1e9):
+    """float64 loops over (head, query, key) for a [N, C_s], z [N, N, C_z], mask [N]
+    (attention_pair_bias.py:189-244, attention.py:94-135, :265-302)."""
+    a = np.asarray(a, dtype=np.float64)
+    z = np.asarray(z, dtype=np.float64)
+    P = {k: np.asarray(v, dtype=np.float64) for k, v in p.items()}
+    n, cs = a.shape
+    hc = P["mha.linear_q.weight"].shape[0]
+    c = hc // no_heads
+    mask = np.ones(n) if mask is None else np.asarray(mask, dtype=np.float64)
+    an = np.stack([_ln(a[i], P["layer_norm_a.weight"], P["layer_norm_a.bias"]) for i in range(n)])
+    zb_b = P.get("layer_norm_z.bias", np.zeros_like(P["layer_norm_z.weight"]))
+    q = np.zeros((n, hc)); k = np.zeros((n, hc)); v = np.zeros((n, hc)); g = np.zeros((n, hc))
+    for i in range(n):
+        for o in range(hc):
+            q[i, o] = ((an[i] * P["mha.linear_q.weight"][o]).sum() + P["mha.linear_q.bias"][o]) / math.sqrt(c)
+            k[i, o] = (an[i] * P["mha.linear_k.weight"][o]).sum()
+            v[i, o] = (an[i] * P["mha.linear_v.weight"][o]).sum()
+            g[i, o] = _sig((an[i] * P["mha.linear_g.weight"][o]).sum())
+    og = np.zeros((n, hc))
+    for h in range(no_heads):
+        sl = slice(h * c, (h + 1) * c)
+        for i in range(n):
+            logits = np.zeros(n)
+            for j in range(n):
+                zn = _ln(z[i, j], P["layer_norm_z.weight"], zb_b)
+                logits[j] = (q[i, sl] * k[j, sl]).sum() + inf * (mask[j] - 1) + (zn * P["linear_z.weight"][h]).sum()
+            w = np.exp(logits - logits.max())
+            w /= w.sum()
+            for d in range(c):
+                og[i, h * c + d] = (w * v[:, h * c + d]).sum() * g[i, h * c + d]
+    out = np.zeros((n, cs))
+    for i in range(n):
+        for o in range(cs):
+            out[i, o] = (og[i] * P["mha.linear_o.weight"][o]).sum()
+    return out

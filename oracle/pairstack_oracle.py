@@ -14,7 +14,9 @@ reference's stock (no alternative kernel) path through
       openfold3/core/model/latent/base_blocks.py:307-406,
   * TemplatePairBlock.forward (per-template loop, tri_mul_first=True), TemplatePairStack.forward
     with its final LayerNorm, and the mean / ReLU / linear_t tail of TemplateEmbedderAllAtom
-      openfold3/core/model/latent/template_module.py:148-193, :302-378, :462-465.
+      openfold3/core/model/latent/template_module.py:148-193, :302-378, :462-465,
+  * AttentionPairBias.forward of the trunk (single representation, pair bias from z)
+      openfold3/core/model/layers/attention_pair_bias.py:121-244.
 
 It may be imported by tests/, by __graft_entry__.smoke() and by the
 cpu_baseline leg of bench.py, as the checker or the timed CPU baseline.
@@ -200,6 +202,55 @@ def pair_bias(z, p):
     zn = layer_norm(z, p["layer_norm_z.weight"], bias)
     out = linear(zn, p["linear_z.weight"])
     return out.movedim(-1, -3)
+
+
+def attention_pair_bias(a, z, mask, p, no_heads: int, inf: float = INF):
+    """AttentionPairBias.forward of the trunk (no AdaLN; attention_pair_bias.py:189-244) with
+    Attention._prep_qkv / _attention / _wrap_up (attention.py:265-302, :94-135).
+
+    a: [*, N, C_s]; z: [*, N, N, C_z]; mask: [*, N] or None.  Returns the update [*, N, C_s]
+    (the caller adds it to s, pairformer.py:189-201).  Parameters under the reference's names:
+    layer_norm_a.*, layer_norm_z.*, linear_z.weight, mha.linear_q.weight / .bias,
+    mha.linear_k.weight, mha.linear_v.weight, mha.linear_g.weight, mha.linear_o.weight.
+    """
+    if mask is None:
+        mask = a.new_ones(a.shape[:-1])
+    an = layer_norm(a, p["layer_norm_a.weight"], p["layer_norm_a.bias"])
+    mask_bias = (inf * (mask.to(a.dtype) - 1))[..., None, None, :]   # [*, 1, 1, N]
+    zb = pair_bias(z, p)                                              # [*, H, N, N]
+    c = p["mha.linear_q.weight"].shape[0] // no_heads
+
+    def heads(t):  # [*, N, H*c] -> [*, H, N, c]
+        return t.view(*t.shape[:-1], no_heads, c).transpose(-2, -3)
+
+    q = heads(linear(an, p["mha.linear_q.weight"]) + p["mha.linear_q.bias"]) / math.sqrt(c)
+    k = heads(linear(an, p["mha.linear_k.weight"]))
+    v = heads(linear(an, p["mha.linear_v.weight"]))
+    o = attention_core(q, k, v, [mask_bias, zb])                      # [*, H, N, c]
+    o = o.transpose(-2, -3)                                           # [*, N, H, c]
+    g = torch.sigmoid(linear(an, p["mha.linear_g.weight"]))
+    o = o.reshape(*o.shape[:-2], no_heads * c) * g
+    return linear(o, p["mha.linear_o.weight"])
+
+
+def make_attention_pair_bias_params(gen, c_s: int, c_z: int, c_head: int, no_heads: int):
+    hc = c_head * no_heads
+
+    def lin(o, i):
+        return torch.randn(o, i, generator=gen) / math.sqrt(i)
+
+    p = {
+        "layer_norm_a.weight": 1.0 + 0.1 * torch.randn(c_s, generator=gen),
+        "layer_norm_a.bias": 0.1 * torch.randn(c_s, generator=gen),
+        "mha.linear_q.weight": lin(hc, c_s),
+        "mha.linear_q.bias": 0.1 * torch.randn(hc, generator=gen),
+        "mha.linear_k.weight": lin(hc, c_s),
+        "mha.linear_v.weight": lin(hc, c_s),
+        "mha.linear_g.weight": lin(hc, c_s),
+        "mha.linear_o.weight": lin(c_s, hc),
+    }
+    p.update(make_pair_bias_params(gen, c_z, no_heads))
+    return p
 
 
 def make_pair_bias_params(gen, c_z: int, no_heads: int, offset: bool = True):

@@ -34,7 +34,8 @@ def test_header_declares_expected_entry_points():
                      "of3_version", "of3_last_hip_error", "of3_status_string", "of3_padded_n",
                      "of3_trimul_workspace_bytes", "of3_triattn_workspace_bytes",
                      "of3_trimul_workspace_bytes_for", "of3_triattn_workspace_bytes_for",
-                     "of3_transition_fwd", "of3_pair_bias_fwd", "of3_layer_norm_fwd", "of3_template_tail_fwd"):
+                     "of3_transition_fwd", "of3_pair_bias_fwd", "of3_layer_norm_fwd", "of3_template_tail_fwd",
+                     "of3_attn_pair_bias_fwd", "of3_attn_pair_bias_workspace_bytes"):
         assert required in names
 
 
@@ -168,3 +169,22 @@ def test_template_entry_points_validate(lib):
     assert lib.of3_template_tail_fwd(p, None, p, p, p, 1, 2, 16, 64, 128, 1, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
     assert lib.of3_template_tail_fwd(p, p, p, None, p, 1, 2, 16, 64, 128, 0, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
     assert lib.of3_template_tail_fwd(p, p, p, p, p, 1, 2, 16, 64, 128, 1, 7, None) == L.OF3_EINVAL
+
+
+def test_attn_pair_bias_entry_point_validates(lib):
+    from of3pair import _lib as L
+
+    assert lib.of3_attn_pair_bias_workspace_bytes(1, 768, 384, 16, 24) == 3 * 16 * 768 * 32 * 2 + 2 * 768 * 384 * 2
+    assert lib.of3_attn_pair_bias_workspace_bytes(1, 768, 384, 12, 32) > 0
+    for bad in ((1, 768, 256, 16, 16), (1, 768, 384, 16, 32), (1, 768, 384, 32, 12), (0, 768, 384, 16, 24),
+                (1, 1 << 17, 384, 16, 24)):
+        assert lib.of3_attn_pair_bias_workspace_bytes(*bad) == L.OF3_EINVAL
+    p = 256
+    args = [p] * 2 + [None] + [p] * 9 + [1, 64, 384, 16, 24, 1e9, 0, p, 1 << 30]
+    assert lib.of3_attn_pair_bias_fwd(*args, L.OF3_DTYPE_F32, None) == L.OF3_EINVAL      # bf16 only
+    small = list(args)
+    small[-1] = 1024
+    assert lib.of3_attn_pair_bias_fwd(*small, L.OF3_DTYPE_BF16, None) == L.OF3_ENOSPC
+    nul = list(args)
+    nul[5] = None                                                                         # b_q missing
+    assert lib.of3_attn_pair_bias_fwd(*nul, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL

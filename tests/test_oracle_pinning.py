@@ -316,3 +316,54 @@ def test_template_stack_is_blocks_then_layer_norm():
     a = orc.template_stack(t, shared, blocks, g, b, 4)
     bb = orc.template_stack(t, shared.expand(nt, n, n), blocks, g, b, 4)
     assert torch.equal(a, bb)
+
+
+def test_attention_pair_bias_matches_bruteforce_and_sdpa():
+    gen = torch.Generator().manual_seed(61)
+    n, cs, cz, c, h = 7, 24, 16, 6, 4
+    p = orc.make_attention_pair_bias_params(gen, cs, cz, c, h)
+    a = torch.randn(n, cs, generator=gen)
+    z = torch.randn(n, n, cz, generator=gen)
+    mask = torch.tensor([1, 1, 0, 1, 1, 1, 0.0])
+    got = orc.attention_pair_bias(a, z, mask, p, h)
+    assert got.shape == (n, cs)
+    assert np.abs(got.double().numpy() - bf.attention_pair_bias(a, z, mask, p, h)).max() < FP32_TOL
+    assert np.abs(orc.attention_pair_bias(a, z, None, p, h).double().numpy()
+                  - bf.attention_pair_bias(a, z, None, p, h)).max() < FP32_TOL
+    # the same through torch's scaled_dot_product_attention (its own 1/sqrt(c) scaling)
+    F = torch.nn.functional
+    an = F.layer_norm(a, (cs,), p["layer_norm_a.weight"], p["layer_norm_a.bias"], 1e-5)
+    heads = lambda t: t.view(n, h, c).transpose(0, 1)  # noqa: E731
+    q = heads(F.linear(an, p["mha.linear_q.weight"], p["mha.linear_q.bias"]))
+    k, v = heads(F.linear(an, p["mha.linear_k.weight"])), heads(F.linear(an, p["mha.linear_v.weight"]))
+    bias = orc.pair_bias(z, p) + (1e9 * (mask - 1))[None, None, :]
+    o = F.scaled_dot_product_attention(q, k, v, attn_mask=bias).transpose(0, 1).reshape(n, h * c)
+    want = F.linear(o * torch.sigmoid(F.linear(an, p["mha.linear_g.weight"])), p["mha.linear_o.weight"])
+    assert (got - want).abs().max() < FP32_TOL
+
+
+def test_attention_pair_bias_invariants():
+    gen = torch.Generator().manual_seed(62)
+    n, cs, cz, c, h = 9, 32, 16, 8, 4
+    p = orc.make_attention_pair_bias_params(gen, cs, cz, c, h)
+    a = torch.randn(2, n, cs, generator=gen)
+    z = torch.randn(2, n, n, cz, generator=gen)
+    mask = torch.ones(2, n)
+    mask[1, -3:] = 0
+    out = orc.attention_pair_bias(a, z, mask, p, h)
+    # a masked key does not influence any query: changing its features changes nothing but its own row
+    a2 = a.clone()
+    a2[1, -1] += 3.0
+    out2 = orc.attention_pair_bias(a2, z, mask, p, h)
+    assert (out2[1, :-1] - out[1, :-1]).abs().max() < 1e-5 and (out2[0] - out[0]).abs().max() == 0
+    # a bias constant along the keys cancels in the softmax: adding a per-query shift to z's projection
+    q = dict(p)
+    q["mha.linear_o.weight"] = torch.zeros_like(p["mha.linear_o.weight"])
+    assert orc.attention_pair_bias(a, z, mask, q, h).abs().max() == 0
+    # batch elements are independent
+    assert (orc.attention_pair_bias(a[:1], z[:1], mask[:1], p, h) - out[:1]).abs().max() < 1e-6
+    # a fully masked sequence degenerates to the uniform average of v (all logits shifted alike)
+    m0 = torch.zeros(1, n)
+    o0 = orc.attention_pair_bias(a[:1], torch.zeros(1, n, n, cz), m0, p, h)
+    o1 = orc.attention_pair_bias(a[:1], torch.zeros(1, n, n, cz), torch.ones(1, n), p, h)
+    assert torch.isfinite(o0).all() and o0.shape == o1.shape
