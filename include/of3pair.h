@@ -179,7 +179,7 @@ int of3_pair_bias_fwd(const void* z, const int64_t z_strides[3], const void* ln_
  * a, out: contiguous [B][N][C_s] (out may alias a); pair_bias: contiguous [B][H][N][N], what
  * of3_pair_bias_fwd returns for this module's layer_norm_z / linear_z; mask: fp32 [B][N] or null
  * (all ones); w_q, w_k, w_v, w_g: [H*D][C_s]; b_q: [H*D]; w_o: [C_s][H*D].  bf16 only, the AF3
- * trunk shape: C_s = H*D = 384, D a multiple of 8 up to 32 (16 heads of 24).  The workspace holds
+ * trunk shape: C_s = H*D = 384, D in {8, 16, 24} (16 heads of 24).  The workspace holds
  * q, k, v, the gate and the gated attention output. */
 int64_t of3_attn_pair_bias_workspace_bytes(int64_t B, int64_t N, int64_t C_s, int64_t H, int64_t D);
 int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* mask, const void* ln_w,

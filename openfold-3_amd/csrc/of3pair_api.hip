@@ -557,7 +557,7 @@ int of3_template_tail_fwd(const void* t, const void* ln_w, const void* ln_b, con
 }
 
 int64_t of3_attn_pair_bias_workspace_bytes(int64_t B, int64_t N, int64_t C_s, int64_t H, int64_t D) {
-  if (B < 1 || N < 1 || N > (1 << 16) || C_s != 384 || H < 1 || D < 8 || D > 32 || (D % 8) != 0 || H * D != C_s)
+  if (B < 1 || N < 1 || N > (1 << 16) || C_s != 384 || H < 1 || D < 8 || D > 24 || (D % 8) != 0 || H * D != C_s)
     return OF3_EINVAL;
   const int64_t Np = (N + 31) / 32 * 32;
   return 3 * align256(B * H * Np * 32 * 2) + 2 * align256(B * N * H * D * 2);

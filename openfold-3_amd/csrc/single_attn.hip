@@ -16,8 +16,12 @@
 //     channels of one position); for v the positions are the A operand, so that a lane holds one
 //     channel of 4-position runs and V^T [B][H][32][Np] is written with 8-byte stores.
 //     q carries log2(e) / sqrt(D) (the softmax below uses exp2), g is stored after the sigmoid.
+//     The first padding channel (index D) carries the key mask: q gets 1 there and k gets
+//     inf * (mask[key] - 1) * log2(e), or -inf for the rows between N and Np, so the q.k
+//     product itself adds the mask bias and gives padded keys a weight of exactly zero.
 //  2. single_attn: one wave per (batch, head, 32 queries), flash style over 32-key tiles:
-//     S^T = K Q^T with the accumulator initialised to (pair bias + mask bias) * log2(e), running
+//     S^T = K Q^T with the accumulator initialised to pair bias * log2(e), the next tile's
+//     operands requested before the current tile's arithmetic, running
 //     maximum and sum in fp32, O^T = V^T P^T with P^T taken from the S^T registers; the result
 //     is divided by the sum, multiplied by the gate and written as [B][N][H*D].
 //  3. single_out: the same tiling as 1 without the LayerNorm: out = [a +] og Wo^T.
@@ -95,13 +99,19 @@ __device__ __forceinline__ void fill_tile(u32x4_t* act, const bf16_t* __restrict
 // (w-row l32, half lh) holds positions 8*(v/4) + 4*lh + (v%4).
 template <bool WEIGHTS_ARE_A>
 __device__ __forceinline__ f32x16_t tile_product(const u32x4_t* act, const bf16_t* __restrict__ w_row, int l32, int lh) {
-  f32x16_t acc = zero16();
-#pragma unroll 6
+  // the lane's whole weight row half (24 chunks) is requested before the first MFMA: one trip to
+  // L2 per tile instead of one per k-step
+  u32x4_t w[kK / 16];
+#pragma unroll
   for (int s = 0; s < kK / 16; ++s) {
-    u32x4_t w = {0u, 0u, 0u, 0u};
-    if (w_row) w = *reinterpret_cast<const u32x4_t*>(w_row + 16 * s + 8 * lh);
+    w[s] = u32x4_t{0u, 0u, 0u, 0u};
+    if (w_row) w[s] = *reinterpret_cast<const u32x4_t*>(w_row + 16 * s + 8 * lh);
+  }
+  f32x16_t acc = zero16();
+#pragma unroll
+  for (int s = 0; s < kK / 16; ++s) {
     const u32x4_t x = act[act_slot(l32, 2 * s + lh)];
-    acc = WEIGHTS_ARE_A ? mfma_32x32x16(w, x, acc) : mfma_32x32x16(x, w, acc);
+    acc = WEIGHTS_ARE_A ? mfma_32x32x16(w[s], x, acc) : mfma_32x32x16(x, w[s], acc);
   }
   return acc;
 }
@@ -134,8 +144,16 @@ __global__ __launch_bounds__(256) void single_proj_kernel(SingleAttnArgs p) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int d = 16 * lh + v;
-          f[v] = d < D ? (f[v] + bf16_to_f32(p.bq[h * D + d])) * q_scale : 0.f;
+          f[v] = d < D ? (f[v] + bf16_to_f32(p.bq[h * D + d])) * q_scale : (d == D ? 1.f : 0.f);
         }
+      } else if (kind == 1) {
+        // the key's mask bias rides in the first padding channel (q holds 1 there)
+        float mb = 0.f;
+        if (pos >= N) mb = -__builtin_inff();
+        else if (p.mask) mb = p.inf * kLog2e * (p.mask[(size_t)b * N + pos] - 1.f);
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (16 * lh + v == D) f[v] = mb;
       } else if (kind == 3) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) f[v] = sigmoidf_fast(f[v]);
@@ -153,10 +171,6 @@ __global__ __launch_bounds__(256) void single_proj_kernel(SingleAttnArgs p) {
           if (16 * lh + 8 < D) *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
         }
       } else if (pos < Np) {
-        if (pos >= N) {  // padded key rows are read by the attention kernel: zeros
-          o0 = u32x4_t{0u, 0u, 0u, 0u};
-          o1 = o0;
-        }
         bf16_t* dst = (kind == 0 ? p.q : p.k) + (((size_t)b * H + h) * Np + pos) * kDP + 16 * lh;
         *reinterpret_cast<u32x4_t*>(dst) = o0;
         *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
@@ -181,19 +195,19 @@ __global__ __launch_bounds__(256) void single_proj_kernel(SingleAttnArgs p) {
 }
 
 // ---- 2. attention core -------------------------------------------------------------------
-// 16 consecutive bf16 / fp32 values starting at element `first` of a row of `n` valid elements,
-// as floats; elements at or past n give `fill`
-__device__ __forceinline__ void load16_bf16(const bf16_t* __restrict__ row, int first, int n, bool vec_ok, float fill,
-                                            float (&out)[16]) {
+// 16 consecutive bf16 values starting at element `first` of a row of `n` valid elements, packed
+// as they are; elements at or past n read as zero
+__device__ __forceinline__ void load16_raw(const bf16_t* __restrict__ row, int first, int n, bool vec_ok, u32x4_t (&out)[2]) {
   if (vec_ok && first + 16 <= n) {
-    float lo[8], hi[8];
-    unpack8(*reinterpret_cast<const u32x4_t*>(row + first), lo);
-    unpack8(*reinterpret_cast<const u32x4_t*>(row + first + 8), hi);
-#pragma unroll
-    for (int v = 0; v < 8; ++v) out[v] = lo[v], out[8 + v] = hi[v];
+    out[0] = *reinterpret_cast<const u32x4_t*>(row + first);
+    out[1] = *reinterpret_cast<const u32x4_t*>(row + first + 8);
   } else {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) out[v] = first + v < n ? bf16_to_f32(row[first + v]) : fill;
+    for (int w = 0; w < 8; ++w) {
+      const uint32_t lo = first + 2 * w < n ? row[first + 2 * w] : 0u;
+      const uint32_t hi = first + 2 * w + 1 < n ? row[first + 2 * w + 1] : 0u;
+      out[w >> 2][w & 3] = lo | (hi << 16);
+    }
   }
 }
 
@@ -215,42 +229,45 @@ __global__ __launch_bounds__(256) void single_attn_kernel(SingleAttnArgs p, int 
   const bf16_t* K = p.k + bh * Np * kDP;
   const bf16_t* Vt = p.vt + bh * kDP * Np;
   const bf16_t* pb_row = p.pair_bias + (bh * N + qrow) * N;
-  const float* mask = p.mask ? p.mask + (size_t)b * N : nullptr;
   const bool vec_ok = (N % 8) == 0;  // 16-byte aligned runs of the bias rows
-  const float mscale = p.inf * kLog2e;
 
   u32x4_t qop[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s) qop[s] = *reinterpret_cast<const u32x4_t*>(Q + 16 * s + 8 * lh);
   const int krow = rowperm16(l32);
 
+  // operands of one key tile: K rows dealt by rowperm16 (a lane ends up with keys k0 + 16*lh + v);
+  // V^T rows = padded channels dealt by rowperm16, lane-half lh and k-step s2 feed keys
+  // 16*lh + 8*s2 .. +7, the keys registers 8*s2 .. 8*s2+7 of that lane-half hold in S^T; the
+  // lane's 16 pair-bias values
+  auto load_tile = [&](int kt, u32x4_t (&kc)[2], u32x4_t (&vc)[2], u32x4_t (&braw)[2]) {
+    const int k0 = 32 * kt;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) kc[s] = *reinterpret_cast<const u32x4_t*>(K + (size_t)(k0 + krow) * kDP + 16 * s + 8 * lh);
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) vc[s2] = *reinterpret_cast<const u32x4_t*>(Vt + (size_t)krow * Np + k0 + 16 * lh + 8 * s2);
+    load16_raw(pb_row, k0 + 16 * lh, N, vec_ok, braw);
+  };
+
   float m_run = -__builtin_inff(), l_run = 0.f;
   f32x16_t oacc = zero16();
   const int nkt = (N + 31) / 32;
+  u32x4_t kn[2], vn[2], bn[2];
+  load_tile(0, kn, vn, bn);
   for (int kt = 0; kt < nkt; ++kt) {
-    const int k0 = 32 * kt;
-    u32x4_t kc[2], vc[2];
+    u32x4_t kc[2], vc[2], braw[2];
 #pragma unroll
-    for (int s = 0; s < 2; ++s) kc[s] = *reinterpret_cast<const u32x4_t*>(K + (size_t)(k0 + krow) * kDP + 16 * s + 8 * lh);
-    // V^T rows = padded channels dealt by rowperm16; lane-half lh, k-step s2 feeds keys 16*lh + 8*s2 .. +7,
-    // the keys that registers 8*s2 .. 8*s2+7 of the same lane-half hold in S^T
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) vc[s2] = *reinterpret_cast<const u32x4_t*>(Vt + (size_t)krow * Np + k0 + 16 * lh + 8 * s2);
+    for (int s = 0; s < 2; ++s) kc[s] = kn[s], vc[s] = vn[s], braw[s] = bn[s];
+    if (kt + 1 < nkt) load_tile(kt + 1, kn, vn, bn);  // in flight under this tile's arithmetic
 
-    // this lane's 16 keys of the tile: k0 + 16*lh + v
-    float bias[16];
-    load16_bf16(pb_row, k0 + 16 * lh, N, vec_ok, 0.f, bias);
     f32x16_t s;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int key = k0 + 16 * lh + v;
-      float mb = 0.f;
-      if (key >= N) mb = -__builtin_inff();  // padded keys: weight exactly zero
-      else if (mask) mb = mscale * (mask[key] - 1.f);
-      s[v] = bias[v] * kLog2e + mb;
+    for (int w = 0; w < 8; ++w) {
+      s[2 * w] = bf16_lo(braw[w >> 2][w & 3]) * kLog2e;
+      s[2 * w + 1] = bf16_hi(braw[w >> 2][w & 3]) * kLog2e;
     }
     s = mfma_32x32x16(kc[0], qop[0], s);
-    s = mfma_32x32x16(kc[1], qop[1], s);
+    s = mfma_32x32x16(kc[1], qop[1], s);  // includes the mask bias (-inf for keys past N)
 
     float mx = s[0];
 #pragma unroll
@@ -278,13 +295,13 @@ __global__ __launch_bounds__(256) void single_attn_kernel(SingleAttnArgs p, int 
   const float inv = fast_rcp(l_run + xhalf(l_run));
   if (q_valid && 16 * lh < D) {
     const size_t off = ((size_t)b * N + qrow) * (H * D) + h * D + 16 * lh;
-    float gate[16];
-    load16_bf16(p.g + off, 0, D - 16 * lh, true, 0.f, gate);
+    u32x4_t graw[2];
+    load16_raw(p.g + off, 0, D - 16 * lh, true, graw);
     u32x4_t o0, o1;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      o0[w] = pack_bf16(oacc[2 * w] * inv * gate[2 * w], oacc[2 * w + 1] * inv * gate[2 * w + 1]);
-      o1[w] = pack_bf16(oacc[8 + 2 * w] * inv * gate[8 + 2 * w], oacc[8 + 2 * w + 1] * inv * gate[8 + 2 * w + 1]);
+      o0[w] = pack_bf16(oacc[2 * w] * inv * bf16_lo(graw[0][w]), oacc[2 * w + 1] * inv * bf16_hi(graw[0][w]));
+      o1[w] = pack_bf16(oacc[8 + 2 * w] * inv * bf16_lo(graw[1][w]), oacc[8 + 2 * w + 1] * inv * bf16_hi(graw[1][w]));
     }
     bf16_t* dst = p.og + off;
     *reinterpret_cast<u32x4_t*>(dst) = o0;
@@ -313,10 +330,13 @@ __global__ __launch_bounds__(256) void single_out_kernel(SingleAttnArgs p) {
       for (int v = 0; v < 16; ++v) f[v] = acc[v];
       if (p.add_residual) {
         // the reference adds the module's bf16 output to s: round before the add
-        float r[16];
-        load16_bf16(p.a + off, 0, 16, true, 0.f, r);
+        u32x4_t r[2];
+        load16_raw(p.a + off, 0, 16, true, r);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) f[v] = bf16_to_f32(to_bf16(f[v])) + r[v];
+        for (int w = 0; w < 8; ++w) {
+          f[2 * w] = bf16_to_f32(to_bf16(f[2 * w])) + bf16_lo(r[w >> 2][w & 3]);
+          f[2 * w + 1] = bf16_to_f32(to_bf16(f[2 * w + 1])) + bf16_hi(r[w >> 2][w & 3]);
+        }
       }
       u32x4_t o0, o1;
 #pragma unroll
@@ -333,11 +353,11 @@ __global__ __launch_bounds__(256) void single_out_kernel(SingleAttnArgs p) {
 }  // namespace
 
 hipError_t single_attn_launch(const SingleAttnArgs& a, hipStream_t stream) {
-  if (a.H * a.D != kK || a.D > kDP || (a.D % 8) != 0 || a.H < 1 || a.N < 1 || a.B < 1 || a.B > 65535 || a.H > 65535)
+  if (a.H * a.D != kK || a.D >= kDP || (a.D % 8) != 0 || a.H < 1 || a.N < 1 || a.B < 1 || a.B > 65535 || a.H > 65535)
     return hipErrorInvalidValue;
   if (a.Np != (a.N + 31) / 32 * 32) return hipErrorInvalidValue;
   const int row_blocks = a.Np / 32;
-  hipLaunchKernelGGL(single_proj_kernel, dim3(row_blocks, 4, a.B), dim3(256), 0, stream, a);
+  hipLaunchKernelGGL(single_proj_kernel, dim3(row_blocks, a.H, a.B), dim3(256), 0, stream, a);  // one tile per wave
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(single_attn_kernel, dim3((row_blocks + 3) / 4, a.H, a.B), dim3(256), 0, stream, a, row_blocks);

@@ -299,7 +299,7 @@ def attention_pair_bias(a, z, mask, norm_a_weight, norm_a_bias, norm_z_weight, n
     need = lib.of3_attn_pair_bias_workspace_bytes(B, N, CS, H, D)
     if need < 0:
         raise ValueError("attention_pair_bias: supported shape is C_s = no_heads * c = 384 with c a multiple of 8 "
-                         "up to 32; got C_s=%d heads=%d c=%d" % (CS, H, D))
+                         "up to 24; got C_s=%d heads=%d c=%d" % (CS, H, D))
     ws = _workspace(a.device, need)
     w = [_w(t, a.dtype) for t in (norm_a_weight, norm_a_bias, q_weight, q_bias, k_weight, v_weight, g_weight, o_weight)]
     with torch.cuda.device(a.device):

@@ -175,8 +175,8 @@ def test_attn_pair_bias_entry_point_validates(lib):
     from of3pair import _lib as L
 
     assert lib.of3_attn_pair_bias_workspace_bytes(1, 768, 384, 16, 24) == 3 * 16 * 768 * 32 * 2 + 2 * 768 * 384 * 2
-    assert lib.of3_attn_pair_bias_workspace_bytes(1, 768, 384, 12, 32) > 0
-    for bad in ((1, 768, 256, 16, 16), (1, 768, 384, 16, 32), (1, 768, 384, 32, 12), (0, 768, 384, 16, 24),
+    assert lib.of3_attn_pair_bias_workspace_bytes(1, 768, 384, 24, 16) > 0
+    for bad in ((1, 768, 256, 16, 16), (1, 768, 384, 16, 32), (1, 768, 384, 12, 32), (1, 768, 384, 32, 12), (0, 768, 384, 16, 24),
                 (1, 1 << 17, 384, 16, 24)):
         assert lib.of3_attn_pair_bias_workspace_bytes(*bad) == L.OF3_EINVAL
     p = 256
