@@ -26,7 +26,8 @@
  *   openfold3/core/model/layers/transition.py
  *       :225-271  SwiGLUTransition.forward (LayerNorm, SwiGLU of
  *                 openfold3/core/model/primitives/activations.py:33-61,
- *                 linear_out, mask)                             -> of3_transition_fwd
+ *                 linear_out, mask)                             -> of3_transition_fwd (pair tensors),
+ *                                                                  of3_transition_rows_fwd (single representation)
  *   openfold3/core/model/layers/attention_pair_bias.py
  *       :151-161  _prep_bias: layer_norm_z, linear_z, permute   -> of3_pair_bias_fwd
  *       :189-244  AttentionPairBias.forward of the trunk (no AdaLN): layer_norm_a, mask bias,
@@ -187,6 +188,17 @@ int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* ma
                            const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C_s, int64_t H,
                            int64_t D, float inf, int add_residual, void* workspace, int64_t workspace_bytes,
                            int dtype, void* stream);
+
+/* ---- transition of the single representation ------------------------------------------- */
+
+/* The same update as of3_transition_fwd for the single representation (PairFormerBlock's
+ * single_transition, pairformer.py:118-122, :203-212): x, out contiguous [rows][C] (any leading
+ * dimensions flattened; out may alias x), mask fp32 [rows] or null.  bf16 only, C = 384, HID a
+ * multiple of 384.  The workspace holds the hidden activations [rows][HID]. */
+int64_t of3_transition_rows_workspace_bytes(int64_t rows, int64_t C, int64_t HID);
+int of3_transition_rows_fwd(const void* x, const float* mask, const void* ln_w, const void* ln_b, const void* w_a,
+                            const void* w_b, const void* w_out, void* out, int64_t rows, int64_t C, int64_t HID,
+                            int add_residual, void* workspace, int64_t workspace_bytes, int dtype, void* stream);
 
 /* ---- template branch: closing LayerNorm and embedder tail ------------------------------ */
 

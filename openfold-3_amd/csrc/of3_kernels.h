@@ -148,6 +148,20 @@ struct SingleAttnArgs {
 };
 hipError_t single_attn_launch(const SingleAttnArgs& args, hipStream_t stream);
 
+// ---- transition of the single representation (single_transition.hip), bf16, C = 384
+struct RowTransitionArgs {
+  const bf16_t* x;            // [rows][384]
+  const float* mask;          // [rows] or null
+  const bf16_t *ln_w, *ln_b;
+  const bf16_t *wa, *wb;      // [HID][384]
+  const bf16_t* wout;         // [384][HID]
+  bf16_t* h;                  // workspace, [rows][HID]
+  bf16_t* out;                // [rows][384]; may alias x
+  long rows;
+  int HID, add_residual;      // HID a multiple of 384
+};
+hipError_t row_transition_launch(const RowTransitionArgs& args, hipStream_t stream);
+
 // ---- fp32 path (pair_f32.hip): whole updates, any N, C and C_hidden <= 256, head width 16/32/64
 struct TrimulF32Args {
   const float* z;

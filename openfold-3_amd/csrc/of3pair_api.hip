@@ -608,4 +608,37 @@ int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* ma
   return e == hipSuccess ? OF3_OK : fail_hip(e);
 }
 
+int64_t of3_transition_rows_workspace_bytes(int64_t rows, int64_t C, int64_t HID) {
+  if (rows < 1 || rows > (1ll << 31) || C != 384 || HID < C || (HID % C) != 0 || HID > (1 << 20)) return OF3_EINVAL;
+  return align256(rows * HID * 2);
+}
+
+int of3_transition_rows_fwd(const void* x, const float* mask, const void* ln_w, const void* ln_b, const void* w_a,
+                            const void* w_b, const void* w_out, void* out, int64_t rows, int64_t C, int64_t HID,
+                            int add_residual, void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
+  if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
+  const int64_t need = of3_transition_rows_workspace_bytes(rows, C, HID);
+  if (need < 0) return OF3_EINVAL;
+  const void* ptrs[] = {x, ln_w, ln_b, w_a, w_b, w_out, out, workspace};
+  for (const void* p : ptrs)
+    if (!p || !aligned16(p)) return OF3_EINVAL;
+  if (mask && !aligned4(mask)) return OF3_EINVAL;
+  if (workspace_bytes < need) return OF3_ENOSPC;
+  of3::RowTransitionArgs a;
+  a.x = bf(x);
+  a.mask = mask;
+  a.ln_w = bf(ln_w);
+  a.ln_b = bf(ln_b);
+  a.wa = bf(w_a);
+  a.wb = bf(w_b);
+  a.wout = bf(w_out);
+  a.h = static_cast<of3::bf16_t*>(workspace);
+  a.out = bf(out);
+  a.rows = (long)rows;
+  a.HID = (int)HID;
+  a.add_residual = add_residual ? 1 : 0;
+  hipError_t e = of3::row_transition_launch(a, static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? OF3_OK : fail_hip(e);
+}
+
 }  // extern "C"

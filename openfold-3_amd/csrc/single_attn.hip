@@ -27,94 +27,15 @@
 //  3. single_out: the same tiling as 1 without the LayerNorm: out = [a +] og Wo^T.
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_rowtile.h"
 
 namespace of3 {
 
 namespace {
 
-constexpr int kK = 384;          // c_s = H * D: reduction length of both linear stages
-constexpr int kChunks = kK / 8;  // 16-byte chunks per position
+using namespace rowtile;
+
 constexpr int kDP = 32;          // head width padded to one MFMA tile
-
-__device__ __forceinline__ float xhalf(float v) { return __shfl_xor(v, 32, 64); }
-
-// LDS tile [32 positions][kChunks]: chunk index XOR position in its low four bits (the 16 lanes
-// of a read phase hold 16 consecutive positions at one chunk index and must hit 16 bank windows;
-// a row is 768 bytes = 3 windows of 256, so without the key they would all hit the same one)
-__device__ __forceinline__ int act_slot(int pos, int chunk) { return pos * kChunks + ((chunk & ~15) | ((chunk ^ pos) & 15)); }
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-
-// rows pos0 .. pos0+31 of src [rows][kK] into the LDS tile; with LN, normalised (statistics in
-// fp32, result rounded to bf16 as the reference's LayerNorm output).  Wave w handles 8 rows, lanes
-// 0..47 one chunk each.  Rows past n_rows repeat the last one (never stored by the callers).
-template <bool LN>
-__device__ __forceinline__ void fill_tile(u32x4_t* act, const bf16_t* __restrict__ src, long pos0, long n_rows,
-                                          const bf16_t* __restrict__ ln_w, const bf16_t* __restrict__ ln_b, int wave,
-                                          int lane) {
-  const bool has = lane < kChunks;
-  float lw[8], lb[8];
-  if (LN && has) {
-    load_affine8(ln_w, lane, lw);
-    load_affine8(ln_b, lane, lb);
-  }
-#pragma unroll
-  for (int r = 0; r < 8; ++r) {
-    const int pos = 8 * wave + r;
-    long row = pos0 + pos;
-    row = row < n_rows ? row : n_rows - 1;
-    u32x4_t raw = {0u, 0u, 0u, 0u};
-    if (has) raw = *reinterpret_cast<const u32x4_t*>(src + row * kK + 8 * lane);
-    if (LN) {
-      float x[8];
-      unpack8(raw, x);
-      float s = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) s += x[i];
-      const float mean = wave_sum(s) * (1.f / kK);
-      float q = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        x[i] = has ? x[i] - mean : 0.f;
-        q += x[i] * x[i];
-      }
-      const float rstd = __builtin_amdgcn_rsqf(wave_sum(q) * (1.f / kK) + kLnEps);
-      if (has) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = x[i] * rstd * lw[i] + lb[i];
-        raw = pack8(x);
-      }
-    }
-    if (has) act[act_slot(pos, lane)] = raw;
-  }
-}
-
-// 32 x 32 output tile with K = kK: `w_row` points at the weight row this lane feeds (or is null
-// for a zero row), positions come from the LDS tile.  WEIGHTS_ARE_A: result lane (position l32,
-// half lh) holds w-rows 16*lh + v (the caller dealt the rows by rowperm16); otherwise lane
-// (w-row l32, half lh) holds positions 8*(v/4) + 4*lh + (v%4).
-template <bool WEIGHTS_ARE_A>
-__device__ __forceinline__ f32x16_t tile_product(const u32x4_t* act, const bf16_t* __restrict__ w_row, int l32, int lh) {
-  // the lane's whole weight row half (24 chunks) is requested before the first MFMA: one trip to
-  // L2 per tile instead of one per k-step
-  u32x4_t w[kK / 16];
-#pragma unroll
-  for (int s = 0; s < kK / 16; ++s) {
-    w[s] = u32x4_t{0u, 0u, 0u, 0u};
-    if (w_row) w[s] = *reinterpret_cast<const u32x4_t*>(w_row + 16 * s + 8 * lh);
-  }
-  f32x16_t acc = zero16();
-#pragma unroll
-  for (int s = 0; s < kK / 16; ++s) {
-    const u32x4_t x = act[act_slot(l32, 2 * s + lh)];
-    acc = WEIGHTS_ARE_A ? mfma_32x32x16(w[s], x, acc) : mfma_32x32x16(x, w[s], acc);
-  }
-  return acc;
-}
 
 // ---- 1. LayerNorm + q, k, v, g ------------------------------------------------------------
 __global__ __launch_bounds__(256) void single_proj_kernel(SingleAttnArgs p) {
@@ -125,7 +46,7 @@ __global__ __launch_bounds__(256) void single_proj_kernel(SingleAttnArgs p) {
   const int N = p.N, Np = p.Np, H = p.H, D = p.D;
   const int b = blockIdx.z;
   const long pos0 = (long)blockIdx.x * 32;
-  fill_tile<true>(act, p.a + (size_t)b * N * kK, pos0, N, p.ln_w, p.ln_b, wave, lane);
+  fill_tile<true>(act, p.a + (size_t)b * N * kK, kK, pos0, N, p.ln_w, p.ln_b, wave, lane);
   __syncthreads();
 
   const long pos = pos0 + l32;  // position of this lane in the weights-are-A tiles
@@ -195,22 +116,6 @@ __global__ __launch_bounds__(256) void single_proj_kernel(SingleAttnArgs p) {
 }
 
 // ---- 2. attention core -------------------------------------------------------------------
-// 16 consecutive bf16 values starting at element `first` of a row of `n` valid elements, packed
-// as they are; elements at or past n read as zero
-__device__ __forceinline__ void load16_raw(const bf16_t* __restrict__ row, int first, int n, bool vec_ok, u32x4_t (&out)[2]) {
-  if (vec_ok && first + 16 <= n) {
-    out[0] = *reinterpret_cast<const u32x4_t*>(row + first);
-    out[1] = *reinterpret_cast<const u32x4_t*>(row + first + 8);
-  } else {
-#pragma unroll
-    for (int w = 0; w < 8; ++w) {
-      const uint32_t lo = first + 2 * w < n ? row[first + 2 * w] : 0u;
-      const uint32_t hi = first + 2 * w + 1 < n ? row[first + 2 * w + 1] : 0u;
-      out[w >> 2][w & 3] = lo | (hi << 16);
-    }
-  }
-}
-
 __global__ __launch_bounds__(256) void single_attn_kernel(SingleAttnArgs p, int q_tiles) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -318,7 +223,7 @@ __global__ __launch_bounds__(256) void single_out_kernel(SingleAttnArgs p) {
   const int N = p.N;
   const int b = blockIdx.z;
   const long pos0 = (long)blockIdx.x * 32;
-  fill_tile<false>(act, p.og + (size_t)b * N * kK, pos0, N, nullptr, nullptr, wave, lane);
+  fill_tile<false>(act, p.og + (size_t)b * N * kK, kK, pos0, N, nullptr, nullptr, wave, lane);
   __syncthreads();
   const long pos = pos0 + l32;
   for (int tile = blockIdx.y * 4 + wave; tile < kK / 32; tile += gridDim.y * 4) {

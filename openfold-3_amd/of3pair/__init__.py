@@ -4,11 +4,12 @@ from .layers import (AttentionPairBias, PairBiasProjection, SwiGLUTransition, Tr
                      TriangleMultiplicationIncoming, TriangleMultiplicationOutgoing,
                      TriangleMultiplicativeUpdate)
 from .pair_stack import PairBlock, PairStack
+from .pairformer import PairFormerBlock, PairFormerStack
 from .template import TemplateEmbedderCore, TemplatePairBlock, TemplatePairStack
 from . import checkpoint
 
 __all__ = [
     "TriangleMultiplicativeUpdate", "TriangleMultiplicationOutgoing", "TriangleMultiplicationIncoming",
     "TriangleAttention", "TriangleAttentionStartingNode", "TriangleAttentionEndingNode", "SwiGLUTransition", "PairBiasProjection", "AttentionPairBias",
-    "PairStack", "PairBlock", "TemplatePairBlock", "TemplatePairStack", "TemplateEmbedderCore", "checkpoint",
+    "PairStack", "PairBlock", "PairFormerBlock", "PairFormerStack", "TemplatePairBlock", "TemplatePairStack", "TemplateEmbedderCore", "checkpoint",
 ]

@@ -43,6 +43,8 @@ SIGNATURES = {
     "of3_attn_pair_bias_workspace_bytes": (c_int64, [c_int64] * 5),
     "of3_attn_pair_bias_fwd": (c_int, [c_void_p] * 12 + [c_int64] * 5 + [ctypes.c_float, c_int, c_void_p, c_int64, c_int,
                                                                     c_void_p]),
+    "of3_transition_rows_workspace_bytes": (c_int64, [c_int64] * 3),
+    "of3_transition_rows_fwd": (c_int, [c_void_p] * 8 + [c_int64] * 3 + [c_int, c_void_p, c_int64, c_int, c_void_p]),
     "of3_layer_norm_fwd": (c_int, [c_void_p] * 4 + [c_int64] * 2 + [c_int, c_void_p]),
     "of3_template_tail_fwd": (c_int, [c_void_p] * 5 + [c_int64] * 5 + [c_int, c_int, c_void_p]),
 }

@@ -30,6 +30,7 @@ SOURCES = [
     "pair_bias.hip",
     "template_tail.hip",
     "single_attn.hip",
+    "single_transition.hip",
     "pair_f32.hip",
 ]
 

@@ -166,9 +166,13 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
                       inplace: bool = False):
     """Update of transition.py:256-268 (LayerNorm, SwiGLU, linear_out, mask), or x + update when
     add_residual.  x [*, N, N, C], mask [*, N, N] or None; a_weight / b_weight [n*C, C] are
-    SwiGLU's linear_a (through SiLU) and linear_b, out_weight [C, n*C]."""
+    SwiGLU's linear_a (through SiLU) and linear_b, out_weight [C, n*C].  With C = 384 (the single
+    representation) x is [*, 384] and mask [*]: any leading dimensions."""
     code = _require_gpu(x, "x")
     lib = _lib.load()
+    if x.shape[-1] == 384:  # the single representation: position-wise over [*, 384] rows
+        return _swiglu_transition_rows(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_weight,
+                                       add_residual, inplace, code)
     x4, lead = _flatten_pair(x)
     B, N, _, C = x4.shape
     HID = a_weight.shape[0]
@@ -187,6 +191,39 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
                          % (C, HID, x.dtype))
     _lib.check(st, "of3_transition_fwd")
     return _finish(x, x4, out4, lead, inplace)
+
+
+def _swiglu_transition_rows(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_weight, add_residual, inplace,
+                            code):
+    """The transition over the single representation s [*, 384] (pairformer.py:203-212): every
+    leading dimension is a row; mask [*] or None."""
+    lib = _lib.load()
+    if x.dtype != torch.bfloat16:
+        raise ValueError("single transition: the kernels are bf16 only, got %s" % x.dtype)
+    C = x.shape[-1]
+    HID = a_weight.shape[0]
+    if tuple(a_weight.shape) != (HID, C) or tuple(b_weight.shape) != (HID, C) or tuple(out_weight.shape) != (C, HID):
+        raise ValueError("transition weights must be [n*C, C], [n*C, C] and [C, n*C]")
+    xc = x if x.is_contiguous() else x.contiguous()
+    rows = xc.numel() // C
+    out = xc if (inplace and xc is x) else torch.empty_like(xc)
+    m = None
+    if mask is not None:
+        if tuple(mask.shape) != tuple(x.shape[:-1]):
+            mask = mask.expand(*x.shape[:-1])
+        m = mask.to(torch.float32).contiguous()
+    need = lib.of3_transition_rows_workspace_bytes(rows, C, HID)
+    if need < 0:
+        raise ValueError("single transition: c_in = 384 with a hidden width that is a multiple of 384; got hidden=%d"
+                         % HID)
+    ws = _workspace(x.device, need)
+    keep = [_w(t, x.dtype) for t in (norm_weight, norm_bias, a_weight, b_weight, out_weight)]
+    with torch.cuda.device(x.device):
+        st = lib.of3_transition_rows_fwd(xc.data_ptr(), None if m is None else m.data_ptr(),
+                                         *[k.data_ptr() for k in keep], out.data_ptr(), rows, C, HID,
+                                         int(bool(add_residual)), ws.data_ptr(), ws.numel(), code, _stream(x))
+    _lib.check(st, "of3_transition_rows_fwd")
+    return out
 
 
 def pair_bias(z, norm_weight, norm_bias, weight):

@@ -212,7 +212,8 @@ class _SwiGLUParams(nn.Module):
 class SwiGLUTransition(nn.Module):
     """AF3 Algorithm 11 as the pair stack uses it (transition.py:225-271): LayerNorm, SwiGLU,
     linear_out, mask.  State-dict keys: layer_norm.{weight,bias}, swiglu.linear_{a,b}.weight,
-    linear_out.weight.  Pair tensors only: x [*, N, N, C_in], mask [*, N, N]."""
+    linear_out.weight.  Pair tensors x [*, N, N, C_in] with mask [*, N, N] (C_in 64 or 128), or the
+    single representation x [*, N, 384] with mask [*, N]."""
 
     def __init__(self, c_in, n, linear_init_params=None):
         super().__init__()

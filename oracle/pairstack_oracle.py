@@ -233,6 +233,29 @@ def attention_pair_bias(a, z, mask, p, no_heads: int, inf: float = INF):
     return linear(o, p["mha.linear_o.weight"])
 
 
+def pairformer_block(s, z, single_mask, pair_mask, p, no_heads_pair: int, no_heads_pair_bias: int,
+                     row_chunk: int | None = None, mask_trans: bool = True):
+    """PairFormerBlock.forward (pairformer.py:124-215): z = pair_stack(z); s = s +
+    attn_pair_bias(s, z, mask = single_mask); s = s + single_transition(s, mask = single_mask if
+    _mask_trans).  ``p`` holds the three sub-modules under pair_stack. / attn_pair_bias. /
+    single_transition.  Returns (s, z)."""
+    z = pair_block(z, pair_mask, _sub(p, "pair_stack."), no_heads_pair, row_chunk=row_chunk, mask_trans=mask_trans)
+    s = s + attention_pair_bias(s, z, single_mask, _sub(p, "attn_pair_bias."), no_heads_pair_bias)
+    s = s + transition_update(s, single_mask if mask_trans else None, _sub(p, "single_transition."))
+    return s, z
+
+
+def make_pairformer_block_params(seed: int, c_s: int, c_z: int, c_hidden_mul: int, c_head_pair: int,
+                                 no_heads_pair: int, c_head_bias: int, no_heads_bias: int, n: int):
+    gen = torch.Generator().manual_seed(seed + 1000)
+    p = {"pair_stack." + k: v for k, v in make_block_params(seed, c_z, c_hidden_mul, c_head_pair, no_heads_pair).items()}
+    p.update({"pair_stack.pair_transition." + k: v for k, v in make_transition_params(gen, c_z, n).items()})
+    p.update({"attn_pair_bias." + k: v
+              for k, v in make_attention_pair_bias_params(gen, c_s, c_z, c_head_bias, no_heads_bias).items()})
+    p.update({"single_transition." + k: v for k, v in make_transition_params(gen, c_s, n).items()})
+    return p
+
+
 def make_attention_pair_bias_params(gen, c_s: int, c_z: int, c_head: int, no_heads: int):
     hc = c_head * no_heads
 

@@ -35,7 +35,8 @@ def test_header_declares_expected_entry_points():
                      "of3_trimul_workspace_bytes", "of3_triattn_workspace_bytes",
                      "of3_trimul_workspace_bytes_for", "of3_triattn_workspace_bytes_for",
                      "of3_transition_fwd", "of3_pair_bias_fwd", "of3_layer_norm_fwd", "of3_template_tail_fwd",
-                     "of3_attn_pair_bias_fwd", "of3_attn_pair_bias_workspace_bytes"):
+                     "of3_attn_pair_bias_fwd", "of3_attn_pair_bias_workspace_bytes", "of3_transition_rows_fwd",
+                     "of3_transition_rows_workspace_bytes"):
         assert required in names
 
 
@@ -188,3 +189,20 @@ def test_attn_pair_bias_entry_point_validates(lib):
     nul = list(args)
     nul[5] = None                                                                         # b_q missing
     assert lib.of3_attn_pair_bias_fwd(*nul, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+
+
+def test_transition_rows_entry_point_validates(lib):
+    from of3pair import _lib as L
+
+    assert lib.of3_transition_rows_workspace_bytes(768, 384, 1536) == 768 * 1536 * 2
+    for bad in ((0, 384, 1536), (768, 128, 512), (768, 384, 1000), (768, 384, 192)):
+        assert lib.of3_transition_rows_workspace_bytes(*bad) == L.OF3_EINVAL
+    p = 256
+    args = [p, None] + [p] * 6 + [64, 384, 1536, 0, p, 1 << 30]
+    assert lib.of3_transition_rows_fwd(*args, L.OF3_DTYPE_F32, None) == L.OF3_EINVAL
+    small = list(args)
+    small[-1] = 16
+    assert lib.of3_transition_rows_fwd(*small, L.OF3_DTYPE_BF16, None) == L.OF3_ENOSPC
+    nul = list(args)
+    nul[4] = None
+    assert lib.of3_transition_rows_fwd(*nul, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL

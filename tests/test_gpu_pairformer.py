@@ -1,0 +1,123 @@
+"""Parity of the single-representation transition and of whole PairFormerBlocks / a PairFormerStack
+(modules -> C ABI -> HIP) with the CPU oracle on the same seeded inputs and weights.  bf16:
+max-norm 2e-2 relative to the oracle's output plus an rms bound per case."""
+import pytest
+import torch
+
+from gpu_util import lib, report  # noqa: F401
+from oracle import pairstack_oracle as orc
+
+import of3pair
+from of3pair import functional as F3
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+REL = 2e-2
+CFG = dict(c_s=384, c_z=128, c_hidden_pair_bias=24, no_heads_pair_bias=16, c_hidden_mul=128, c_hidden_pair_att=32,
+           no_heads_pair=4, transition_type="swiglu", transition_n=4, pair_dropout=0.25,
+           fuse_projection_weights=False, inf=1e9)
+
+
+def _check(name, got, want, rms_rel=5e-3, bf16_ref=None):
+    got = got.float().cpu()
+    want = want.float()
+    rms = float(want.pow(2).mean().sqrt())
+    report(name, got, want, atol=REL * float(want.abs().max()), rtol=0.0)
+    erms = float((got - want).pow(2).mean().sqrt())
+    assert erms <= rms_rel * rms, "%s: rms error %.3g vs rms %.3g" % (name, erms, rms)
+    if bf16_ref is not None:
+        floor = float((bf16_ref.float() - want).pow(2).mean().sqrt())
+        assert erms <= 1.5 * floor, "%s: rms error %.3g above the bf16 reference path's %.3g" % (name, erms, floor)
+
+
+def _round(p):
+    return {k: orc.round_bf16(v) for k, v in p.items()}
+
+
+# rows cover: one partial tile (5), ragged last tile (100), a batch of sequences (2 x 70), n = 2
+@pytest.mark.parametrize("shape,n_mult,masked", [((5,), 4, False), ((100,), 4, True), ((2, 70), 4, True), ((64,), 2, True)])
+def test_single_transition(shape, n_mult, masked):
+    lib()
+    gen = torch.Generator().manual_seed(900 + shape[-1])
+    p = _round(orc.make_transition_params(gen, 384, n_mult))
+    x = orc.round_bf16(1.5 * torch.randn(*shape, 384, generator=gen) + 0.1)
+    mask = (torch.rand(*shape, generator=gen) > 0.25).float() if masked else None
+    m = of3pair.SwiGLUTransition(384, n_mult)
+    m.load_state_dict(p, strict=True)
+    m = m.to(DEV).to(torch.bfloat16).eval()
+    print("single transition", shape, n_mult, masked, flush=True)
+    xg = x.to(DEV).to(torch.bfloat16)
+    got = m(xg, mask=None if mask is None else mask.to(DEV))
+    want = orc.transition_update(x, mask, p)
+    floor = orc.transition_update(x.to(torch.bfloat16), None if mask is None else mask.to(torch.bfloat16),
+                                  {k: v.to(torch.bfloat16) for k, v in p.items()})
+    _check("single transition update", got, want, bf16_ref=floor)
+    assert torch.equal(xg.float().cpu(), x)
+    if mask is not None:
+        masked_out = got.float().cpu()[mask == 0]
+        assert masked_out.numel() == 0 or float(masked_out.abs().max()) == 0.0
+    res = m(xg, mask=None if mask is None else mask.to(DEV), _add_residual=True, _inplace=True)
+    assert res.data_ptr() == xg.data_ptr()
+    _check("single transition x+update", res, x + want, rms_rel=4e-3)
+
+
+def test_single_transition_rejects_fp32():
+    lib()
+    m = of3pair.SwiGLUTransition(384, 4).to(DEV)
+    with pytest.raises(ValueError):
+        m(torch.zeros(8, 384, device=DEV))
+
+
+@pytest.mark.parametrize("mask_trans", [True, False])
+def test_pairformer_block(mask_trans):
+    """One PairFormerBlock of the AF3 trunk shape at N = 72 with a padded tail: (s, z) against the
+    oracle; inputs intact without inplace_safe, identical results with it."""
+    lib()
+    n = 72
+    p = _round(orc.make_pairformer_block_params(3, 384, 128, 128, 32, 4, 24, 16, 4))
+    gen = torch.Generator().manual_seed(91)
+    s = orc.round_bf16(torch.randn(n, 384, generator=gen))
+    z = orc.round_bf16(orc.make_pair_input(92, (), n, 128))
+    single_mask = torch.ones(n)
+    single_mask[-9:] = 0
+    pair_mask = single_mask[:, None] * single_mask[None, :]
+    blk = of3pair.PairFormerBlock(**CFG)
+    blk.load_state_dict(p, strict=True)
+    blk = blk.to(DEV).to(torch.bfloat16).eval()
+    sg, zg = s.to(DEV).to(torch.bfloat16), z.to(DEV).to(torch.bfloat16)
+    print("pairformer block", mask_trans, flush=True)
+    s_got, z_got = blk(sg, zg, single_mask.to(DEV), pair_mask.to(DEV), chunk_size=4, _mask_trans=mask_trans)
+    s_want, z_want = orc.pairformer_block(s, z, single_mask, pair_mask, p, 4, 16, mask_trans=mask_trans)
+    _check("pairformer block z", z_got, z_want, rms_rel=1e-2)
+    _check("pairformer block s", s_got, s_want, rms_rel=1e-2)
+    assert torch.equal(sg.float().cpu(), s) and torch.equal(zg.float().cpu(), z)
+    s2, z2 = blk(sg.clone(), zg.clone(), single_mask.to(DEV), pair_mask.to(DEV), inplace_safe=True,
+                 _mask_trans=mask_trans)
+    assert torch.equal(s2, s_got) and torch.equal(z2, z_got)
+
+
+def test_pairformer_stack_two_blocks_with_batch():
+    """PairFormerStack(**config) with 2 blocks over a batch of 2: block i loads `blocks.<i>.*`."""
+    lib()
+    n = 48
+    blocks = [_round(orc.make_pairformer_block_params(5 + i, 384, 128, 128, 32, 4, 24, 16, 4)) for i in range(2)]
+    gen = torch.Generator().manual_seed(93)
+    s = orc.round_bf16(torch.randn(2, n, 384, generator=gen))
+    z = orc.round_bf16(orc.make_pair_input(94, (2,), n, 128))
+    single_mask = torch.ones(2, n)
+    single_mask[1, -7:] = 0
+    pair_mask = single_mask[:, :, None] * single_mask[:, None, :]
+    stack = of3pair.PairFormerStack(no_blocks=2, blocks_per_ckpt=None, use_reentrant=False,
+                                    clear_cache_between_blocks=False, tune_chunk_size=False, **CFG)
+    sd = {}
+    for i, p in enumerate(blocks):
+        sd.update({"blocks.%d.%s" % (i, k): v for k, v in p.items()})
+    stack.load_state_dict(sd, strict=True)
+    stack = stack.to(DEV).to(torch.bfloat16).eval()
+    s_got, z_got = stack(s.to(DEV).to(torch.bfloat16), z.to(DEV).to(torch.bfloat16), single_mask.to(DEV),
+                         pair_mask.to(DEV))
+    s_want, z_want = s, z
+    for p in blocks:
+        s_want, z_want = orc.pairformer_block(s_want, z_want, single_mask, pair_mask, p, 4, 16)
+    _check("pairformer stack z", z_got, z_want, rms_rel=1.5e-2)
+    _check("pairformer stack s", s_got, s_want, rms_rel=1.5e-2)

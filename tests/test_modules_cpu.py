@@ -204,3 +204,32 @@ def test_checkpoint_loading_reports_missing_and_unexpected_keys(tmp_path):
     torch.save({k[len("model."):]: v for k, v in sd.items()}, path)
     loaded = ck.state_dict_from_checkpoint(ck.load_checkpoint_file(path))
     assert sorted(loaded) == sorted(sd)
+
+
+def test_pairformer_modules_take_the_reference_config_and_names():
+    """architecture.pairformer of the reference's model config (model_config.py:268-287) constructs
+    the stack; parameter names are the reference's."""
+    cfg = dict(c_s=384, c_z=128, c_hidden_pair_bias=24, no_heads_pair_bias=16, c_hidden_mul=128,
+               c_hidden_pair_att=32, no_heads_pair=4, no_blocks=3, transition_type="swiglu", transition_n=4,
+               pair_dropout=0.25, fuse_projection_weights=False, blocks_per_ckpt=None, inf=1e9, use_reentrant=False,
+               clear_cache_between_blocks=False, tune_chunk_size=False)
+    stack = of3pair.PairFormerStack(**cfg)
+    names = set(stack.state_dict())
+    assert len(stack.blocks) == 3
+    for k in ("pair_stack.tri_mul_out.linear_a_p.weight", "pair_stack.tri_att_end.mha.linear_o.weight",
+              "pair_stack.pair_transition.swiglu.linear_a.weight", "attn_pair_bias.layer_norm_a.weight",
+              "attn_pair_bias.layer_norm_z.bias", "attn_pair_bias.linear_z.weight", "attn_pair_bias.mha.linear_q.weight",
+              "attn_pair_bias.mha.linear_q.bias", "attn_pair_bias.mha.linear_g.weight",
+              "single_transition.layer_norm.weight", "single_transition.swiglu.linear_b.weight",
+              "single_transition.linear_out.weight"):
+        assert "blocks.2." + k in names
+    sd = stack.state_dict()
+    assert tuple(sd["blocks.0.attn_pair_bias.mha.linear_q.weight"].shape) == (384, 384)
+    assert tuple(sd["blocks.0.attn_pair_bias.linear_z.weight"].shape) == (16, 128)
+    assert tuple(sd["blocks.0.single_transition.swiglu.linear_a.weight"].shape) == (1536, 384)
+    assert not any(k.endswith("mha.linear_k.bias") for k in names)
+    sig = inspect.signature(of3pair.PairFormerStack.forward)
+    for name in ("s", "z", "single_mask", "pair_mask", "chunk_size", "inplace_safe", "_mask_trans"):
+        assert name in sig.parameters
+    with pytest.raises(ValueError):
+        of3pair.AttentionPairBias(384, 384, 384, 384, 128, 24, 16, use_ada_layer_norm=True)
