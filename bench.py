@@ -19,7 +19,8 @@ Besides the whole-block time the line carries
                 the entries "pair_transition" (the SwiGLU transition that follows the block in
                 every PairBlock) and "pair_bias_proj" (the 16-head pair bias the single-representation
                 attention of a PairFormerBlock takes from z), "attn_pair_bias" (that attention itself
-                over s [N, 384], 16 heads of 24: its three small kernels as one call) and "template_tail" (closing LayerNorm
+                over s [N, 384], 16 heads of 24: its three small kernels as one call), "single_transition"
+                (the SwiGLU transition of s, n = 4: two small kernels as one call) and "template_tail" (closing LayerNorm
                 of the template stack, mean over 4 templates, ReLU and linear_t, c_t = 64 -> c_z
                 = 128, at the same N) are timed right after the block's kernels and are not part
                 of `value`;
@@ -81,6 +82,8 @@ def kernel_model(B, N, C, CH, H, D):
         "pair_bias_proj": {"bound": "hbm", "bytes": U + B * PAIR_BIAS_HEADS * N * N * 2},
         # LayerNorm + q, k, v, g projections, QK^T and PV over 16 heads of 24, output projection
         "attn_pair_bias": {"bound": "mfma", "flops": 10 * B * N * C_S * C_S + 4 * B * N * N * C_S},
+        # three C_s x 4 C_s products per token
+        "single_transition": {"bound": "mfma", "flops": 6 * B * N * C_S * (TRANSITION_N * C_S)},
         # reads the TEMPLATES planes of c_t channels, writes one c_z plane
         "template_tail": {"bound": "hbm", "bytes": B * N * N * 2 * (TEMPLATES * C_T + C)},
     }
@@ -226,9 +229,16 @@ def main():
         P(sp["mha.linear_q.weight"]), P(sp["mha.linear_q.bias"]), P(sp["mha.linear_k.weight"]),
         P(sp["mha.linear_v.weight"]), P(sp["mha.linear_g.weight"]), P(sp["mha.linear_o.weight"]), P(s_out),
         B, N, C_S, PAIR_BIAS_HEADS, C_HEAD_S, 1e9, 0, P(s_ws), s_ws.numel(), _lib.OF3_DTYPE_BF16, s)))]
+    stp = {k_: v.to(dev).to(bf).contiguous() for k_, v in orc.make_transition_params(tgen, C_S, TRANSITION_N).items()}
+    st_ws = torch.empty(int(lib.of3_transition_rows_workspace_bytes(B * N, C_S, TRANSITION_N * C_S)),
+                        dtype=torch.uint8, device=dev)
+    single_transition = [("single_transition", lambda: ck(lib.of3_transition_rows_fwd(
+        P(s_in), None, P(stp["layer_norm.weight"]), P(stp["layer_norm.bias"]), P(stp["swiglu.linear_a.weight"]),
+        P(stp["swiglu.linear_b.weight"]), P(stp["linear_out.weight"]), P(s_out), B * N, C_S, TRANSITION_N * C_S, 0,
+        P(st_ws), st_ws.numel(), _lib.OF3_DTYPE_BF16, s)))]
     launches = (trimul("tri_mul_out.", 1) + trimul("tri_mul_in.", 0)
                 + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr) + transition
-                + pair_bias + attn_pair_bias + template_tail)
+                + pair_bias + attn_pair_bias + single_transition + template_tail)
     for _ in range(max(args.warmup, 1)):
         for _, fn in launches:
             fn()
