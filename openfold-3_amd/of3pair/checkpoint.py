@@ -3,6 +3,7 @@
 The modules keep the reference's parameter names, so loading is a matter of cutting the right
 slice out of a model state dict:
 
+    model.pairformer_stack.*                              -> PairFormerStack      (model.py:95)
     model.pairformer_stack.blocks.<i>.pair_stack.*        -> PairBlock            (pairformer.py:91)
     model.template_embedder.template_pair_stack.*         -> TemplatePairStack    (template_module.py:395)
     model.template_embedder.linear_t.weight               -> TemplateEmbedderCore (template_module.py:403)
@@ -69,6 +70,12 @@ def load_pairformer_pair_blocks(blocks, state_dict: Mapping, stack: str = "model
     for i, blk in enumerate(blocks):
         load_pair_block(blk, state_dict, "%sblocks.%d.pair_stack." % (stack, i))
     return blocks
+
+
+def load_pairformer_stack(stack, state_dict: Mapping, prefix: str = "model.pairformer_stack."):
+    """PairFormerStack <- every key under `prefix` (blocks.<i>.pair_stack.*, .attn_pair_bias.*,
+    .single_transition.*); the number of blocks must match."""
+    return _load(stack, sub_state_dict(state_dict, prefix), prefix)
 
 
 def load_template_embedder(core, state_dict: Mapping, prefix: str = "model.template_embedder."):

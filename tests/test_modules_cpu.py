@@ -233,3 +233,20 @@ def test_pairformer_modules_take_the_reference_config_and_names():
         assert name in sig.parameters
     with pytest.raises(ValueError):
         of3pair.AttentionPairBias(384, 384, 384, 384, 128, 24, 16, use_ada_layer_norm=True)
+
+
+def test_whole_pairformer_stack_loads_from_a_model_state_dict():
+    from of3pair import checkpoint as ck
+
+    cfg = dict(c_s=384, c_z=128, c_hidden_pair_bias=24, no_heads_pair_bias=16, c_hidden_mul=128,
+               c_hidden_pair_att=32, no_heads_pair=4, no_blocks=2, transition_type="swiglu", transition_n=4,
+               pair_dropout=0.25, fuse_projection_weights=False, blocks_per_ckpt=None, inf=1e9)
+    src = of3pair.PairFormerStack(**cfg)
+    gen = torch.Generator().manual_seed(9)
+    sd = {"model.pairformer_stack." + k: torch.randn(v.shape, generator=gen) for k, v in src.state_dict().items()}
+    sd["model.msa_module.blocks.0.linear.weight"] = torch.zeros(1)
+    dst = ck.load_pairformer_stack(of3pair.PairFormerStack(**cfg), sd)
+    for k, v in dst.state_dict().items():
+        assert torch.equal(v, sd["model.pairformer_stack." + k])
+    with pytest.raises(KeyError):
+        ck.load_pairformer_stack(of3pair.PairFormerStack(**dict(cfg, no_blocks=3)), sd)
