@@ -4,7 +4,7 @@ start + end, residual adds fused) on one MI355X.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--n 768] [--no-cpu]
 
 A step is one block forward, in place, on a z that already lives in HBM.  The workload is
-BASELINE config 3: N_token = 768, c_z = 128, c_hidden_mul = 128, 4 heads x 32, batch 1,
+benchmark configuration 3: N_token = 768, c_z = 128, c_hidden_mul = 128, 4 heads x 32, batch 1,
 all-ones mask, bf16, synthetic N(0,1) input and seeded random weights.  Prints one JSON line.
 
 Besides the whole-block time the line carries

@@ -2,7 +2,7 @@
 
 Tolerance (north star, fp32): max-abs error <= 1e-4.  Inputs are N(0,1), weights N(0, 1/fan_in)
 and LayerNorm affine near identity, so outputs are O(1) and an absolute bound is meaningful;
-BASELINE config 1 (N=64, c_z=128, 4 heads x 32, all-ones mask) is the first case."""
+benchmark configuration 1 (N=64, c_z=128, 4 heads x 32, all-ones mask) is the first case."""
 import pytest
 import torch
 
@@ -61,7 +61,7 @@ def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
 
 
 def test_block_config1_fp32():
-    """BASELINE config 1: B=1, N=64, c_z=128, c_hidden_mul=128, 4 heads x 32, all-ones mask, fp32."""
+    """benchmark configuration 1: B=1, N=64, c_z=128, c_hidden_mul=128, 4 heads x 32, all-ones mask, fp32."""
     lib()
     n, c, d, heads = 64, 128, 32, 4
     p = orc.make_block_params(0, c, c, d, heads)

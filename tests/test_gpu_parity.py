@@ -124,7 +124,7 @@ def _pair_stack(c, ch, d, seed):
 
 
 def test_block_config2_n384_padded():
-    """BASELINE config 2: N=384, c_z=128, last 10% of the tokens padded."""
+    """benchmark configuration 2: N=384, c_z=128, last 10% of the tokens padded."""
     lib()
     n = 384
     m, p = _pair_stack(128, 128, 32, seed=0)
@@ -139,7 +139,7 @@ def test_block_config2_n384_padded():
 
 
 def test_block_config3_n768():
-    """BASELINE config 3 (headline shape): N=768, all-ones mask; in place."""
+    """benchmark configuration 3 (headline shape): N=768, all-ones mask; in place."""
     lib()
     n = 768
     m, p = _pair_stack(128, 128, 32, seed=0)
@@ -153,7 +153,7 @@ def test_block_config3_n768():
 
 
 def test_template_stack_config4():
-    """BASELINE config 4: 2 blocks, 4 templates, N=512, c_t=64, 4 heads x 16, each template
+    """benchmark configuration 4: 2 blocks, 4 templates, N=512, c_t=64, 4 heads x 16, each template
     with its own padded tail (0-20% of the tokens)."""
     lib()
     n, t = 512, 4
@@ -172,7 +172,7 @@ def test_template_stack_config4():
 
 
 def test_config5_n2048_modules_at_sampled_positions():
-    """BASELINE config 5 shape: N=2048, c_z=128, the last 256 tokens padded.  A full fp32
+    """benchmark configuration 5 shape: N=2048, c_z=128, the last 256 tokens padded.  A full fp32
     pass on the CPU is out of reach (16 TFLOP per block), so every module's GPU output is
     compared with the oracle at sampled rows / fibres that include the first and last valid
     and padded tokens (oracle/pairstack_oracle.py: trimul_update_at, triattn_update_rows)."""

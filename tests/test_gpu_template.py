@@ -160,7 +160,7 @@ def test_template_embedder_core_with_shared_mask():
 
 
 def test_template_tail_full_size_rows():
-    """BASELINE template shape (4 templates, N = 384, c_t = 64 -> c_z = 128): the tail is
+    """Template shape of the benchmark configurations (4 templates, N = 384, c_t = 64 -> c_z = 128): the tail is
     position-wise, so the oracle evaluates sampled rows of the same input; every output is finite."""
     lib()
     n, nt = 384, 4

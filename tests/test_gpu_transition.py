@@ -119,7 +119,7 @@ def test_transition_fp32(c, n_mult, n, batch):
 
 @pytest.mark.parametrize("n,rows", [(768, [0, 1, 383, 767]), (2048, [0, 1023, 2047])])
 def test_transition_full_size_at_sampled_rows(n, rows):
-    """BASELINE sizes (N = 768 and 2048, c_z = 128, n = 4): the update is position-wise, so the
+    """Benchmark sizes (N = 768 and 2048, c_z = 128, n = 4): the update is position-wise, so the
     oracle evaluates whole rows of the same input; the rest of the output is checked through
     a size-independent property (masked positions exactly zero, unmasked ones finite)."""
     lib()
@@ -198,7 +198,7 @@ def test_template_pair_blocks_with_transition():
 
 
 def test_pair_block_config2_n384_padded():
-    """BASELINE config 2 shape through the whole PairBlock (pair stack + transition, n = 4)."""
+    """benchmark configuration 2 shape through the whole PairBlock (pair stack + transition, n = 4)."""
     lib()
     import math
     n, c = 384, 128
