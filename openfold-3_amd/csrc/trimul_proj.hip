@@ -49,8 +49,9 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
 
   // LayerNorm affine parameters of this lane's 8 channels, kept packed (8 registers instead
   // of 16) and unpacked once per tile
-  const u32x4_t lw_pk = *reinterpret_cast<const u32x4_t*>(p.ln_w + 8 * ln_chunk);
-  const u32x4_t lb_pk = *reinterpret_cast<const u32x4_t*>(p.ln_b + 8 * ln_chunk);
+  u32x4_t lw_pk = *reinterpret_cast<const u32x4_t*>(p.ln_w + 8 * ln_chunk);
+  u32x4_t lb_pk = *reinterpret_cast<const u32x4_t*>(p.ln_b + 8 * ln_chunk);
+  __asm__ volatile("" : "+v"(lw_pk), "+v"(lb_pk));  // waited for here, once
 
   // this wave's job: gate and projection rows 32*ot .. +31 of a (pair 0) or b (pair 1),
   // resident in registers as MFMA A operands for the whole kernel
@@ -66,6 +67,11 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
       wg[s] = *reinterpret_cast<const u32x4_t*>(Wg + row * C + 16 * s + 8 * lh);
       wp[s] = *reinterpret_cast<const u32x4_t*>(Wp + row * C + 16 * s + 8 * lh);
     }
+    // the weights count as used here: the compiler waits for them once, before the tile loop,
+    // instead of carrying "may still be in flight" into every iteration (where its wait for
+    // them would also be a wait for the tile's prefetch and the previous tile's stores)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) __asm__ volatile("" : "+v"(wg[s]), "+v"(wp[s]));
   }
   bf16_t* const out = pair ? p.b : p.a;
 
@@ -77,47 +83,54 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
   // part of the address is computed once, the tile adds a wave-uniform base.
   const int ln_pos0 = wave * (TP / NW) + ln_pp;
   const int ln_row = ln_pos0 >> 5, ln_k = ln_pos0 & 31;
-  const int64_t ln_off = ln_row * p.z_view.stride_r + ln_k * p.z_view.stride_k + 8 * ln_chunk;
+  // Everything a tile reads from global memory (its z values and this lane's mask values) is
+  // requested one tile ahead by a fixed number of unconditional loads (positions past the end
+  // are clamped to the last one and zeroed through the mask value), and every tile issues the
+  // same 16 stores (the padding rows of a and b are written too, with zeros).  With fixed
+  // counts the compiler's wait for the prefetched values can leave the previous tile's stores
+  // in flight; with a load or store under a condition it cannot, and waits for all of them.
   u32x4_t raw[LN_ITERS];
+  float mraw[TPW];
+  const float* const mask_base = p.mask ? p.mask : reinterpret_cast<const float*>(p.ln_w);  // dummy when absent
+  const int64_t msb = p.mask ? p.mask_view.stride_b : 0, msr = p.mask ? p.mask_view.stride_r : 0,
+                msk = p.mask ? p.mask_view.stride_k : 0;
+  // Positions of the tile are dealt to MFMA columns so that a lane finishes TPW consecutive
+  // positions: position  32*TPW*tgroup + TPW*l32 + tt  is column l32 of this wave's tile tt.
+  const int pos0 = 32 * TPW * tgroup + TPW * l32;
   auto load_tile = [&](int tile_id) {
     const int b = tile_id / tiles_per_batch;
     const int rem = tile_id - b * tiles_per_batch;
     const int r0 = (rem / panels) * TR;
     const int k0 = (rem % panels) * 32;
-    const bf16_t* base = p.z + b * p.z_view.stride_b + r0 * p.z_view.stride_r + k0 * p.z_view.stride_k;
-    const bool row_ok = r0 + ln_row < N;
+    int row = r0 + ln_row;
+    row = row < N ? row : N - 1;
+    const bf16_t* base = p.z + b * p.z_view.stride_b + row * p.z_view.stride_r + 8 * ln_chunk;
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      u32x4_t v = {0u, 0u, 0u, 0u};
-      if (row_ok && k0 + ln_k + it * PPI < N)
-        v = *reinterpret_cast<const u32x4_t*>(base + ln_off + (it * PPI) * p.z_view.stride_k);
-      raw[it] = v;
+      int k = k0 + ln_k + it * PPI;
+      k = k < N ? k : N - 1;
+      raw[it] = *reinterpret_cast<const u32x4_t*>(base + k * p.z_view.stride_k);
+    }
+    int mr = r0 + (pos0 >> 5);
+    mr = mr < N ? mr : N - 1;
+    const float* mrow = mask_base + b * msb + mr * msr;
+#pragma unroll
+    for (int tt = 0; tt < TPW; ++tt) {
+      int k = k0 + (pos0 & 31) + tt;
+      k = k < N ? k : N - 1;
+      mraw[tt] = mrow[k * msk];
     }
   };
 
-  // Positions of the tile are dealt to MFMA columns so that a lane finishes TPW consecutive
-  // positions: position  32*TPW*tgroup + TPW*l32 + tt  is column l32 of this wave's tile tt.
-  const int pos0 = 32 * TPW * tgroup + TPW * l32;
-
-  int tile_id = blockIdx.x;
-  if (tile_id < total_tiles) load_tile(tile_id);
-
-  for (int buf = 0; tile_id < total_tiles; tile_id += gridDim.x, buf ^= 1) {
+  auto do_tile = [&](int tile_id, int buf) {
     const int b = tile_id / tiles_per_batch;
     const int rem = tile_id - b * tiles_per_batch;
     const int r = (rem / panels) * TR + (pos0 >> 5);  // this lane's row and first k
     const int kfirst = (rem % panels) * 32 + (pos0 & 31);
 
     float mval[TPW];
-    const float* mrow = p.mask ? p.mask + b * p.mask_view.stride_b + r * p.mask_view.stride_r +
-                                     kfirst * p.mask_view.stride_k
-                               : nullptr;
 #pragma unroll
-    for (int tt = 0; tt < TPW; ++tt) {
-      float m = 0.f;
-      if (kfirst + tt < N && r < N) m = mrow ? mrow[tt * p.mask_view.stride_k] : 1.f;
-      mval[tt] = m;
-    }
+    for (int tt = 0; tt < TPW; ++tt) mval[tt] = (kfirst + tt < N && r < N) ? (p.mask ? mraw[tt] : 1.f) : 0.f;
 
     // ---- LayerNorm phase: wave w normalises positions [16w, 16w+16) of the tile
     float lw[8], lb[8];
@@ -154,8 +167,9 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
       for (int v = 0; v < 16; ++v) res[tt][v] = (mval[tt] * sigmoidf_fast(accg[v])) * accp[v];
     }
     // stores: register v of a lane is channel 32*ot + 8*(v/4) + 4*lh + v%4; k-panel layout
-    // plane[k / 32][row][k % 32]
-    if (r < N) {
+    // plane[k / 32][row][k % 32].  r < Np always (Np is a multiple of 128): rows between N and
+    // Np receive zeros
+    {
       // lane base: channel 32*ot + 4*lh of this batch element, row r, first k of the lane;
       // the 16 registers add wave-uniform channel offsets
       const size_t plane = (size_t)Np * Np;
@@ -172,7 +186,18 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
         }
       }
     }
+  };
+
+  // the first tile is peeled: the loop proper is only entered with a tile's stores in flight
+  int tile_id = blockIdx.x;
+  int buf = 0;
+  if (tile_id < total_tiles) {
+    load_tile(tile_id);
+    do_tile(tile_id, buf);
+    tile_id += gridDim.x;
+    buf ^= 1;
   }
+  for (; tile_id < total_tiles; tile_id += gridDim.x, buf ^= 1) do_tile(tile_id, buf);
 }
 
 template <int C, int CH>
