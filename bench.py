@@ -24,6 +24,9 @@ Besides the whole-block time the line carries
                 of the template stack, mean over 4 templates, ReLU and linear_t, c_t = 64 -> c_z
                 = 128, at the same N) are timed right after the block's kernels and are not part
                 of `value`;
+  pairformer_block_ms  wall clock of one whole PairFormerBlock (of3pair.PairFormerBlock: the pair-stack
+                block plus pair transition, pair bias, attention over s and single transition) at
+                the same N, for orientation; not part of `value`;
   cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path)
                 timed once on the host cores for the same workload.
 """
@@ -273,6 +276,24 @@ def main():
     roofline = {"kernel": "trimul_contract", "bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS,
                 "unit": "TFLOP/s", "frac": dom["frac"], "traffic": MEASURED_TRAFFIC.get(("trimul_contract", N))}
 
+    # ---- a whole PairFormerBlock through the module interface (pair stack, pair transition, pair
+    # bias, attention over s, single transition), wall clock; informative, not part of `value`
+    import of3pair
+    pf = of3pair.PairFormerBlock(C_S, C, C_HEAD_S, PAIR_BIAS_HEADS, CH, D, H, "swiglu", TRANSITION_N, 0.25, False, 1e9)
+    pf.load_state_dict({k_: v for k_, v in orc.make_pairformer_block_params(0, C_S, C, CH, D, H, C_HEAD_S,
+                                                                             PAIR_BIAS_HEADS, TRANSITION_N).items()})
+    pf = pf.to(dev).to(bf).eval()
+    s_pf, z_pf = torch.randn(B, N, C_S, device=dev).to(bf), z_host.to(dev).to(bf)
+    sm, pm = torch.ones(B, N, device=dev), torch.ones(B, N, N, device=dev)
+    for _ in range(2):
+        pf(s_pf, z_pf, sm, pm, inplace_safe=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        pf(s_pf, z_pf, sm, pm, inplace_safe=True)
+    torch.cuda.synchronize()
+    pairformer_block_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
     # ---- CPU baseline: the oracle on the host cores, one block of the same workload
     cpu = None
     if not args.no_cpu:
@@ -292,6 +313,7 @@ def main():
         "config": {"workload": "pair-stack block (trimul out+in, tri-attn start+end, residuals), B=1, N_token=%d, "
                                "c_z=128, c_hidden_mul=128, 4 heads x 32, all-ones mask" % N},
         "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
+        "pairformer_block_ms": round(pairformer_block_ms, 4),
     }
     print(json.dumps(line))
 

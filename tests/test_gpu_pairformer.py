@@ -121,3 +121,43 @@ def test_pairformer_stack_two_blocks_with_batch():
         s_want, z_want = orc.pairformer_block(s_want, z_want, single_mask, pair_mask, p, 4, 16)
     _check("pairformer stack z", z_got, z_want, rms_rel=1.5e-2)
     _check("pairformer stack s", s_got, s_want, rms_rel=1.5e-2)
+
+
+def test_pairformer_block_in_a_hip_graph_replays_like_eager():
+    """A whole PairFormerBlock (about thirty kernel launches) captured once its one-time set-up has
+    run; replays with eager work and synchronisations in between must reproduce the eager result
+    bit for bit, also for a new input copied into the static buffers."""
+    lib()
+    n = 64
+    p = _round(orc.make_pairformer_block_params(11, 384, 128, 128, 32, 4, 24, 16, 4))
+    blk = of3pair.PairFormerBlock(**CFG)
+    blk.load_state_dict(p, strict=True)
+    blk = blk.to(DEV).to(torch.bfloat16).eval()
+    gen = torch.Generator().manual_seed(95)
+    s0 = orc.round_bf16(torch.randn(n, 384, generator=gen)).to(DEV).to(torch.bfloat16)
+    z0 = orc.round_bf16(orc.make_pair_input(96, (), n, 128)).to(DEV).to(torch.bfloat16)
+    single_mask = torch.ones(n, device=DEV)
+    single_mask[-5:] = 0
+    pair_mask = single_mask[:, None] * single_mask[None, :]
+    s_eager, z_eager = blk(s0, z0, single_mask, pair_mask)  # also the warm-up: workspaces exist now
+    torch.cuda.synchronize()
+    s_static, z_static = s0.clone(), z0.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        s_out, z_out = blk(s_static, z_static, single_mask, pair_mask)
+    for rep in range(3):
+        s_static.copy_(s0)
+        z_static.copy_(z0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(s_out, s_eager) and torch.equal(z_out, z_eager), "replay %d differs" % rep
+        other_s, other_z = blk(s0 * 0.5, z0 * 0.5, single_mask, pair_mask)  # eager work on the same workspaces
+        assert torch.isfinite(other_s).all() and torch.isfinite(other_z).all()
+        torch.cuda.synchronize()
+    s1 = orc.round_bf16(torch.randn(n, 384, generator=gen)).to(DEV).to(torch.bfloat16)
+    s_static.copy_(s1)
+    z_static.copy_(z0)
+    graph.replay()
+    torch.cuda.synchronize()
+    s_want, z_want = blk(s1, z0, single_mask, pair_mask)
+    assert torch.equal(s_out, s_want) and torch.equal(z_out, z_want)
