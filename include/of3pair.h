@@ -55,7 +55,8 @@
  *
  * dtype: OF3_DTYPE_BF16 selects the MFMA kernels described above.  OF3_DTYPE_F32 (the
  * reference's default inference precision) is served by of3_trimul_fwd / of3_triattn_fwd /
- * of3_transition_fwd / of3_pair_bias_fwd / of3_layer_norm_fwd / of3_template_tail_fwd only:
+ * of3_transition_fwd / of3_pair_bias_fwd / of3_layer_norm_fwd / of3_template_tail_fwd /
+ * of3_attn_pair_bias_fwd / of3_transition_rows_fwd only:
  * every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
  * element counts, any N, C and CH <= 256, H*D <= 256 with D in {16, 32, 64}; plain fp32
  * arithmetic in the reference's order of operations (no MFMA, not the fast path).  The
@@ -179,10 +180,12 @@ int of3_pair_bias_fwd(const void* z, const int64_t z_strides[3], const void* ln_
  * with an = LayerNorm(a), q = an Wq^T + bq, k = an Wk^T, v = an Wv^T split into H heads of width D.
  * a, out: contiguous [B][N][C_s] (out may alias a); pair_bias: contiguous [B][H][N][N], what
  * of3_pair_bias_fwd returns for this module's layer_norm_z / linear_z; mask: fp32 [B][N] or null
- * (all ones); w_q, w_k, w_v, w_g: [H*D][C_s]; b_q: [H*D]; w_o: [C_s][H*D].  bf16 only, the AF3
- * trunk shape: C_s = H*D = 384, D in {8, 16, 24} (16 heads of 24).  The workspace holds
- * q, k, v, the gate and the gated attention output. */
+ * (all ones); w_q, w_k, w_v, w_g: [H*D][C_s]; b_q: [H*D]; w_o: [C_s][H*D].  bf16: the AF3 trunk
+ * shape, C_s = H*D = 384, D in {8, 16, 24} (16 heads of 24); fp32: C_s <= 512, H*D <= 512,
+ * D <= 64.  The workspace holds q, k, v, the gate and the gated attention output
+ * (of3_attn_pair_bias_workspace_bytes: bf16; ..._for: either dtype). */
 int64_t of3_attn_pair_bias_workspace_bytes(int64_t B, int64_t N, int64_t C_s, int64_t H, int64_t D);
+int64_t of3_attn_pair_bias_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C_s, int64_t H, int64_t D);
 int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* mask, const void* ln_w,
                            const void* ln_b, const void* w_q, const void* b_q, const void* w_k, const void* w_v,
                            const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C_s, int64_t H,
@@ -193,9 +196,11 @@ int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* ma
 
 /* The same update as of3_transition_fwd for the single representation (PairFormerBlock's
  * single_transition, pairformer.py:118-122, :203-212): x, out contiguous [rows][C] (any leading
- * dimensions flattened; out may alias x), mask fp32 [rows] or null.  bf16 only, C = 384, HID a
- * multiple of 384.  The workspace holds the hidden activations [rows][HID]. */
+ * dimensions flattened; out may alias x), mask fp32 [rows] or null.  bf16: C = 384, HID a
+ * multiple of 384, the workspace holds the hidden activations [rows][HID]; fp32: C <= 512,
+ * HID <= 2048, no workspace (null, 0 is accepted). */
 int64_t of3_transition_rows_workspace_bytes(int64_t rows, int64_t C, int64_t HID);
+int64_t of3_transition_rows_workspace_bytes_for(int dtype, int64_t rows, int64_t C, int64_t HID);
 int of3_transition_rows_fwd(const void* x, const float* mask, const void* ln_w, const void* ln_b, const void* w_a,
                             const void* w_b, const void* w_out, void* out, int64_t rows, int64_t C, int64_t HID,
                             int add_residual, void* workspace, int64_t workspace_bytes, int dtype, void* stream);

@@ -162,6 +162,29 @@ struct RowTransitionArgs {
 };
 hipError_t row_transition_launch(const RowTransitionArgs& args, hipStream_t stream);
 
+// ---- fp32 versions of the single-representation kernels (single_f32.hip)
+struct SingleAttnF32Args {
+  const float* a;            // [B][N][C]
+  const float* pair_bias;    // [B][H][N][N]
+  const float* mask;         // [B][N] or null
+  const float *ln_w, *ln_b, *wq, *bq, *wk, *wv, *wg, *wo;
+  float *q, *k, *v, *g, *og;  // workspace, [B][N][H*D] each
+  float* out;                 // [B][N][C]; may alias a
+  float inf;
+  int B, N, C, H, D, add_residual;
+};
+hipError_t single_attn_fwd_f32(const SingleAttnF32Args& args, hipStream_t stream);
+
+struct RowTransitionF32Args {
+  const float* x;
+  const float* mask;
+  const float *ln_w, *ln_b, *wa, *wb, *wout;
+  float* out;
+  long rows;
+  int C, HID, add_residual;
+};
+hipError_t row_transition_fwd_f32(const RowTransitionF32Args& args, hipStream_t stream);
+
 // ---- fp32 path (pair_f32.hip): whole updates, any N, C and C_hidden <= 256, head width 16/32/64
 struct TrimulF32Args {
   const float* z;

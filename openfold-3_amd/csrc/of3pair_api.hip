@@ -563,11 +563,58 @@ int64_t of3_attn_pair_bias_workspace_bytes(int64_t B, int64_t N, int64_t C_s, in
   return 3 * align256(B * H * Np * 32 * 2) + 2 * align256(B * N * H * D * 2);
 }
 
+int64_t of3_attn_pair_bias_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C_s, int64_t H, int64_t D) {
+  if (dtype == OF3_DTYPE_BF16) return of3_attn_pair_bias_workspace_bytes(B, N, C_s, H, D);
+  if (dtype != OF3_DTYPE_F32 || B < 1 || B > 65535 || N < 1 || N > (1 << 16) || C_s < 1 || C_s > 512 || H < 1 ||
+      D < 1 || D > 64 || H * D > 512)
+    return OF3_EINVAL;
+  return 5 * align256(B * N * H * D * 4);
+}
+
 int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* mask, const void* ln_w,
                            const void* ln_b, const void* w_q, const void* b_q, const void* w_k, const void* w_v,
                            const void* w_g, const void* w_o, void* out, int64_t B, int64_t N, int64_t C_s, int64_t H,
                            int64_t D, float inf, int add_residual, void* workspace, int64_t workspace_bytes,
                            int dtype, void* stream) {
+  if (dtype == OF3_DTYPE_F32) {
+    const int64_t need32 = of3_attn_pair_bias_workspace_bytes_for(dtype, B, N, C_s, H, D);
+    if (need32 < 0) return OF3_EINVAL;
+    const void* p32[] = {a, pair_bias, ln_w, ln_b, w_q, b_q, w_k, w_v, w_g, w_o, out, workspace};
+    for (const void* p : p32)
+      if (!p || !aligned4(p)) return OF3_EINVAL;
+    if (mask && !aligned4(mask)) return OF3_EINVAL;
+    if (workspace_bytes < need32) return OF3_ENOSPC;
+    const int64_t part = align256(B * N * H * D * 4);
+    char* ws = static_cast<char*>(workspace);
+    auto f = [](const void* p) { return static_cast<const float*>(p); };
+    of3::SingleAttnF32Args s;
+    s.a = f(a);
+    s.pair_bias = f(pair_bias);
+    s.mask = mask;
+    s.ln_w = f(ln_w);
+    s.ln_b = f(ln_b);
+    s.wq = f(w_q);
+    s.bq = f(b_q);
+    s.wk = f(w_k);
+    s.wv = f(w_v);
+    s.wg = f(w_g);
+    s.wo = f(w_o);
+    s.q = reinterpret_cast<float*>(ws);
+    s.k = reinterpret_cast<float*>(ws + part);
+    s.v = reinterpret_cast<float*>(ws + 2 * part);
+    s.g = reinterpret_cast<float*>(ws + 3 * part);
+    s.og = reinterpret_cast<float*>(ws + 4 * part);
+    s.out = static_cast<float*>(out);
+    s.inf = inf;
+    s.B = (int)B;
+    s.N = (int)N;
+    s.C = (int)C_s;
+    s.H = (int)H;
+    s.D = (int)D;
+    s.add_residual = add_residual ? 1 : 0;
+    hipError_t e = of3::single_attn_fwd_f32(s, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? OF3_OK : fail_hip(e);
+  }
   if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
   const int64_t need = of3_attn_pair_bias_workspace_bytes(B, N, C_s, H, D);
   if (need < 0 || B > 65535) return OF3_EINVAL;
@@ -613,9 +660,39 @@ int64_t of3_transition_rows_workspace_bytes(int64_t rows, int64_t C, int64_t HID
   return align256(rows * HID * 2);
 }
 
+int64_t of3_transition_rows_workspace_bytes_for(int dtype, int64_t rows, int64_t C, int64_t HID) {
+  if (dtype == OF3_DTYPE_BF16) return of3_transition_rows_workspace_bytes(rows, C, HID);
+  if (dtype != OF3_DTYPE_F32 || rows < 1 || rows > (1ll << 31) || C < 1 || C > 512 || HID < 1 || HID > 2048)
+    return OF3_EINVAL;
+  return 0;  // the hidden activations stay on chip
+}
+
 int of3_transition_rows_fwd(const void* x, const float* mask, const void* ln_w, const void* ln_b, const void* w_a,
                             const void* w_b, const void* w_out, void* out, int64_t rows, int64_t C, int64_t HID,
                             int add_residual, void* workspace, int64_t workspace_bytes, int dtype, void* stream) {
+  if (dtype == OF3_DTYPE_F32) {
+    if (of3_transition_rows_workspace_bytes_for(dtype, rows, C, HID) < 0) return OF3_EINVAL;
+    const void* p32[] = {x, ln_w, ln_b, w_a, w_b, w_out, out};
+    for (const void* p : p32)
+      if (!p || !aligned4(p)) return OF3_EINVAL;
+    if (mask && !aligned4(mask)) return OF3_EINVAL;
+    auto f = [](const void* p) { return static_cast<const float*>(p); };
+    of3::RowTransitionF32Args a;
+    a.x = f(x);
+    a.mask = mask;
+    a.ln_w = f(ln_w);
+    a.ln_b = f(ln_b);
+    a.wa = f(w_a);
+    a.wb = f(w_b);
+    a.wout = f(w_out);
+    a.out = static_cast<float*>(out);
+    a.rows = (long)rows;
+    a.C = (int)C;
+    a.HID = (int)HID;
+    a.add_residual = add_residual ? 1 : 0;
+    hipError_t e = of3::row_transition_fwd_f32(a, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? OF3_OK : fail_hip(e);
+  }
   if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
   const int64_t need = of3_transition_rows_workspace_bytes(rows, C, HID);
   if (need < 0) return OF3_EINVAL;

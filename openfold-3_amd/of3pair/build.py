@@ -32,6 +32,7 @@ SOURCES = [
     "single_attn.hip",
     "single_transition.hip",
     "pair_f32.hip",
+    "single_f32.hip",
 ]
 
 # packed fp32 VALU ops are disabled on purpose (device code only)

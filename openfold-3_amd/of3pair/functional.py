@@ -198,8 +198,6 @@ def _swiglu_transition_rows(x, mask, norm_weight, norm_bias, a_weight, b_weight,
     """The transition over the single representation s [*, 384] (pairformer.py:203-212): every
     leading dimension is a row; mask [*] or None."""
     lib = _lib.load()
-    if x.dtype != torch.bfloat16:
-        raise ValueError("single transition: the kernels are bf16 only, got %s" % x.dtype)
     C = x.shape[-1]
     HID = a_weight.shape[0]
     if tuple(a_weight.shape) != (HID, C) or tuple(b_weight.shape) != (HID, C) or tuple(out_weight.shape) != (C, HID):
@@ -212,11 +210,11 @@ def _swiglu_transition_rows(x, mask, norm_weight, norm_bias, a_weight, b_weight,
         if tuple(mask.shape) != tuple(x.shape[:-1]):
             mask = mask.expand(*x.shape[:-1])
         m = mask.to(torch.float32).contiguous()
-    need = lib.of3_transition_rows_workspace_bytes(rows, C, HID)
+    need = lib.of3_transition_rows_workspace_bytes_for(code, rows, C, HID)
     if need < 0:
-        raise ValueError("single transition: c_in = 384 with a hidden width that is a multiple of 384; got hidden=%d"
-                         % HID)
-    ws = _workspace(x.device, need)
+        raise ValueError("single transition: bf16 supports c_in = 384 with a hidden width that is a multiple of 384, "
+                         "fp32 c_in <= 512 and hidden <= 2048; got hidden=%d in %s" % (HID, x.dtype))
+    ws = _workspace(x.device, max(need, 256))
     keep = [_w(t, x.dtype) for t in (norm_weight, norm_bias, a_weight, b_weight, out_weight)]
     with torch.cuda.device(x.device):
         st = lib.of3_transition_rows_fwd(xc.data_ptr(), None if m is None else m.data_ptr(),
@@ -310,10 +308,8 @@ def attention_pair_bias(a, z, mask, norm_a_weight, norm_a_bias, norm_z_weight, n
     """AttentionPairBias.forward of the trunk (attention_pair_bias.py:189-244): attention over
     the single representation a [*, N, C_s] with the pair bias of z [*, N, N, C_z] and the key
     mask [*, N].  Returns the update (or a + update with add_residual; inplace writes into a).
-    bf16 only, C_s = no_heads * head width = 384."""
+    bf16: C_s = no_heads * head width = 384; fp32: C_s <= 512."""
     code = _require_gpu(a, "a")
-    if a.dtype != torch.bfloat16:
-        raise ValueError("attention_pair_bias: the kernels are bf16 only, got %s" % a.dtype)
     lib = _lib.load()
     bias = pair_bias(z, norm_z_weight, norm_z_bias, z_weight)  # [*, H, N, N]
     lead = a.shape[:-2]
@@ -333,10 +329,10 @@ def attention_pair_bias(a, z, mask, norm_a_weight, norm_a_bias, norm_z_weight, n
     m = None
     if mask is not None:
         m = mask.to(torch.float32).expand(*lead, N).contiguous()
-    need = lib.of3_attn_pair_bias_workspace_bytes(B, N, CS, H, D)
+    need = lib.of3_attn_pair_bias_workspace_bytes_for(code, B, N, CS, H, D)
     if need < 0:
-        raise ValueError("attention_pair_bias: supported shape is C_s = no_heads * c = 384 with c a multiple of 8 "
-                         "up to 24; got C_s=%d heads=%d c=%d" % (CS, H, D))
+        raise ValueError("attention_pair_bias: bf16 supports C_s = no_heads * c = 384 with c a multiple of 8 up to "
+                         "24, fp32 C_s <= 512 and c <= 64; got C_s=%d heads=%d c=%d in %s" % (CS, H, D, a.dtype))
     ws = _workspace(a.device, need)
     w = [_w(t, a.dtype) for t in (norm_a_weight, norm_a_bias, q_weight, q_bias, k_weight, v_weight, g_weight, o_weight)]
     with torch.cuda.device(a.device):

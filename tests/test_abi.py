@@ -36,7 +36,8 @@ def test_header_declares_expected_entry_points():
                      "of3_trimul_workspace_bytes_for", "of3_triattn_workspace_bytes_for",
                      "of3_transition_fwd", "of3_pair_bias_fwd", "of3_layer_norm_fwd", "of3_template_tail_fwd",
                      "of3_attn_pair_bias_fwd", "of3_attn_pair_bias_workspace_bytes", "of3_transition_rows_fwd",
-                     "of3_transition_rows_workspace_bytes"):
+                     "of3_transition_rows_workspace_bytes", "of3_attn_pair_bias_workspace_bytes_for",
+                     "of3_transition_rows_workspace_bytes_for"):
         assert required in names
 
 
@@ -182,7 +183,14 @@ def test_attn_pair_bias_entry_point_validates(lib):
         assert lib.of3_attn_pair_bias_workspace_bytes(*bad) == L.OF3_EINVAL
     p = 256
     args = [p] * 2 + [None] + [p] * 9 + [1, 64, 384, 16, 24, 1e9, 0, p, 1 << 30]
-    assert lib.of3_attn_pair_bias_fwd(*args, L.OF3_DTYPE_F32, None) == L.OF3_EINVAL      # bf16 only
+    assert lib.of3_attn_pair_bias_fwd(*args, 7, None) == L.OF3_EINVAL                     # unknown dtype
+    wide = list(args)
+    wide[14] = 1024                                                                       # C_s beyond the fp32 kernels
+    assert lib.of3_attn_pair_bias_fwd(*wide, L.OF3_DTYPE_F32, None) == L.OF3_EINVAL
+    assert lib.of3_attn_pair_bias_workspace_bytes_for(L.OF3_DTYPE_F32, 2, 100, 384, 16, 24) == 5 * 2 * 100 * 384 * 4
+    assert lib.of3_attn_pair_bias_workspace_bytes_for(L.OF3_DTYPE_BF16, 1, 768, 384, 16, 24) == \
+        lib.of3_attn_pair_bias_workspace_bytes(1, 768, 384, 16, 24)
+    assert lib.of3_attn_pair_bias_workspace_bytes_for(L.OF3_DTYPE_F32, 1, 100, 384, 4, 96) == L.OF3_EINVAL
     small = list(args)
     small[-1] = 1024
     assert lib.of3_attn_pair_bias_fwd(*small, L.OF3_DTYPE_BF16, None) == L.OF3_ENOSPC
@@ -199,7 +207,12 @@ def test_transition_rows_entry_point_validates(lib):
         assert lib.of3_transition_rows_workspace_bytes(*bad) == L.OF3_EINVAL
     p = 256
     args = [p, None] + [p] * 6 + [64, 384, 1536, 0, p, 1 << 30]
-    assert lib.of3_transition_rows_fwd(*args, L.OF3_DTYPE_F32, None) == L.OF3_EINVAL
+    assert lib.of3_transition_rows_fwd(*args, 7, None) == L.OF3_EINVAL
+    wide = list(args)
+    wide[10] = 4096                                                                       # hidden width beyond the fp32 kernel
+    assert lib.of3_transition_rows_fwd(*wide, L.OF3_DTYPE_F32, None) == L.OF3_EINVAL
+    assert lib.of3_transition_rows_workspace_bytes_for(L.OF3_DTYPE_F32, 768, 384, 1536) == 0
+    assert lib.of3_transition_rows_workspace_bytes_for(L.OF3_DTYPE_F32, 768, 600, 1536) == L.OF3_EINVAL
     small = list(args)
     small[-1] = 16
     assert lib.of3_transition_rows_fwd(*small, L.OF3_DTYPE_BF16, None) == L.OF3_ENOSPC

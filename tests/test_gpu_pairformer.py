@@ -61,11 +61,41 @@ def test_single_transition(shape, n_mult, masked):
     _check("single transition x+update", res, x + want, rms_rel=4e-3)
 
 
-def test_single_transition_rejects_fp32():
+@pytest.mark.parametrize("shape,n_mult", [((50,), 4), ((2, 19), 2)])
+def test_single_transition_fp32(shape, n_mult):
     lib()
-    m = of3pair.SwiGLUTransition(384, 4).to(DEV)
-    with pytest.raises(ValueError):
-        m(torch.zeros(8, 384, device=DEV))
+    gen = torch.Generator().manual_seed(940 + shape[-1])
+    p = orc.make_transition_params(gen, 384, n_mult)
+    x = 1.5 * torch.randn(*shape, 384, generator=gen) + 0.1
+    mask = (torch.rand(*shape, generator=gen) > 0.25).float()
+    m = of3pair.SwiGLUTransition(384, n_mult)
+    m.load_state_dict(p, strict=True)
+    m = m.to(DEV).eval()
+    got = m(x.to(DEV), mask=mask.to(DEV))
+    want = orc.transition_update(x, mask, p)
+    report("single transition fp32", got.cpu(), want, atol=1e-4, rtol=0.0)
+    res = m(x.to(DEV), mask=None, _add_residual=True)
+    report("single transition fp32 x+update", res.cpu(), x + orc.transition_update(x, None, p), atol=1e-4, rtol=0.0)
+
+
+def test_pairformer_block_fp32():
+    """The whole block in fp32 (small widths keep the CPU oracle quick): max-abs 1e-4."""
+    lib()
+    n = 40
+    p = orc.make_pairformer_block_params(21, 384, 128, 128, 32, 4, 24, 16, 4)
+    gen = torch.Generator().manual_seed(97)
+    s = torch.randn(n, 384, generator=gen)
+    z = orc.make_pair_input(98, (), n, 128)
+    single_mask = torch.ones(n)
+    single_mask[-6:] = 0
+    pair_mask = single_mask[:, None] * single_mask[None, :]
+    blk = of3pair.PairFormerBlock(**CFG)
+    blk.load_state_dict(p, strict=True)
+    blk = blk.to(DEV).eval()
+    s_got, z_got = blk(s.to(DEV), z.to(DEV), single_mask.to(DEV), pair_mask.to(DEV))
+    s_want, z_want = orc.pairformer_block(s, z, single_mask, pair_mask, p, 4, 16)
+    report("pairformer block fp32 z", z_got.cpu(), z_want, atol=2e-4, rtol=0.0)
+    report("pairformer block fp32 s", s_got.cpu(), s_want, atol=2e-4, rtol=0.0)
 
 
 @pytest.mark.parametrize("mask_trans", [True, False])

@@ -103,6 +103,31 @@ def test_attention_pair_bias_rejects_unsupported():
     z = torch.zeros(8, 8, 128, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
         m(a, z)
-    m2 = of3pair.AttentionPairBias(C_S, C_S, C_S, C_S, C_Z, C_HEAD, HEADS).to(DEV)
+    m2 = of3pair.AttentionPairBias(768, 768, 768, 768, C_Z, 48, 16).to(DEV)  # c_s beyond the fp32 kernels
     with pytest.raises(ValueError):
-        m2(torch.zeros(8, C_S, device=DEV), torch.zeros(8, 8, C_Z, device=DEV))  # fp32
+        m2(torch.zeros(8, 768, device=DEV), torch.zeros(8, 8, C_Z, device=DEV))
+
+
+@pytest.mark.parametrize("n,batch,c_s,c_head,heads,masked", [(37, (), 384, 24, 16, True), (130, (2,), 96, 12, 8, True),
+                                                             (16, (), 256, 64, 4, False)])
+def test_attention_pair_bias_fp32(n, batch, c_s, c_head, heads, masked):
+    """fp32 (the reference's default inference precision): max-abs 1e-4 against the oracle."""
+    lib()
+    gen = torch.Generator().manual_seed(850 + n)
+    p = orc.make_attention_pair_bias_params(gen, c_s, 64, c_head, heads)
+    a = torch.randn(*batch, n, c_s, generator=gen)
+    z = orc.make_pair_input(851 + n, batch, n, 64)
+    mask = None
+    if masked:
+        mask = torch.ones(*batch, n)
+        mask[..., n - 5:] = 0
+    m = of3pair.AttentionPairBias(c_s, c_s, c_s, c_s, 64, c_head, heads)
+    m.load_state_dict(p, strict=True)
+    m = m.to(DEV).eval()
+    got = m(a.to(DEV), z.to(DEV), mask=None if mask is None else mask.to(DEV))
+    want = orc.attention_pair_bias(a, z, mask, p, heads)
+    report("attention pair bias fp32", got.cpu(), want, atol=1e-4, rtol=0.0)
+    ag = a.to(DEV)
+    res = m(ag, z.to(DEV), mask=None if mask is None else mask.to(DEV), _add_residual=True, _inplace=True)
+    assert res.data_ptr() == ag.data_ptr()
+    report("attention pair bias fp32 a+update", res.cpu(), a + want, atol=1e-4, rtol=0.0)
