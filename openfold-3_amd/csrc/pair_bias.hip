@@ -10,6 +10,7 @@
 // consecutive positions of one head, i.e. 32 contiguous output bytes.
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -117,17 +118,10 @@ __global__ __launch_bounds__(512) void pair_bias_kernel(PairBiasArgs p, int tile
 template <int C>
 hipError_t launch(const PairBiasArgs& a, hipStream_t stream) {
   auto kern = pair_bias_kernel<C>;
-  static int grid_cap = 0;
-  if (grid_cap == 0) {
-    int dev = 0, cus = 0, per_cu = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 512, 0);
-    if (e != hipSuccess) return e;
-    grid_cap = cus * (per_cu > 0 ? per_cu : 1);
-  }
+  static int cache[kMaxDevices];
+  int grid_cap = 0;
+  hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 512, dev, v); }, &grid_cap);
+  if (e != hipSuccess) return e;
   const int tiles_per_row = (a.N + 255) / 256;
   const long total = (long)a.B * a.N * tiles_per_row;
   const int grid = (int)(total < grid_cap ? total : grid_cap);

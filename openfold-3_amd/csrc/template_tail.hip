@@ -16,6 +16,7 @@
 // one position, 32 contiguous bytes) and the positions as B operands read from the LDS tile.
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -172,28 +173,15 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const bf16_t* __restric
   }
 }
 
-int grid_cap_for(const void* kern, int threads, hipError_t* err) {
-  int dev = 0, cus = 0, per_cu = 0;
-  *err = hipGetDevice(&dev);
-  if (*err != hipSuccess) return 0;
-  *err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-  if (*err != hipSuccess) return 0;
-  *err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, threads, 0);
-  if (*err != hipSuccess) return 0;
-  return cus * (per_cu > 0 ? per_cu : 1);
-}
-
 }  // namespace
 
 hipError_t template_tail_launch(const TemplateTailArgs& a, int CT, int CZ, hipStream_t stream) {
   if (CT != 64 || CZ != 128 || a.T < 1 || a.P < 1 || a.B < 1) return hipErrorInvalidValue;
   auto kern = template_tail_kernel<64, 128>;
-  static int grid_cap = 0;
-  if (grid_cap == 0) {
-    hipError_t e;
-    grid_cap = grid_cap_for(reinterpret_cast<const void*>(kern), 512, &e);
-    if (e != hipSuccess) return e;
-  }
+  static int cache[kMaxDevices];
+  int grid_cap = 0;
+  hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 512, dev, v); }, &grid_cap);
+  if (e != hipSuccess) return e;
   const long tiles_per_batch = (a.P + 255) / 256;
   const long total = tiles_per_batch * a.B;
   if (total > 0x7fffffffl) return hipErrorInvalidValue;
@@ -205,12 +193,11 @@ hipError_t template_tail_launch(const TemplateTailArgs& a, int CT, int CZ, hipSt
 hipError_t layer_norm_launch(const bf16_t* x, const bf16_t* w, const bf16_t* b, bf16_t* out, long rows, int C,
                              hipStream_t stream) {
   if (rows < 1 || !(C == 64 || C == 128)) return hipErrorInvalidValue;
-  static int grid_cap = 0;
-  if (grid_cap == 0) {
-    hipError_t e;
-    grid_cap = grid_cap_for(reinterpret_cast<const void*>(layer_norm_kernel<128>), 256, &e);
-    if (e != hipSuccess) return e;
-  }
+  static int cache[kMaxDevices];
+  int grid_cap = 0;
+  hipError_t e = per_device(
+      cache, [&](int dev, int* v) { return resident_blocks(layer_norm_kernel<128>, 256, dev, v); }, &grid_cap);
+  if (e != hipSuccess) return e;
   const int rows_per_block = 4 * 4 * (64 / (C / 8));
   const long blocks = (rows + rows_per_block - 1) / rows_per_block;
   const int grid = (int)(blocks < grid_cap ? blocks : grid_cap);

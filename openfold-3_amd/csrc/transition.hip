@@ -32,6 +32,7 @@
 
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -378,17 +379,17 @@ template <int C>
 hipError_t launch(const TransitionArgs& a, hipStream_t stream) {
   auto kern = transition_kernel<C>;
   constexpr int smem = (kStagesW * 2 * 32 * (C / 8) + kStagesO * C * 4 + kWaves * 32 * (C / 8)) * 16;
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) return e;
-    cus = n;
-  }
+  static int cache[kMaxDevices];
+  int cus = 0;
+  hipError_t e = per_device(
+      cache,
+      [&](int dev, int* v) {
+        hipError_t s = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        return s != hipSuccess ? s : cu_count(dev, v);
+      },
+      &cus);
+  if (e != hipSuccess) return e;
   if ((uint64_t)(a.N - 1) * (uint64_t)a.x_view.stride_k * 2 + 2 * C > 0xffffffffull ||
       (a.mask && (uint64_t)(a.N - 1) * (uint64_t)a.mask_view.stride_k * 4 + 4 > 0xffffffffull))
     return hipErrorInvalidValue;

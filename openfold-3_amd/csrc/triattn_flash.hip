@@ -32,6 +32,7 @@
 //    keys exactly as the reference's does (-1e9 absorbs the logits in fp32).
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -337,13 +338,17 @@ constexpr int lds_bytes() {
 template <int D>
 hipError_t launch(const TriattnFlashArgs& a, hipStream_t stream) {
   auto kern = triattn_flash_kernel<D>;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<D>());
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static int cache[kMaxDevices];
+  int configured = 0;
+  hipError_t e = per_device(
+      cache,
+      [&](int, int* v) {
+        *v = 1;
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   lds_bytes<D>());
+      },
+      &configured);
+  if (e != hipSuccess) return e;
   const int n_qc = (a.N + 32 * kRQ - 1) / (32 * kRQ), n_rg = (a.N + kRows - 1) / kRows;
   const long total = (long)n_qc * n_rg * a.B * a.H;
   const int per_xcd = (int)((total + 7) / 8);

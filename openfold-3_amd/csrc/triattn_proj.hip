@@ -14,6 +14,7 @@
 // double-buffered LDS tile (one barrier per tile).
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -241,17 +242,10 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
 template <int C, int D>
 hipError_t launch(const TriattnProjArgs& a, hipStream_t stream) {
   auto kern = triattn_proj_kernel<C, D>;
-  static int grid_cap = 0;
-  if (grid_cap == 0) {
-    int dev = 0, cus = 0, per_cu = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 512, 0);
-    if (e != hipSuccess) return e;
-    grid_cap = cus * (per_cu > 0 ? per_cu : 1);
-  }
+  static int cache[kMaxDevices];
+  int grid_cap = 0;
+  hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 512, dev, v); }, &grid_cap);
+  if (e != hipSuccess) return e;
   const int tiles_per_row = a.Jp / 128;
   const long total = (long)a.B * a.N * tiles_per_row;
   const int grid = (int)(total < grid_cap ? total : grid_cap);

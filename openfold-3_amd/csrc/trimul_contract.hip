@@ -33,6 +33,7 @@
 // lane chooses its *global* chunk as chunk' ^ key(row).
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -308,18 +309,17 @@ hipError_t launch_contract(const bf16_t* a, const bf16_t* b, bf16_t* x, int plan
   constexpr int BM = 256;
   auto kern = contract_kernel<BN, kNS>;
   const size_t smem = ((size_t)kNS * (BM + BN) * 4 + 4 * 512) * sizeof(u32x4_t);  // ring + epilogue staging
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return e;
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem);
-    if (e != hipSuccess) return e;
-    cus = n;
-  }
+  static int cache[kMaxDevices];
+  int cus = 0;
+  hipError_t e = per_device(
+      cache,
+      [&](int dev, int* v) {
+        hipError_t s = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        return s != hipSuccess ? s : cu_count(dev, v);
+      },
+      &cus);
+  if (e != hipSuccess) return e;
   const int tiles_m = (Np + BM - 1) / BM, tiles_n = (Np + BN - 1) / BN;
   const int total = planes * tiles_m * tiles_n;
   const int tiles_per_xcd = (total + 7) / 8;

@@ -17,6 +17,7 @@
 // layout these are 256 contiguous bytes per channel, so 32 lanes write whole 128-byte lines.
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -203,17 +204,10 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
 template <int C, int CH>
 hipError_t launch(const TrimulProjArgs& a, hipStream_t stream) {
   auto kern = trimul_proj_kernel<C, CH>;
-  static int grid_cap = 0;
-  if (grid_cap == 0) {
-    int dev = 0, cus = 0, per_cu = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return e;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 512, 0);
-    if (e != hipSuccess) return e;
-    grid_cap = cus * (per_cu > 0 ? per_cu : 1);
-  }
+  static int cache[kMaxDevices];
+  int grid_cap = 0;
+  hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 512, dev, v); }, &grid_cap);
+  if (e != hipSuccess) return e;
   const int panels = a.Np / 32;
   const long total = (long)a.B * ((a.N + 3) / 4) * panels;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
