@@ -19,7 +19,8 @@
 //     The first padding channel (index D) carries the key mask: q gets 1 there and k gets
 //     inf * (mask[key] - 1) * log2(e), or -inf for the rows between N and Np, so the q.k
 //     product itself adds the mask bias and gives padded keys a weight of exactly zero.
-//  2. single_attn: one wave per (batch, head, 32 queries), flash style over 32-key tiles:
+//  2. single_attn: one work-group per (batch, head, 32 queries), its four waves splitting the key
+//     tiles and merging their partial softmaxes through LDS at the end; flash style over 32-key tiles:
 //     S^T = K Q^T with the accumulator initialised to pair bias * log2(e), the next tile's
 //     operands requested before the current tile's arithmetic, running
 //     maximum and sum in fp32, O^T = V^T P^T with P^T taken from the S^T registers; the result
@@ -116,13 +117,18 @@ __global__ __launch_bounds__(256) void single_proj_kernel(SingleAttnArgs p) {
 }
 
 // ---- 2. attention core -------------------------------------------------------------------
-__global__ __launch_bounds__(256) void single_attn_kernel(SingleAttnArgs p, int q_tiles) {
+constexpr int kSplit = 4;  // waves sharing one (batch, head, 32 queries)
+
+__global__ __launch_bounds__(64 * kSplit) void single_attn_kernel(SingleAttnArgs p, int q_tiles) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
   const int N = p.N, Np = p.Np, H = p.H, D = p.D;
-  const int qt = blockIdx.x * 4 + wave;
-  if (qt >= q_tiles) return;  // whole wave; the kernel has no barrier
+  // the kSplit waves of a work-group share one (batch, head, 32 queries) and split its key tiles
+  // (wave w takes tiles w, w+kSplit, ...): a single wave walking all tiles is bound by the latency of
+  // its own MFMA -> softmax -> MFMA chain, and the problem offers few waves otherwise
+  __shared__ float merge[kSplit][18][64];
+  const int qt = blockIdx.x;
   const int h = blockIdx.y, b = blockIdx.z;
   const int q0 = qt * 32;
   int qrow = q0 + l32;
@@ -158,12 +164,12 @@ __global__ __launch_bounds__(256) void single_attn_kernel(SingleAttnArgs p, int 
   f32x16_t oacc = zero16();
   const int nkt = (N + 31) / 32;
   u32x4_t kn[2], vn[2], bn[2];
-  load_tile(0, kn, vn, bn);
-  for (int kt = 0; kt < nkt; ++kt) {
+  if (wave < nkt) load_tile(wave, kn, vn, bn);
+  for (int kt = wave; kt < nkt; kt += kSplit) {
     u32x4_t kc[2], vc[2], braw[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) kc[s] = kn[s], vc[s] = vn[s], braw[s] = bn[s];
-    if (kt + 1 < nkt) load_tile(kt + 1, kn, vn, bn);  // in flight under this tile's arithmetic
+    if (kt + kSplit < nkt) load_tile(kt + kSplit, kn, vn, bn);  // in flight under this tile's arithmetic
 
     f32x16_t s;
 #pragma unroll
@@ -196,8 +202,29 @@ __global__ __launch_bounds__(256) void single_attn_kernel(SingleAttnArgs p, int 
     oacc = mfma_32x32x16(vc[1], pop[1], oacc);
   }
 
+  // ---- merge the partial softmaxes: common maximum, rescaled sums and accumulators
+  merge[wave][16][lane] = m_run;  // -inf for a wave without tiles
+  merge[wave][17][lane] = l_run + xhalf(l_run);
+#pragma unroll
+  for (int v = 0; v < 16; ++v) merge[wave][v][lane] = oacc[v];
+  __syncthreads();
+  if (wave != 0) return;
+  float m_tot = merge[0][16][lane];  // wave 0 always has tile 0: finite
+#pragma unroll
+  for (int w = 1; w < kSplit; ++w) m_tot = fmaxf(m_tot, merge[w][16][lane]);
+  float l_tot = 0.f;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) oacc[v] = 0.f;
+#pragma unroll
+  for (int w = 0; w < kSplit; ++w) {
+    const float sc = fast_exp2(merge[w][16][lane] - m_tot);  // 0 for a wave without tiles
+    l_tot += merge[w][17][lane] * sc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) oacc[v] += merge[w][v][lane] * sc;
+  }
+
   // lane (query l32, half lh) owns head channels 16*lh + v
-  const float inv = fast_rcp(l_run + xhalf(l_run));
+  const float inv = fast_rcp(l_tot);
   if (q_valid && 16 * lh < D) {
     const size_t off = ((size_t)b * N + qrow) * (H * D) + h * D + 16 * lh;
     u32x4_t graw[2];
@@ -265,7 +292,7 @@ hipError_t single_attn_launch(const SingleAttnArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL(single_proj_kernel, dim3(row_blocks, a.H, a.B), dim3(256), 0, stream, a);  // one tile per wave
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(single_attn_kernel, dim3((row_blocks + 3) / 4, a.H, a.B), dim3(256), 0, stream, a, row_blocks);
+  hipLaunchKernelGGL(single_attn_kernel, dim3(row_blocks, a.H, a.B), dim3(64 * kSplit), 0, stream, a, row_blocks);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(single_out_kernel, dim3(row_blocks, 3, a.B), dim3(256), 0, stream, a);
