@@ -18,53 +18,67 @@ __device__ __forceinline__ float xhalf(float v) { return __shfl_xor(v, 32, 64); 
 // a row is 768 bytes = 3 windows of 256, so without the key they would all hit the same one)
 __device__ __forceinline__ int act_slot(int pos, int chunk) { return pos * kChunks + ((chunk & ~15) | ((chunk ^ pos) & 15)); }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-
-// rows pos0 .. pos0+31 of src (kK channels per row, rows row_stride elements apart) into the LDS tile; with LN, normalised (statistics in
-// fp32, result rounded to bf16 as the reference's LayerNorm output).  Wave w handles 8 rows, lanes
-// 0..47 one chunk each.  Rows past n_rows repeat the last one (never stored by the callers).
+// rows pos0 .. pos0+31 of src (kK channels per row, rows row_stride elements apart) into the LDS
+// tile; with LN, normalised (statistics in fp32, result rounded to bf16 as the reference's
+// LayerNorm output).  Wave w handles rows 8w .. 8w+7, four at a time: 16 lanes per row, three
+// 16-byte chunks per lane, row sums by DPP lane permutations (no LDS traffic).  Rows past n_rows
+// repeat the last one (never stored by the callers).
 template <bool LN>
 __device__ __forceinline__ void fill_tile(u32x4_t* act, const bf16_t* __restrict__ src, long row_stride, long pos0, long n_rows,
                                           const bf16_t* __restrict__ ln_w, const bf16_t* __restrict__ ln_b, int wave,
                                           int lane) {
-  const bool has = lane < kChunks;
-  float lw[8], lb[8];
-  if (LN && has) {
-    load_affine8(ln_w, lane, lw);
-    load_affine8(ln_b, lane, lb);
+  static_assert(kChunks == 48, "three chunks per lane, 16 lanes per row");
+  const int g = lane >> 4, li = lane & 15;
+  u32x4_t wpk[3], bpk[3];
+  if (LN) {
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      wpk[c] = *reinterpret_cast<const u32x4_t*>(ln_w + 8 * (li + 16 * c));
+      bpk[c] = *reinterpret_cast<const u32x4_t*>(ln_b + 8 * (li + 16 * c));
+    }
+  }
+  u32x4_t raw[2][3];
+#pragma unroll
+  for (int it = 0; it < 2; ++it) {
+    long row = pos0 + 8 * wave + 4 * it + g;
+    row = row < n_rows ? row : n_rows - 1;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) raw[it][c] = *reinterpret_cast<const u32x4_t*>(src + row * row_stride + 8 * (li + 16 * c));
   }
 #pragma unroll
-  for (int r = 0; r < 8; ++r) {
-    const int pos = 8 * wave + r;
-    long row = pos0 + pos;
-    row = row < n_rows ? row : n_rows - 1;
-    u32x4_t raw = {0u, 0u, 0u, 0u};
-    if (has) raw = *reinterpret_cast<const u32x4_t*>(src + row * row_stride + 8 * lane);
+  for (int it = 0; it < 2; ++it) {
+    const int pos = 8 * wave + 4 * it + g;
     if (LN) {
-      float x[8];
-      unpack8(raw, x);
+      float x[3][8];
       float s = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) s += x[i];
-      const float mean = wave_sum(s) * (1.f / kK);
+      for (int c = 0; c < 3; ++c) {
+        unpack8(raw[it][c], x[c]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += x[c][i];
+      }
+      const float mean = group_sum<16>(s) * (1.f / kK);
       float q = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        x[i] = has ? x[i] - mean : 0.f;
-        q += x[i] * x[i];
-      }
-      const float rstd = __builtin_amdgcn_rsqf(wave_sum(q) * (1.f / kK) + kLnEps);
-      if (has) {
+      for (int c = 0; c < 3; ++c)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = x[i] * rstd * lw[i] + lb[i];
-        raw = pack8(x);
+        for (int i = 0; i < 8; ++i) {
+          x[c][i] -= mean;
+          q += x[c][i] * x[c][i];
+        }
+      const float rstd = __builtin_amdgcn_rsqf(group_sum<16>(q) * (1.f / kK) + kLnEps);
+#pragma unroll
+      for (int c = 0; c < 3; ++c) {
+        float w[8], bb[8];
+        unpack8(wpk[c], w);
+        unpack8(bpk[c], bb);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[c][i] = x[c][i] * rstd * w[i] + bb[i];
+        raw[it][c] = pack8(x[c]);
       }
     }
-    if (has) act[act_slot(pos, lane)] = raw;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) act[act_slot(pos, li + 16 * c)] = raw[it][c];
   }
 }
 
