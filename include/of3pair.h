@@ -197,7 +197,7 @@ int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* ma
 /* The same update as of3_transition_fwd for the single representation (PairFormerBlock's
  * single_transition, pairformer.py:118-122, :203-212): x, out contiguous [rows][C] (any leading
  * dimensions flattened; out may alias x), mask fp32 [rows] or null.  bf16: C = 384, HID a
- * multiple of 384, the workspace holds the hidden activations [rows][HID]; fp32: C <= 512,
+ * multiple of 384 up to 1920, the workspace holds the hidden activations [rows][HID]; fp32: C <= 512,
  * HID <= 2048, no workspace (null, 0 is accepted). */
 int64_t of3_transition_rows_workspace_bytes(int64_t rows, int64_t C, int64_t HID);
 int64_t of3_transition_rows_workspace_bytes_for(int dtype, int64_t rows, int64_t C, int64_t HID);

@@ -656,7 +656,7 @@ int of3_attn_pair_bias_fwd(const void* a, const void* pair_bias, const float* ma
 }
 
 int64_t of3_transition_rows_workspace_bytes(int64_t rows, int64_t C, int64_t HID) {
-  if (rows < 1 || rows > (1ll << 31) || C != 384 || HID < C || (HID % C) != 0 || HID > (1 << 20)) return OF3_EINVAL;
+  if (rows < 1 || rows > (1ll << 31) || C != 384 || HID < C || (HID % C) != 0 || HID > 5 * C) return OF3_EINVAL;
   return align256(rows * HID * 2);
 }
 

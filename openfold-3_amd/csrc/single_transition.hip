@@ -5,10 +5,12 @@
 // built from the row tiles of the single-representation attention.
 //  1. hidden: a work-group normalises 32 rows into the LDS tile; each wave computes one tile of 32
 //     hidden channels for both products and writes silu(a) * b as bf16 into h [rows][HID].
-//  2. out: a wave owns one tile of 32 output channels and walks the hidden dimension in slices
-//     of 384 (the work-group reloads the LDS tile per slice), then applies mask and residual.
+//  2. out: a work-group owns 32 rows x 32 output channels, holds the rows' hidden activations in
+//     LDS (one tile per slice of 384) and lets its four waves take different slices; the partial
+//     tiles are added through LDS, then mask and residual.
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 #include "of3_rowtile.h"
 
 namespace of3 {
@@ -48,21 +50,34 @@ __global__ __launch_bounds__(256) void row_transition_hidden_kernel(RowTransitio
   }
 }
 
+// One work-group per (32 rows, 32 output channels); its waves split the hidden dimension in
+// slices of 384 (wave w takes slices w, w+4, ...) and add their partial tiles through LDS.  Every
+// slice of the rows' hidden activations sits in its own LDS tile, filled by all waves together.
 __global__ __launch_bounds__(256) void row_transition_out_kernel(RowTransitionArgs p) {
-  __shared__ u32x4_t act[32 * kChunks];
+  extern __shared__ u32x4_t dyn[];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
   const long pos0 = (long)blockIdx.x * 32;
-  const int tile = blockIdx.y * 4 + wave;  // 32 output channels; gridDim.y * 4 = kK / 32
+  const int tile = blockIdx.y;  // 32 output channels
+  const int slices = p.HID / kK;
+  u32x4_t* act = dyn;                                                  // [slices][32 * kChunks]
+  float* merge = reinterpret_cast<float*>(dyn + slices * 32 * kChunks);  // [4][16][64]
+  for (int sl = 0; sl < slices; ++sl)
+    fill_tile<false>(act + sl * 32 * kChunks, p.h + sl * kK, p.HID, pos0, p.rows, nullptr, nullptr, wave, lane);
+  __syncthreads();
   const size_t wrow = (size_t)(32 * tile + rowperm16(l32)) * p.HID;
   f32x16_t acc = zero16();
-  for (int k0 = 0; k0 < p.HID; k0 += kK) {
-    if (k0) __syncthreads();  // everybody has read the previous slice
-    fill_tile<false>(act, p.h + k0, p.HID, pos0, p.rows, nullptr, nullptr, wave, lane);
-    __syncthreads();
-    acc = tile_product<true>(act, p.wout + wrow + k0, l32, lh, acc);
-  }
+  for (int sl = wave; sl < slices; sl += 4) acc = tile_product<true>(act + sl * 32 * kChunks, p.wout + wrow + sl * kK, l32, lh, acc);
+#pragma unroll
+  for (int v = 0; v < 16; ++v) merge[(wave * 16 + v) * 64 + lane] = acc[v];
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int w = 1; w < 4; ++w)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] += merge[(w * 16 + v) * 64 + lane];
+
   const long pos = pos0 + l32;
   if (pos < p.rows) {
     const float m = p.mask ? p.mask[pos] : 1.f;
@@ -102,7 +117,22 @@ hipError_t row_transition_launch(const RowTransitionArgs& a, hipStream_t stream)
   hipLaunchKernelGGL(row_transition_hidden_kernel, dim3((unsigned)row_blocks, hidden_groups), dim3(256), 0, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(row_transition_out_kernel, dim3((unsigned)row_blocks, kK / 32 / 4), dim3(256), 0, stream, a);
+  // LDS: one tile per hidden slice plus the merge area; at most 5 slices fit a CU's 160 KB
+  const int slices = a.HID / kK;
+  const size_t smem = (size_t)slices * 32 * kChunks * sizeof(u32x4_t) + 4 * 16 * 64 * sizeof(float);
+  if (smem > 160 * 1024) return hipErrorInvalidValue;
+  static int cache[kMaxDevices];
+  int configured = 0;
+  e = per_device(
+      cache,
+      [&](int, int* v) {
+        *v = 1;
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(row_transition_out_kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      },
+      &configured);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(row_transition_out_kernel, dim3((unsigned)row_blocks, kK / 32), dim3(256), smem, stream, a);
   return hipGetLastError();
 }
 
