@@ -6,12 +6,20 @@
 //   pair transition           transition.py:225-271, activations.py:33-61
 //   pair-bias projection      attention_pair_bias.py:151-161
 // These kernels are written for exactness and generality (any N, C, C_hidden <= 256, head
-// width <= 64), with plain fp32 FMA arithmetic, full-precision expf and no MFMA; they are the
-// precision reference of the library on the GPU, not its fast path (that is the bf16 path).
+// width <= 64) with full-precision expf; they are the precision reference of the library on the
+// GPU, not its fast path (that is the bf16 path).  The linear layers of the position-wise passes
+// run on the fp32 matrix pipe (v_mfma_f32_32x32x2_f32: exact fp32 products, fp32 sums) in
+// work-groups of 32 positions whenever the channel counts are multiples of 8 and the weights are
+// 16-byte aligned; plain FMA kernels of 8 positions serve every other shape.
 //
 // Layouts (workspace, fp32): a, b, x  [B][CH][N][N] with a[b][c][i][k] (k contracted);
 // q, k, v [B][N(i)][H][N(j)][D]; triangle bias [B][H][N][N]; o [B][N][N][H*D].
+#include <cstdint>
+#include <initializer_list>
+
+#include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -53,6 +61,83 @@ __device__ __forceinline__ float dot_row(const float* __restrict__ x, const floa
   float acc = 0.f;
   for (int k = 0; k < n; ++k) acc = fmaf(x[k], w[k], acc);
   return acc;
+}
+
+
+// ---- linear layers on the fp32 matrix pipe ---------------------------------------------------
+constexpr int kTP = 32;  // positions per work-group of the matrix-pipe kernels
+
+// row of accumulator register v in lane half lh of a 32 x 32 MFMA result (the lane's column is lane & 31)
+__device__ __forceinline__ int acc_row(int v, int lh) { return 8 * (v >> 2) + 4 * lh + (v & 3); }
+
+// LayerNorm of kTP positions (32 lanes each) into the LDS tile xn[kTP][ldx]; same arithmetic as
+// layer_norm_rows
+template <typename Src>
+__device__ __forceinline__ void layer_norm_tile(Src src, const float* __restrict__ w, const float* __restrict__ bsh,
+                                                int C, float* xn, int ldx) {
+  const int l = threadIdx.x & 31;
+  for (int pos = threadIdx.x >> 5; pos < kTP; pos += kThreads / 32) {
+    const float* row = src(pos);
+    float s = 0.f;
+    if (row)
+      for (int c = l; c < C; c += 32) s += row[c];
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, 32);
+    const float mean = s / (float)C;
+    float q = 0.f;
+    if (row)
+      for (int c = l; c < C; c += 32) {
+        const float d = row[c] - mean;
+        q += d * d;
+      }
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 32);
+    const float rstd = 1.0f / sqrtf(q / (float)C + kEps);
+    for (int c = l; c < C; c += 32) xn[pos * ldx + c] = row ? (row[c] - mean) * rstd * w[c] + bsh[c] : 0.f;
+  }
+}
+
+// NW linear layers at once for one 32 x 32 tile: the kTP positions of the LDS tile xs[kTP][ldx]
+// (K values per row, K % 8 == 0, 16-byte aligned rows) against rows o0 .. o0+31 of each W[n]
+// ([n_out][K] row-major, 16-byte aligned; rows past n_out-1 repeat the last one and are not
+// used by the caller).  The summation index is dealt so that both operands are read as float4:
+// MFMA step 4j+e pairs k = 8j+e (lanes 0-31) with k = 8j+4+e (lanes 32-63).
+// OUT_ROWS: the outputs are the MFMA rows (lane & 31 = position, register v = output
+// o0 + acc_row(v, lh)); otherwise the positions are (lane & 31 = output o0 + ..., register v =
+// position acc_row(v, lh)).  The caller picks whichever makes its stores contiguous over lanes.
+template <int NW, bool OUT_ROWS>
+__device__ __forceinline__ void linear_tiles(const float* xs, int ldx, const float* const (&W)[NW], int o0, int n_out,
+                                             int K, f32x16_t (&acc)[NW]) {
+  const int lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  int row = o0 + l32;
+  row = row < n_out ? row : n_out - 1;
+  const float4* xr = reinterpret_cast<const float4*>(xs + l32 * ldx + 4 * lh);
+  const float4* wr[NW];
+#pragma unroll
+  for (int n = 0; n < NW; ++n) {
+    wr[n] = reinterpret_cast<const float4*>(W[n] + (size_t)row * K + 4 * lh);
+    acc[n] = zero16();
+  }
+  const int steps = K / 8;
+#pragma unroll 2
+  for (int j = 0; j < steps; ++j) {
+    const float4 x = xr[2 * j];
+#pragma unroll
+    for (int n = 0; n < NW; ++n) {
+      const float4 w = wr[n][2 * j];
+      if (OUT_ROWS) {
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x2f32(w.x, x.x, acc[n], 0, 0, 0);
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x2f32(w.y, x.y, acc[n], 0, 0, 0);
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x2f32(w.z, x.z, acc[n], 0, 0, 0);
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x2f32(w.w, x.w, acc[n], 0, 0, 0);
+      } else {
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, w.x, acc[n], 0, 0, 0);
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, w.y, acc[n], 0, 0, 0);
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, w.z, acc[n], 0, 0, 0);
+        acc[n] = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, w.w, acc[n], 0, 0, 0);
+      }
+    }
+  }
 }
 
 // ---- triangle multiplication -----------------------------------------------------------------
@@ -167,6 +252,90 @@ __global__ __launch_bounds__(kThreads) void trimul_out_f32(TrimulF32 p, int grou
   }
 }
 
+
+// the two position-wise passes of the triangle multiplication on the matrix pipe: 32 positions of
+// one row per work-group
+__global__ __launch_bounds__(kThreads) void trimul_proj_mm_f32(TrimulF32 p, int groups) {
+  extern __shared__ float smem[];
+  const int N = p.N, C = p.C, CH = p.CH, ldx = C + 4;
+  float* xn = smem;              // [kTP][ldx]
+  float* msk = smem + kTP * ldx; // [kTP]
+  const int g = blockIdx.x % groups, r = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int k0 = g * kTP;
+  layer_norm_tile(
+      [&](int pos) -> const float* {
+        const int k = k0 + pos;
+        return k < N ? p.z + b * p.zv.stride_b + r * p.zv.stride_r + k * p.zv.stride_k : nullptr;
+      },
+      p.ln_in_w, p.ln_in_b, C, xn, ldx);
+  if (threadIdx.x < kTP) {
+    const int k = k0 + threadIdx.x;
+    msk[threadIdx.x] = (k < N && p.mask) ? p.mask[b * p.mv.stride_b + r * p.mv.stride_r + k * p.mv.stride_k] : 1.f;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int n_ot = (CH + 31) / 32;
+  const int k = k0 + l32;  // lanes = positions: a and b are written k-contiguous
+  const float m = msk[l32];
+  for (int t = wave; t < 2 * n_ot; t += kThreads / 64) {
+    const int pair = t / n_ot, o0 = 32 * (t - pair * n_ot);
+    const float* const W[2] = {pair ? p.w_bg : p.w_ag, pair ? p.w_bp : p.w_ap};
+    f32x16_t acc[2];
+    linear_tiles<2, true>(xn, ldx, W, o0, CH, C, acc);
+    float* dst = pair ? p.b : p.a;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int c = o0 + acc_row(v, lh);
+      // mask * sigmoid(gate) * projection, in the reference's order of multiplication
+      if (c < CH && k < N) dst[(((size_t)b * CH + c) * N + r) * N + k] = m * sigmoid_f32(acc[0][v]) * acc[1][v];
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void trimul_out_mm_f32(TrimulF32 p, int groups) {
+  extern __shared__ float smem[];
+  const int N = p.N, C = p.C, CH = p.CH, ldc = C + 4, ldh = CH + 4;
+  float* zn = smem;             // [kTP][ldc]  LayerNorm(z)
+  float* xs = zn + kTP * ldc;   // [kTP][ldh]  x gathered from the channel-major planes
+  float* xo = xs + kTP * ldh;   // [kTP][ldh]  LayerNorm(x)
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kTP;
+  layer_norm_tile(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.z + b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k : nullptr;
+      },
+      p.ln_in_w, p.ln_in_b, C, zn, ldc);
+  for (int idx = threadIdx.x; idx < kTP * CH; idx += kThreads) {
+    const int pos = idx % kTP, c = idx / kTP, j = j0 + pos;
+    xs[pos * ldh + c] = j < N ? p.x[(((size_t)b * CH + c) * N + i) * N + j] : 0.f;
+  }
+  __syncthreads();
+  layer_norm_tile([&](int pos) -> const float* { return j0 + pos < N ? xs + pos * ldh : nullptr; }, p.ln_out_w,
+                  p.ln_out_b, CH, xo, ldh);
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int n_ot = (C + 31) / 32;
+  for (int t = wave; t < n_ot; t += kThreads / 64) {
+    const int o0 = 32 * t, co = o0 + l32;  // lanes = output channels: rows of out are written contiguously
+    const float* const Wz[1] = {p.w_z};
+    const float* const Wg[1] = {p.w_g};
+    f32x16_t lin[1], gate[1];
+    linear_tiles<1, false>(xo, ldh, Wz, o0, C, CH, lin);
+    linear_tiles<1, false>(zn, ldc, Wg, o0, C, C, gate);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int j = j0 + acc_row(v, lh);
+      if (co < C && j < N) {
+        float res = lin[0][v] * sigmoid_f32(gate[0][v]);
+        const size_t o = b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k + co;
+        if (p.add_residual) res = p.z[o] + res;
+        p.out[o] = res;
+      }
+    }
+  }
+}
+
 // ---- triangle attention ----------------------------------------------------------------------
 struct TriattnF32 {
   const float *x, *mask;
@@ -203,6 +372,100 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_f32(TriattnF32 p, int g
     } else {
       const int h = ch - 3 * HD;
       p.tb[(((size_t)b * H + h) * N + i) * N + j] = dot_row(xn[pos], p.w_b + h * C, C);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void triattn_proj_mm_f32(TriattnF32 p, int groups) {
+  extern __shared__ float smem[];
+  const int N = p.N, C = p.C, H = p.H, D = p.D, HD = H * D, ldx = C + 4;
+  float* xn = smem;  // [kTP][ldx]
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kTP;
+  layer_norm_tile(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+      },
+      p.ln_w, p.ln_b, C, xn, ldx);
+  __syncthreads();
+  const float scale = 1.0f / sqrtf((float)D);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int n_ot = (HD + 31) / 32, n_bt = (H + 31) / 32;
+  for (int t = wave; t < n_ot + n_bt; t += kThreads / 64) {
+    if (t < n_ot) {
+      // q, k, v: lanes = head channels (d-contiguous stores)
+      const int o0 = 32 * t, hd = o0 + l32, h = hd / D, d = hd - h * D;
+      const float* const W[3] = {p.w_q, p.w_k, p.w_v};
+      f32x16_t acc[3];
+      linear_tiles<3, false>(xn, ldx, W, o0, HD, C, acc);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int j = j0 + acc_row(v, lh);
+        if (hd < HD && j < N) {
+          const size_t o = ((((size_t)b * N + i) * H + h) * N + j) * D + d;
+          p.q[o] = acc[0][v] * scale;  // q / sqrt(c) after the projection (attention.py:283-284)
+          p.k[o] = acc[1][v];
+          p.v[o] = acc[2][v];
+        }
+      }
+    } else {
+      // triangle bias: lanes = positions (j-contiguous stores)
+      const int o0 = 32 * (t - n_ot), j = j0 + l32;
+      const float* const W[1] = {p.w_b};
+      f32x16_t acc[1];
+      linear_tiles<1, true>(xn, ldx, W, o0, H, C, acc);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int h = o0 + acc_row(v, lh);
+        if (h < H && j < N) p.tb[(((size_t)b * H + h) * N + i) * N + j] = acc[0][v];
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int groups) {
+  extern __shared__ float smem[];
+  const int N = p.N, C = p.C, HD = p.H * p.D, ldx = C + 4, ldh = HD + 4;
+  float* xn = smem;             // [kTP][ldx]
+  float* og = xn + kTP * ldx;   // [kTP][ldh]  gated attention output
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kTP;
+  layer_norm_tile(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+      },
+      p.ln_w, p.ln_b, C, xn, ldx);
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  for (int t = wave; t < (HD + 31) / 32; t += kThreads / 64) {
+    const int o0 = 32 * t, hd = o0 + l32;
+    const float* const W[1] = {p.w_g};
+    f32x16_t gate[1];
+    linear_tiles<1, false>(xn, ldx, W, o0, HD, C, gate);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int pos = acc_row(v, lh), j = j0 + pos;
+      if (hd < HD)
+        og[pos * ldh + hd] = j < N ? p.o[(((size_t)b * N + i) * N + j) * HD + hd] * sigmoid_f32(gate[0][v]) : 0.f;
+    }
+  }
+  __syncthreads();
+  for (int t = wave; t < (C + 31) / 32; t += kThreads / 64) {
+    const int o0 = 32 * t, co = o0 + l32;
+    const float* const W[1] = {p.w_o};
+    f32x16_t acc[1];
+    linear_tiles<1, false>(og, ldh, W, o0, C, HD, acc);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int j = j0 + acc_row(v, lh);
+      if (co < C && j < N) {
+        float res = acc[0][v];
+        const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
+        if (p.add_residual) res = p.x[o] + res;
+        p.out[o] = res;
+      }
     }
   }
 }
@@ -449,6 +712,32 @@ __global__ __launch_bounds__(kThreads) void layer_norm_f32(const float* __restri
   }
 }
 
+
+// ---- host side of the matrix-pipe kernels
+size_t tile_bytes(int K) { return (size_t)kTP * (K + 4) * sizeof(float); }  // one LDS tile [kTP][K + 4]
+
+bool aligned16(std::initializer_list<const void*> ptrs) {
+  for (const void* q : ptrs)
+    if (reinterpret_cast<uintptr_t>(q) % 16 != 0) return false;
+  return true;
+}
+
+// the largest tiles (three of 256 channels) exceed the default dynamic LDS limit: raised once per
+// device and kernel (slot = index of the kernel's cache)
+template <typename Kern>
+hipError_t allow_lds(Kern kern, int slot) {
+  static int cache[4][kMaxDevices];
+  int done = 0;
+  return per_device(
+      cache[slot],
+      [&](int, int* v) {
+        *v = 1;
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)(3 * tile_bytes(kMaxC)));
+      },
+      &done);
+}
+
 }  // namespace
 
 hipError_t template_tail_fwd_f32(const TemplateTailF32Args& a, hipStream_t stream) {
@@ -510,11 +799,27 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   const int groups = (a.N + kP - 1) / kP;
   const long blocks = (long)a.B * a.N * groups;
   if (a.C > kMaxC || a.CH > kMaxC || blocks > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(trimul_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  const bool mm = a.C % 8 == 0 && a.CH % 8 == 0 &&
+                  aligned16({a.w_ap, a.w_ag, a.w_bp, a.w_bg, a.w_g, a.w_z});
+  const int mgroups = (a.N + kTP - 1) / kTP;
+  const unsigned mblocks = (unsigned)((long)a.B * a.N * mgroups);
+  if (mm) {
+    hipError_t e = allow_lds(trimul_proj_mm_f32, 0);
+    if (e == hipSuccess) e = allow_lds(trimul_out_mm_f32, 1);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(trimul_proj_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + kTP * sizeof(float), stream,
+                       p, mgroups);
+  } else {
+    hipLaunchKernelGGL(trimul_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  }
   const unsigned t = (unsigned)((a.N + 63) / 64);
   hipLaunchKernelGGL(trimul_contract_f32, dim3(t, t, (unsigned)(a.B * a.CH)), dim3(kThreads), 0, stream, p.a, p.b, p.x,
                      a.N);
-  hipLaunchKernelGGL(trimul_out_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  if (mm)
+    hipLaunchKernelGGL(trimul_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + 2 * tile_bytes(a.CH), stream,
+                       p, mgroups);
+  else
+    hipLaunchKernelGGL(trimul_out_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
   return hipGetLastError();
 }
 
@@ -550,7 +855,17 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   const int qgroups = (a.N + 127) / 128;
   const long cblocks = (long)a.B * a.N * a.H * qgroups;
   if (a.C > kMaxC || a.H * a.D > kMaxC || blocks > 0x7fffffffL || cblocks > 0x7fffffffL) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(triattn_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  const bool mm = a.C % 8 == 0 && (a.H * a.D) % 8 == 0 && aligned16({a.w_q, a.w_k, a.w_v, a.w_b, a.w_g, a.w_o});
+  const int mgroups = (a.N + kTP - 1) / kTP;
+  const unsigned mblocks = (unsigned)((long)a.B * a.N * mgroups);
+  if (mm) {
+    hipError_t e = allow_lds(triattn_proj_mm_f32, 2);
+    if (e == hipSuccess) e = allow_lds(triattn_out_mm_f32, 3);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(triattn_proj_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C), stream, p, mgroups);
+  } else {
+    hipLaunchKernelGGL(triattn_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  }
   if (a.D == 32)
     hipLaunchKernelGGL(triattn_core_f32<32>, dim3((unsigned)cblocks), dim3(128), 0, stream, p, qgroups);
   else if (a.D == 16)
@@ -559,7 +874,11 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     hipLaunchKernelGGL(triattn_core_f32<64>, dim3((unsigned)cblocks), dim3(128), 0, stream, p, qgroups);
   else
     return hipErrorInvalidValue;
-  hipLaunchKernelGGL(triattn_out_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
+  if (mm)
+    hipLaunchKernelGGL(triattn_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + tile_bytes(a.H * a.D), stream,
+                       p, mgroups);
+  else
+    hipLaunchKernelGGL(triattn_out_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
   return hipGetLastError();
 }
 

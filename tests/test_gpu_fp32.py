@@ -28,7 +28,8 @@ def _load(module, params):
 
 
 @pytest.mark.parametrize("outgoing", [True, False])
-@pytest.mark.parametrize("c,ch,n,batch,masked", [(128, 128, 64, (1,), False), (64, 64, 45, (2,), True), (96, 40, 33, (), True)])
+@pytest.mark.parametrize("c,ch,n,batch,masked", [(128, 128, 64, (1,), False), (64, 64, 45, (2,), True), (96, 40, 33, (), True),
+                                                  (36, 20, 19, (), True)])  # channel counts off the multiples of 8: the plain FMA kernels
 def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
     lib()
     gen = torch.Generator().manual_seed(300 + n)
@@ -44,7 +45,7 @@ def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
 
 @pytest.mark.parametrize("starting", [True, False])
 @pytest.mark.parametrize("c,d,heads,n,batch,masked", [(128, 32, 4, 64, (1,), False), (64, 16, 4, 45, (2,), True),
-                                                     (48, 64, 2, 37, (), True)])
+                                                     (48, 64, 2, 37, (), True), (36, 16, 3, 21, (), True)])
 def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
     lib()
     gen = torch.Generator().manual_seed(400 + n)
