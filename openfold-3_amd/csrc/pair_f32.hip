@@ -470,37 +470,50 @@ __global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int
   }
 }
 
-// one thread per query of one (b, i, h); keys in chunks of 32 through LDS, and with them the
-// [128 queries x 32 keys] slice of the triangle bias (loaded row-wise, 128 contiguous bytes per
-// query, instead of one cache line per thread and key); online softmax
+// Attention core on the fp32 matrix pipe.  Work-group = 4 waves = 128 queries of one (b, i, h), a
+// wave owns 32 of them; keys in chunks of 32 through LDS, and with them the [128 queries x 32 keys]
+// slice of the triangle bias (loaded row-wise, 128 contiguous bytes per query); online softmax.
+//   S^T = K Q^T   rows = keys, columns = queries: a lane ends with 16 logits of one query
+//   O^T = V^T P^T rows = head channels; the weights go from the S^T accumulator registers straight
+//                 into the B operand: MFMA step v pairs the keys acc_row(v, 0) and acc_row(v, 1)
+// Logits in the reference's order: q.k, then the mask bias, then the triangle bias.
 template <int D>
-__global__ __launch_bounds__(128) void triattn_core_f32(TriattnF32 p, int qgroups) {
-  constexpr int KC = 32;
-  __shared__ float ks[KC][D], vs[KC][D], mbs[KC];
-  __shared__ float tbs[128][KC + 1];  // +1: the threads of a wave read one column
+__global__ __launch_bounds__(kThreads) void triattn_core_f32(TriattnF32 p, int qgroups) {
+  static_assert(D % 8 == 0 && D <= 64, "head widths 16, 32, 64");
+  constexpr int KC = 32, LD = D + 4;  // padded rows: the 16 lanes of a float4 read phase cover all banks
+  constexpr int OB = (D + 31) / 32;   // 32-channel blocks of the output
+  static_assert(kThreads == 256, "four waves of 32 queries");
+  __shared__ __align__(16) float ks[KC * LD];
+  __shared__ float vs[KC * LD], mbs[KC];
+  __shared__ float tbs[128][KC + 1];
   const int N = p.N, H = p.H;
   const int qg = blockIdx.x % qgroups, h = (blockIdx.x / qgroups) % H, i = (blockIdx.x / (qgroups * H)) % N,
             b = blockIdx.x / (qgroups * H * N);
-  const int qi = qg * 128 + threadIdx.x;
+  const int lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int qloc = 32 * (threadIdx.x >> 6) + l32;  // this lane's query among the work-group's 128
+  const int qi = qg * 128 + qloc;
   const bool active = qi < N;
   const size_t bih = (((size_t)b * N + i) * H + h) * N;
-  float qv[D], ov[D];
+  // B operands of S^T: MFMA step 4j+e pairs d = 8j+e (lanes 0-31) with d = 8j+4+e (lanes 32-63)
+  float qv[D / 8][4];
 #pragma unroll
-  for (int d = 0; d < D; ++d) {
-    qv[d] = active ? p.q[(bih + qi) * D + d] : 0.f;
-    ov[d] = 0.f;
-  }
+  for (int j = 0; j < D / 8; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) qv[j][e] = active ? p.q[(bih + qi) * D + 8 * j + 4 * lh + e] : 0.f;
+  f32x16_t oacc[OB];
+#pragma unroll
+  for (int ob = 0; ob < OB; ++ob) oacc[ob] = zero16();
   const float* tbq = p.tb + (((size_t)b * H + h) * N + (size_t)qg * 128) * N;  // row of query qg*128
   float m = -__builtin_inff(), l = 0.f;
   for (int k0 = 0; k0 < N; k0 += KC) {
     __syncthreads();
-    for (int e = threadIdx.x; e < KC * D; e += 128) {
+    for (int e = threadIdx.x; e < KC * D; e += kThreads) {
       const int kk = e / D, d = e % D;
       const bool in = k0 + kk < N;
-      ks[kk][d] = in ? p.k[(bih + k0 + kk) * D + d] : 0.f;
-      vs[kk][d] = in ? p.v[(bih + k0 + kk) * D + d] : 0.f;
+      ks[kk * LD + d] = in ? p.k[(bih + k0 + kk) * D + d] : 0.f;
+      vs[kk * LD + d] = in ? p.v[(bih + k0 + kk) * D + d] : 0.f;
     }
-    for (int e = threadIdx.x; e < 128 * KC; e += 128) {
+    for (int e = threadIdx.x; e < 128 * KC; e += kThreads) {
       const int r = e / KC, c = e % KC;
       tbs[r][c] = (qg * 128 + r < N && k0 + c < N) ? tbq[(size_t)r * N + k0 + c] : 0.f;
     }
@@ -512,38 +525,59 @@ __global__ __launch_bounds__(128) void triattn_core_f32(TriattnF32 p, int qgroup
     }
     __syncthreads();
     const int kn = N - k0 < KC ? N - k0 : KC;
-    float s[KC];
+    f32x16_t s = zero16();
+#pragma unroll
+    for (int j = 0; j < D / 8; ++j) {
+      const float4 kk = *reinterpret_cast<const float4*>(ks + l32 * LD + 8 * j + 4 * lh);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.x, qv[j][0], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.y, qv[j][1], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.z, qv[j][2], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.w, qv[j][3], s, 0, 0, 0);
+    }
     float cmax = -__builtin_inff();
 #pragma unroll
-    for (int kk = 0; kk < KC; ++kk) {
-      float acc = 0.f;
-#pragma unroll
-      for (int d = 0; d < D; ++d) acc = fmaf(qv[d], ks[kk][d], acc);
-      // logits in the reference's order: q.k, then the mask bias, then the triangle bias
-      acc = acc + mbs[kk];
-      acc = acc + tbs[threadIdx.x][kk];
-      s[kk] = kk < kn ? acc : -__builtin_inff();
-      cmax = fmaxf(cmax, s[kk]);
+    for (int v = 0; v < 16; ++v) {
+      const int kk = acc_row(v, lh);
+      float a = s[v] + mbs[kk];
+      a = a + tbs[qloc][kk];
+      a = kk < kn ? a : -__builtin_inff();
+      s[v] = a;
+      cmax = fmaxf(cmax, a);
     }
+    cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));  // the other half of the query's keys
     const float m_new = fmaxf(m, cmax);
     const float alpha = expf(m - m_new);
     l *= alpha;
 #pragma unroll
-    for (int d = 0; d < D; ++d) ov[d] *= alpha;
+    for (int ob = 0; ob < OB; ++ob)
 #pragma unroll
-    for (int kk = 0; kk < KC; ++kk) {
-      const float pw = expf(s[kk] - m_new);
+      for (int v = 0; v < 16; ++v) oacc[ob][v] *= alpha;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const float pw = expf(s[v] - m_new);
       l += pw;
+      s[v] = pw;
+    }
 #pragma unroll
-      for (int d = 0; d < D; ++d) ov[d] = fmaf(pw, vs[kk][d], ov[d]);
+    for (int ob = 0; ob < OB; ++ob) {
+      const int ch = 32 * ob + l32 < D ? 32 * ob + l32 : D - 1;  // rows past D are computed and dropped
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        oacc[ob] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[acc_row(v, lh) * LD + ch], s[v], oacc[ob], 0, 0, 0);
     }
     m = m_new;
   }
+  l += __shfl_xor(l, 32, 64);
   if (active) {
     const float inv = 1.0f / l;
     float* dst = p.o + ((((size_t)b * N + i) * N + qi) * H + h) * D;
 #pragma unroll
-    for (int d = 0; d < D; ++d) dst[d] = ov[d] * inv;
+    for (int ob = 0; ob < OB; ++ob)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ch = 32 * ob + acc_row(v, lh);
+        if (ch < D) dst[ch] = oacc[ob][v] * inv;
+      }
   }
 }
 
@@ -867,11 +901,11 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     hipLaunchKernelGGL(triattn_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
   }
   if (a.D == 32)
-    hipLaunchKernelGGL(triattn_core_f32<32>, dim3((unsigned)cblocks), dim3(128), 0, stream, p, qgroups);
+    hipLaunchKernelGGL(triattn_core_f32<32>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
   else if (a.D == 16)
-    hipLaunchKernelGGL(triattn_core_f32<16>, dim3((unsigned)cblocks), dim3(128), 0, stream, p, qgroups);
+    hipLaunchKernelGGL(triattn_core_f32<16>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
   else if (a.D == 64)
-    hipLaunchKernelGGL(triattn_core_f32<64>, dim3((unsigned)cblocks), dim3(128), 0, stream, p, qgroups);
+    hipLaunchKernelGGL(triattn_core_f32<64>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
   else
     return hipErrorInvalidValue;
   if (mm)
