@@ -653,6 +653,55 @@ __global__ __launch_bounds__(kThreads) void transition_f32(TransitionF32 p, int 
   }
 }
 
+// the same on the matrix pipe, 32 positions per work-group (hidden activations stay in LDS)
+__global__ __launch_bounds__(kThreads) void transition_mm_f32(TransitionF32 p, int groups) {
+  extern __shared__ float smem[];
+  const int N = p.N, C = p.C, HID = p.HID, ldx = C + 4, ldh = HID + 4;
+  float* xn = smem;             // [kTP][ldx]
+  float* hid = xn + kTP * ldx;  // [kTP][ldh]
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kTP;
+  layer_norm_tile(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+      },
+      p.ln_w, p.ln_b, C, xn, ldx);
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  for (int t = wave; t < (HID + 31) / 32; t += kThreads / 64) {
+    const int o0 = 32 * t, hd = o0 + l32;
+    const float* const W[2] = {p.w_a, p.w_b};
+    f32x16_t acc[2];
+    linear_tiles<2, false>(xn, ldx, W, o0, HID, C, acc);
+    if (hd < HID) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float a = acc[0][v];
+        hid[acc_row(v, lh) * ldh + hd] = (a * sigmoid_f32(a)) * acc[1][v];
+      }
+    }
+  }
+  __syncthreads();
+  for (int t = wave; t < (C + 31) / 32; t += kThreads / 64) {
+    const int o0 = 32 * t, co = o0 + l32;
+    const float* const W[1] = {p.w_out};
+    f32x16_t acc[1];
+    linear_tiles<1, false>(hid, ldh, W, o0, C, HID, acc);
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int j = j0 + acc_row(v, lh);
+      if (co < C && j < N) {
+        float res = acc[0][v];
+        if (p.mask) res *= p.mask[b * p.mv.stride_b + i * p.mv.stride_r + j * p.mv.stride_k];
+        const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
+        if (p.add_residual) res = p.x[o] + res;
+        p.out[o] = res;
+      }
+    }
+  }
+}
+
 // ---- pair-bias projection ---------------------------------------------------------------------
 struct PairBiasF32 {
   const float* z;
@@ -756,10 +805,11 @@ bool aligned16(std::initializer_list<const void*> ptrs) {
   return true;
 }
 
-// the largest tiles (three of 256 channels) exceed the default dynamic LDS limit: raised once per
-// device and kernel (slot = index of the kernel's cache)
+// the largest tiles exceed the default dynamic LDS limit: raised to max_bytes once per device and
+// kernel (slot = index of the kernel's cache)
+constexpr size_t kLdsLimit = 160 * 1024;
 template <typename Kern>
-hipError_t allow_lds(Kern kern, int slot) {
+hipError_t allow_lds(Kern kern, int slot, size_t max_bytes = 3 * (size_t)kTP * (kMaxC + 4) * sizeof(float)) {
   static int cache[4][kMaxDevices];
   int done = 0;
   return per_device(
@@ -767,7 +817,7 @@ hipError_t allow_lds(Kern kern, int slot) {
       [&](int, int* v) {
         *v = 1;
         return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)(3 * tile_bytes(kMaxC)));
+                                   (int)max_bytes);
       },
       &done);
 }
@@ -934,6 +984,16 @@ hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
   p.C = a.C;
   p.HID = a.HID;
   p.add_residual = a.add_residual;
+  const size_t mm_bytes = tile_bytes(a.C) + tile_bytes(a.HID);
+  if (a.C % 8 == 0 && a.HID % 8 == 0 && mm_bytes <= kLdsLimit && aligned16({a.w_a, a.w_b, a.w_out})) {
+    hipError_t e = allow_lds(transition_mm_f32, 0, kLdsLimit);
+    if (e != hipSuccess) return e;
+    const int mgroups = (a.N + kTP - 1) / kTP;
+    const long mblocks = (long)a.B * a.N * mgroups;
+    if (mblocks > 0x7fffffffL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(transition_mm_f32, dim3((unsigned)mblocks), dim3(kThreads), mm_bytes, stream, p, mgroups);
+    return hipGetLastError();
+  }
   const int groups = (a.N + kP - 1) / kP;
   const long blocks = (long)a.B * a.N * groups;
   hipLaunchKernelGGL(transition_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
