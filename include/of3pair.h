@@ -58,8 +58,10 @@
  * of3_transition_fwd / of3_pair_bias_fwd / of3_layer_norm_fwd / of3_template_tail_fwd /
  * of3_attn_pair_bias_fwd / of3_transition_rows_fwd only:
  * every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
- * element counts, any N, C and CH <= 256, H*D <= 256 with D in {16, 32, 64}; plain fp32
- * arithmetic in the reference's order of operations (no MFMA, not the fast path).  The
+ * element counts, any N, C and CH <= 256, H*D <= 256 with D in {16, 32, 64}; fp32
+ * arithmetic in the reference's order of operations (not the fast path; the linear layers
+ * and the attention core use the fp32 matrix instructions when the channel counts are
+ * multiples of 8 and the weights 16-byte aligned, plain FMA kernels otherwise).  The
  * stage entry points are bf16 only.
  */
 #ifndef OF3PAIR_H

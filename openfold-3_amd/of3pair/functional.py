@@ -5,8 +5,8 @@ attention.py:366-413), here with a single implementation and no dispatch.
 All functions run on the current CUDA(HIP) stream of the tensors' device, are forward-only
 and accept bf16 or fp32 pair tensors shaped [*, N, N, C] (any number of leading batch
 dimensions, a transposed view in the two N dimensions is fine and is not copied).  bf16 runs
-the MFMA kernels; fp32 (the reference's default inference precision) runs the library's plain
-fp32 kernels; parameters are converted to the tensor's dtype.
+the bf16 MFMA kernels; fp32 (the reference's default inference precision) runs the library's
+fp32 kernels (slower, the precision path); parameters are converted to the tensor's dtype.
 """
 from __future__ import annotations
 
