@@ -222,6 +222,82 @@ __global__ __launch_bounds__(kThreads) void trimul_contract_f32(const float* __r
     }
 }
 
+// the same on the fp32 matrix pipe: 128 x 128 tile, four waves of 64 x 64 (2 x 2 MFMA blocks).
+// a and b chunks of 32 k-values sit in LDS as [row][32 + 4] so that a lane's operand values for four
+// MFMA steps are one float4 (step 4j+e pairs k = 8j+e in lanes 0-31 with k = 8j+4+e in lanes 32-63);
+// i is the MFMA row side and j the column side: the lanes of a store cover 32 consecutive j.
+__global__ __launch_bounds__(kThreads) void trimul_contract_mm_f32(const float* __restrict__ a,
+                                                                  const float* __restrict__ b,
+                                                                  float* __restrict__ x, int N) {
+  constexpr int T = 128, BK = 32, LD = BK + 4;
+  __shared__ __align__(16) float as[T * LD];
+  __shared__ __align__(16) float bs[T * LD];
+  const size_t plane = (size_t)blockIdx.z * N * N;
+  const int i0 = blockIdx.y * T, j0 = blockIdx.x * T;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wi = 64 * (wave >> 1), wj = 64 * (wave & 1);
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int v = 0; v < 2; ++v) acc[u][v] = zero16();
+  // a chunk travels global -> registers while the previous one is multiplied, and registers -> LDS
+  // between two barriers; a wave's load covers two rows of 128 contiguous bytes
+  constexpr int LI = T * BK / kThreads;
+  float a_r[LI], b_r[LI];
+  const int ld_row = threadIdx.x / BK, ld_k = threadIdx.x % BK;  // + it * (kThreads / BK) rows
+  auto fetch = [&](int k0) {
+    const bool kin = k0 + ld_k < N;
+#pragma unroll
+    for (int it = 0; it < LI; ++it) {
+      const int row = ld_row + it * (kThreads / BK);
+      a_r[it] = (kin && i0 + row < N) ? a[plane + (size_t)(i0 + row) * N + k0 + ld_k] : 0.f;
+      b_r[it] = (kin && j0 + row < N) ? b[plane + (size_t)(j0 + row) * N + k0 + ld_k] : 0.f;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < N; k0 += BK) {
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < LI; ++it) {
+      const int row = ld_row + it * (kThreads / BK);
+      as[row * LD + ld_k] = a_r[it];
+      bs[row * LD + ld_k] = b_r[it];
+    }
+    __syncthreads();
+    if (k0 + BK < N) fetch(k0 + BK);
+#pragma unroll
+    for (int j = 0; j < BK / 8; ++j) {
+      float4 av[2], bv[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        av[u] = *reinterpret_cast<const float4*>(as + (wi + 32 * u + l32) * LD + 8 * j + 4 * lh);
+        bv[u] = *reinterpret_cast<const float4*>(bs + (wj + 32 * u + l32) * LD + 8 * j + 4 * lh);
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+          acc[u][v] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u].x, bv[v].x, acc[u][v], 0, 0, 0);
+          acc[u][v] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u].y, bv[v].y, acc[u][v], 0, 0, 0);
+          acc[u][v] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u].z, bv[v].z, acc[u][v], 0, 0, 0);
+          acc[u][v] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[u].w, bv[v].w, acc[u][v], 0, 0, 0);
+        }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < 2; ++u)
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+      const int j = j0 + wj + 32 * v + l32;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = i0 + wi + 32 * u + acc_row(r, lh);
+        if (i < N && j < N) x[plane + (size_t)i * N + j] = acc[u][v][r];
+      }
+    }
+}
+
 __global__ __launch_bounds__(kThreads) void trimul_out_f32(TrimulF32 p, int groups) {
   __shared__ float zn[kP][kMaxC];
   __shared__ float xs[kP][kMaxC];
@@ -478,7 +554,7 @@ __global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int
 //                 into the B operand: MFMA step v pairs the keys acc_row(v, 0) and acc_row(v, 1)
 // Logits in the reference's order: q.k, then the mask bias, then the triangle bias.
 template <int D>
-__global__ __launch_bounds__(kThreads) void triattn_core_f32(TriattnF32 p, int qgroups) {
+__global__ __launch_bounds__(kThreads, 2) void triattn_core_f32(TriattnF32 p, int qgroups) {
   static_assert(D % 8 == 0 && D <= 64, "head widths 16, 32, 64");
   constexpr int KC = 32, LD = D + 4;  // padded rows: the 16 lanes of a float4 read phase cover all banks
   constexpr int OB = (D + 31) / 32;   // 32-channel blocks of the output
@@ -505,25 +581,47 @@ __global__ __launch_bounds__(kThreads) void triattn_core_f32(TriattnF32 p, int q
   for (int ob = 0; ob < OB; ++ob) oacc[ob] = zero16();
   const float* tbq = p.tb + (((size_t)b * H + h) * N + (size_t)qg * 128) * N;  // row of query qg*128
   float m = -__builtin_inff(), l = 0.f;
-  for (int k0 = 0; k0 < N; k0 += KC) {
-    __syncthreads();
-    for (int e = threadIdx.x; e < KC * D; e += kThreads) {
-      const int kk = e / D, d = e % D;
+  // a chunk's K, V, bias slice and mask values travel global -> registers while the previous chunk
+  // is being computed, and registers -> LDS between two barriers
+  constexpr int KVI = KC * D / kThreads, TBI = 128 * KC / kThreads;
+  float k_r[KVI], v_r[KVI], tb_r[TBI], mb_r = 0.f;
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int it = 0; it < KVI; ++it) {
+      const int e = threadIdx.x + it * kThreads, kk = e / D, d = e % D;
       const bool in = k0 + kk < N;
-      ks[kk * LD + d] = in ? p.k[(bih + k0 + kk) * D + d] : 0.f;
-      vs[kk * LD + d] = in ? p.v[(bih + k0 + kk) * D + d] : 0.f;
+      k_r[it] = in ? p.k[(bih + k0 + kk) * D + d] : 0.f;
+      v_r[it] = in ? p.v[(bih + k0 + kk) * D + d] : 0.f;
     }
-    for (int e = threadIdx.x; e < 128 * KC; e += kThreads) {
-      const int r = e / KC, c = e % KC;
-      tbs[r][c] = (qg * 128 + r < N && k0 + c < N) ? tbq[(size_t)r * N + k0 + c] : 0.f;
+#pragma unroll
+    for (int it = 0; it < TBI; ++it) {
+      const int e = threadIdx.x + it * kThreads, r = e / KC, c = e % KC;
+      tb_r[it] = (qg * 128 + r < N && k0 + c < N) ? tbq[(size_t)r * N + k0 + c] : 0.f;
     }
     if (threadIdx.x < KC) {
       const int kx = k0 + threadIdx.x;
       float mv = 1.f;
       if (kx < N && p.mask) mv = p.mask[b * p.mv.stride_b + i * p.mv.stride_r + kx * p.mv.stride_k];
-      mbs[threadIdx.x] = p.inf * (mv - 1.f);
+      mb_r = p.inf * (mv - 1.f);
     }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < N; k0 += KC) {
     __syncthreads();
+#pragma unroll
+    for (int it = 0; it < KVI; ++it) {
+      const int e = threadIdx.x + it * kThreads, kk = e / D, d = e % D;
+      ks[kk * LD + d] = k_r[it];
+      vs[kk * LD + d] = v_r[it];
+    }
+#pragma unroll
+    for (int it = 0; it < TBI; ++it) {
+      const int e = threadIdx.x + it * kThreads;
+      tbs[e / KC][e % KC] = tb_r[it];
+    }
+    if (threadIdx.x < KC) mbs[threadIdx.x] = mb_r;
+    __syncthreads();
+    if (k0 + KC < N) fetch(k0 + KC);
     const int kn = N - k0 < KC ? N - k0 : KC;
     f32x16_t s = zero16();
 #pragma unroll
@@ -896,9 +994,17 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   } else {
     hipLaunchKernelGGL(trimul_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
   }
-  const unsigned t = (unsigned)((a.N + 63) / 64);
-  hipLaunchKernelGGL(trimul_contract_f32, dim3(t, t, (unsigned)(a.B * a.CH)), dim3(kThreads), 0, stream, p.a, p.b, p.x,
-                     a.N);
+  // the contraction has no shape or alignment condition of its own; the FMA kernel stays with the
+  // FMA passes so that odd shapes run one family of kernels
+  if (mm) {
+    const unsigned t = (unsigned)((a.N + 127) / 128);
+    hipLaunchKernelGGL(trimul_contract_mm_f32, dim3(t, t, (unsigned)(a.B * a.CH)), dim3(kThreads), 0, stream, p.a, p.b,
+                       p.x, a.N);
+  } else {
+    const unsigned t = (unsigned)((a.N + 63) / 64);
+    hipLaunchKernelGGL(trimul_contract_f32, dim3(t, t, (unsigned)(a.B * a.CH)), dim3(kThreads), 0, stream, p.a, p.b,
+                       p.x, a.N);
+  }
   if (mm)
     hipLaunchKernelGGL(trimul_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + 2 * tile_bytes(a.CH), stream,
                        p, mgroups);
