@@ -27,6 +27,8 @@ Besides the whole-block time the line carries
   pairformer_block_ms  wall clock of one whole PairFormerBlock (of3pair.PairFormerBlock: the pair-stack
                 block plus pair transition, pair bias, attention over s and single transition) at
                 the same N, for orientation; not part of `value`;
+  fp32_block_ms  wall clock of the same pair-stack block in fp32 (the reference's default inference
+                precision; of3pair.PairStack on fp32 tensors), for orientation; not part of `value`;
   cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path)
                 timed once on the host cores for the same workload.
 """
@@ -294,6 +296,20 @@ def main():
     torch.cuda.synchronize()
     pairformer_block_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # ---- the same pair-stack block in fp32 through the module interface, wall clock; informative
+    ps32 = of3pair.PairStack(C, CH, D, H)
+    ps32.load_state_dict(params, strict=True)
+    ps32 = ps32.to(dev).eval()
+    z32, m32 = z_host.to(dev), torch.ones(B, N, N, device=dev)
+    ps32(z32, m32)
+    torch.cuda.synchronize()
+    fp32_reps = max(1, min(5, args.steps))
+    t0 = time.perf_counter()
+    for _ in range(fp32_reps):
+        ps32(z32, m32)
+    torch.cuda.synchronize()
+    fp32_block_ms = (time.perf_counter() - t0) * 1e3 / fp32_reps
+
     # ---- CPU baseline: the oracle on the host cores, one block of the same workload
     cpu = None
     if not args.no_cpu:
@@ -313,7 +329,7 @@ def main():
         "config": {"workload": "pair-stack block (trimul out+in, tri-attn start+end, residuals), B=1, N_token=%d, "
                                "c_z=128, c_hidden_mul=128, 4 heads x 32, all-ones mask" % N},
         "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
-        "pairformer_block_ms": round(pairformer_block_ms, 4),
+        "pairformer_block_ms": round(pairformer_block_ms, 4), "fp32_block_ms": round(fp32_block_ms, 3),
     }
     print(json.dumps(line))
 
