@@ -29,7 +29,8 @@
 //    0, ...], B = [1, 0, ...]) right after the triangle bias, i.e. (tb + mb) + q.k in the
 //    fp32 accumulator: masked keys get weight exactly 0, padded keys (N not a multiple of
 //    32) carry -inf, and a fully masked row degenerates to a uniform average over all real
-//    keys exactly as the reference's does (-1e9 absorbs the logits in fp32).
+//    keys exactly as the reference's does (-1e9 absorbs the logits in fp32).  A key tile whose
+//    32 mask biases are all zero (checked wave-wide once per tile) skips that k-step.
 #include "of3_device.h"
 #include "of3_kernels.h"
 #include "of3_launch.h"
@@ -203,6 +204,8 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
   const u32x4_t one_op = {lh == 0 ? 0x3F80u : 0u, 0u, 0u, 0u};
   auto tile = [&](int buf) {
     const u32x4_t mb_op = {lh == 0 ? pack_bf16(mb_cur, 0.f) : 0u, 0u, 0u, 0u};
+    // a tile without a masked or padded key (the usual case) adds nothing: its mask k-step is skipped
+    const bool has_mb = __builtin_amdgcn_ballot_w64(mb_cur != 0.f) != 0;
     const u32x4_t* tbuf = tb_lds + buf * kTbSlots;
     const u32x4_t* kvb = kv_mine + buf * KVS;
     u32x4_t kc[KSQ], vc[2];
@@ -226,7 +229,7 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
     };
 
     f32x16_t s = bias_init(0);
-    s = mfma_32x32x16(mb_op, one_op, s);
+    if (has_mb) s = mfma_32x32x16(mb_op, one_op, s);
 #pragma unroll
     for (int ks = 0; ks < KSQ; ++ks) s = mfma_32x32x16(kc[ks], qop[0][ks], s);
 
@@ -266,7 +269,7 @@ __global__ __launch_bounds__(64 * kRows) void triattn_flash_kernel(TriattnFlashA
       for (int w = 0; w < 4; ++w) pop0[w] = expw(w);
       __builtin_amdgcn_sched_barrier(0);
       if (rq + 1 < kRQ) {
-        sn = mfma_32x32x16(mb_op, one_op, sn);
+        if (has_mb) sn = mfma_32x32x16(mb_op, one_op, sn);
         sn = mfma_32x32x16(kc[0], qop[rq + 1 < kRQ ? rq + 1 : 0][0], sn);
       }
       __builtin_amdgcn_sched_barrier(0);
