@@ -105,9 +105,12 @@ __device__ __forceinline__ void layer_norm_tile(Src src, const float* __restrict
 // OUT_ROWS: the outputs are the MFMA rows (lane & 31 = position, register v = output
 // o0 + acc_row(v, lh)); otherwise the positions are (lane & 31 = output o0 + ..., register v =
 // position acc_row(v, lh)).  The caller picks whichever makes its stores contiguous over lanes.
-template <int NW, bool OUT_ROWS>
+// ldw: row stride of W (K when the whole row is summed; larger when xs holds a slice of the inputs
+// and W points at that slice's first column); ACCUMULATE keeps the values acc came in with.
+template <int NW, bool OUT_ROWS, bool ACCUMULATE = false>
 __device__ __forceinline__ void linear_tiles(const float* xs, int ldx, const float* const (&W)[NW], int o0, int n_out,
-                                             int K, f32x16_t (&acc)[NW]) {
+                                             int K, f32x16_t (&acc)[NW], int ldw = 0) {
+  if (ldw == 0) ldw = K;
   const int lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
   int row = o0 + l32;
   row = row < n_out ? row : n_out - 1;
@@ -115,8 +118,8 @@ __device__ __forceinline__ void linear_tiles(const float* xs, int ldx, const flo
   const float4* wr[NW];
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
-    wr[n] = reinterpret_cast<const float4*>(W[n] + (size_t)row * K + 4 * lh);
-    acc[n] = zero16();
+    wr[n] = reinterpret_cast<const float4*>(W[n] + (size_t)row * ldw + 4 * lh);
+    if (!ACCUMULATE) acc[n] = zero16();
   }
   const int steps = K / 8;
 #pragma unroll 2
@@ -751,10 +754,12 @@ __global__ __launch_bounds__(kThreads) void transition_f32(TransitionF32 p, int 
   }
 }
 
-// the same on the matrix pipe, 32 positions per work-group (hidden activations stay in LDS)
-__global__ __launch_bounds__(kThreads) void transition_mm_f32(TransitionF32 p, int groups) {
+// the same on the matrix pipe, 32 positions per work-group.  The hidden dimension is walked in
+// slices of `hchunk` (a multiple of 32): a slice of the hidden activations is computed into LDS and
+// at once folded into the output accumulators, so that LDS holds one slice, not the whole hidden row
+__global__ __launch_bounds__(kThreads) void transition_mm_f32(TransitionF32 p, int groups, int hchunk) {
   extern __shared__ float smem[];
-  const int N = p.N, C = p.C, HID = p.HID, ldx = C + 4, ldh = HID + 4;
+  const int N = p.N, C = p.C, HID = p.HID, ldx = C + 4, ldh = hchunk + 4;
   float* xn = smem;             // [kTP][ldx]
   float* hid = xn + kTP * ldx;  // [kTP][ldh]
   const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
@@ -765,32 +770,48 @@ __global__ __launch_bounds__(kThreads) void transition_mm_f32(TransitionF32 p, i
         return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
       },
       p.ln_w, p.ln_b, C, xn, ldx);
-  __syncthreads();
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
-  for (int t = wave; t < (HID + 31) / 32; t += kThreads / 64) {
-    const int o0 = 32 * t, hd = o0 + l32;
-    const float* const W[2] = {p.w_a, p.w_b};
-    f32x16_t acc[2];
-    linear_tiles<2, false>(xn, ldx, W, o0, HID, C, acc);
-    if (hd < HID) {
+  // output tiles of this wave (C <= 256: at most two), accumulated over the hidden slices
+  constexpr int kMaxOT = (kMaxC / 32 + kThreads / 64 - 1) / (kThreads / 64);
+  f32x16_t out_acc[kMaxOT][1];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float a = acc[0][v];
-        hid[acc_row(v, lh) * ldh + hd] = (a * sigmoid_f32(a)) * acc[1][v];
+  for (int u = 0; u < kMaxOT; ++u) out_acc[u][0] = zero16();
+  const int n_ot = (C + 31) / 32;
+  for (int h0 = 0; h0 < HID; h0 += hchunk) {
+    const int hn = HID - h0 < hchunk ? HID - h0 : hchunk;  // a multiple of 8
+    __syncthreads();  // xn is complete (first slice); nobody reads the previous slice any more
+    for (int t = wave; t < (hn + 31) / 32; t += kThreads / 64) {
+      const int o0 = 32 * t, hd = o0 + l32;
+      const float* const W[2] = {p.w_a + (size_t)h0 * C, p.w_b + (size_t)h0 * C};
+      f32x16_t acc[2];
+      linear_tiles<2, false>(xn, ldx, W, o0, hn, C, acc);
+      if (hd < hn) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float a = acc[0][v];
+          hid[acc_row(v, lh) * ldh + hd] = (a * sigmoid_f32(a)) * acc[1][v];
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < kMaxOT; ++u) {
+      const int t = wave + u * (kThreads / 64);
+      if (t < n_ot) {
+        const float* const W[1] = {p.w_out + h0};
+        linear_tiles<1, false, true>(hid, ldh, W, 32 * t, C, hn, out_acc[u], HID);
       }
     }
   }
-  __syncthreads();
-  for (int t = wave; t < (C + 31) / 32; t += kThreads / 64) {
-    const int o0 = 32 * t, co = o0 + l32;
-    const float* const W[1] = {p.w_out};
-    f32x16_t acc[1];
-    linear_tiles<1, false>(hid, ldh, W, o0, C, HID, acc);
+#pragma unroll
+  for (int u = 0; u < kMaxOT; ++u) {
+    const int t = wave + u * (kThreads / 64), co = 32 * t + l32;
+    if (t >= n_ot) continue;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
       const int j = j0 + acc_row(v, lh);
       if (co < C && j < N) {
-        float res = acc[0][v];
+        float res = out_acc[u][0][v];
         if (p.mask) res *= p.mask[b * p.mv.stride_b + i * p.mv.stride_r + j * p.mv.stride_k];
         const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
         if (p.add_residual) res = p.x[o] + res;
@@ -1090,14 +1111,19 @@ hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
   p.C = a.C;
   p.HID = a.HID;
   p.add_residual = a.add_residual;
-  const size_t mm_bytes = tile_bytes(a.C) + tile_bytes(a.HID);
-  if (a.C % 8 == 0 && a.HID % 8 == 0 && mm_bytes <= kLdsLimit && aligned16({a.w_a, a.w_b, a.w_out})) {
+  if (a.C % 8 == 0 && a.HID % 8 == 0 && aligned16({a.w_a, a.w_b, a.w_out})) {
+    // hidden slice: as wide as keeps three work-groups on a CU (about 52 KB of LDS each)
+    int hchunk = (int)((52 * 1024 - tile_bytes(a.C)) / (kTP * sizeof(float))) - 4;
+    hchunk = hchunk / 32 * 32;
+    if (hchunk < 32) hchunk = 32;
+    if (hchunk > a.HID) hchunk = (a.HID + 31) / 32 * 32;
+    const size_t mm_bytes = tile_bytes(a.C) + tile_bytes(hchunk);
     hipError_t e = allow_lds(transition_mm_f32, 0, kLdsLimit);
     if (e != hipSuccess) return e;
     const int mgroups = (a.N + kTP - 1) / kTP;
     const long mblocks = (long)a.B * a.N * mgroups;
     if (mblocks > 0x7fffffffL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(transition_mm_f32, dim3((unsigned)mblocks), dim3(kThreads), mm_bytes, stream, p, mgroups);
+    hipLaunchKernelGGL(transition_mm_f32, dim3((unsigned)mblocks), dim3(kThreads), mm_bytes, stream, p, mgroups, hchunk);
     return hipGetLastError();
   }
   const int groups = (a.N + kP - 1) / kP;
