@@ -93,8 +93,10 @@ struct TransitionArgs {
   const bf16_t *w_a, *w_b;    // [HID][C]  (SwiGLU linear_a: the gated half, linear_b)
   const bf16_t *w_out;        // [C][HID]
   bf16_t* out;                // x_view addressing
-  int B, N, HID;
+  int B, N, HID;              // N positions per row
   int add_residual;
+  int R;                      // rows per batch element (N for a pair tensor taken row by row; 1 when the
+                              // caller hands a contiguous tensor over as one row of N*N positions)
 };
 hipError_t transition_launch(const TransitionArgs& args, int C, hipStream_t stream);
 

@@ -434,10 +434,19 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
   if (dtype != OF3_DTYPE_BF16) return OF3_EINVAL;
   if (!(C == 128 || C == 64) || HID < 128 || HID % 32 != 0 || HID > (1 << 16) || !strides_ok(x_strides))
     return OF3_EINVAL;
-  // positions along a row are addressed with 32-bit byte offsets
-  if ((N - 1) * x_strides[2] * 2 + 2 * C > 0xffffffffll) return OF3_EINVAL;
-  if (mask && (N - 1) * mask_strides[2] * 4 + 4 > 0xffffffffll) return OF3_EINVAL;
-  if (B * N * ((N + 255) / 256) > 0x7fffffffll) return OF3_EINVAL;
+  // A tensor (and mask) whose rows follow one another without gaps is one row of N*N positions per
+  // batch element: the kernel's 256-position tiles then do not stop at row ends, which matters when
+  // N is not a multiple of 256.  Positions along a row are addressed with 32-bit byte offsets.
+  int64_t rows = N, row_len = N;
+  if (x_strides[1] == N * x_strides[2] && (!mask || mask_strides[1] == N * mask_strides[2]) &&
+      (N * N - 1) * x_strides[2] * 2 + 2 * C <= 0xffffffffll &&
+      (!mask || (N * N - 1) * mask_strides[2] * 4 + 4 <= 0xffffffffll)) {
+    rows = 1;
+    row_len = N * N;
+  }
+  if ((row_len - 1) * x_strides[2] * 2 + 2 * C > 0xffffffffll) return OF3_EINVAL;
+  if (mask && (row_len - 1) * mask_strides[2] * 4 + 4 > 0xffffffffll) return OF3_EINVAL;
+  if (B * rows * ((row_len + 255) / 256) > 0x7fffffffll) return OF3_EINVAL;
   for (const void* p : ptrs)
     if (!p || !aligned16(p)) return OF3_EINVAL;
   of3::TransitionArgs args;
@@ -452,7 +461,8 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
   args.w_out = bf(w_out);
   args.out = bf(out);
   args.B = (int)B;
-  args.N = (int)N;
+  args.N = (int)row_len;
+  args.R = (int)rows;
   args.HID = (int)HID;
   args.add_residual = add_residual ? 1 : 0;
   hipError_t e = of3::transition_launch(args, (int)C, static_cast<hipStream_t>(stream));

@@ -147,7 +147,7 @@ __global__ __launch_bounds__(64 * kWaves) void transition_kernel(TransitionArgs 
   for (int s = 0; s < 2; ++s) wo_rd2[s] = arow * 4 + ((2 * lh + s) ^ key_o(arow));
 
   // ---- tile bookkeeping
-  const int tiles_per_batch = N * tiles_per_row;
+  const int tiles_per_batch = p.R * tiles_per_row;
   u32x4_t raw[ITERS];
   float mval;
   auto tile_row = [&](int tile_id, int& j0) {
@@ -394,7 +394,9 @@ hipError_t launch(const TransitionArgs& a, hipStream_t stream) {
       (a.mask && (uint64_t)(a.N - 1) * (uint64_t)a.mask_view.stride_k * 4 + 4 > 0xffffffffull))
     return hipErrorInvalidValue;
   const int tiles_per_row = (a.N + 32 * kWaves - 1) / (32 * kWaves);
-  const long total = (long)a.B * a.N * tiles_per_row;
+  if (a.R < 1) return hipErrorInvalidValue;
+  const long total = (long)a.B * a.R * tiles_per_row;
+  if (total > 0x7fffffffl) return hipErrorInvalidValue;
   const int grid = (int)(total < cus ? total : cus);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * kWaves), smem, stream, a, tiles_per_row, (int)total);
   return hipGetLastError();
