@@ -77,7 +77,8 @@ typedef enum {
   OF3_OK = 0,
   OF3_EINVAL = -1, /* bad shape, stride, alignment, dtype or null pointer */
   OF3_ENOSPC = -2, /* workspace too small */
-  OF3_EHIP = -3    /* HIP launch error; code via of3_last_hip_error() */
+  OF3_EHIP = -3,   /* HIP launch error; code via of3_last_hip_error() */
+  OF3_ESTATIC = -4 /* of3_trimul_fwd_static: the problem needs more than OF3_STATIC_SCRATCH_BYTES */
 } of3_status;
 
 typedef enum { OF3_DTYPE_F32 = 0, OF3_DTYPE_BF16 = 1 } of3_dtype;
@@ -122,6 +123,22 @@ int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask,
                    const void* w_a_p, const void* w_a_g, const void* w_b_p, const void* w_b_g, const void* w_g,
                    const void* w_z, void* out, int64_t B, int64_t N, int64_t C, int64_t CH, int outgoing,
                    int add_residual, void* workspace, int64_t workspace_bytes, int dtype, void* stream);
+
+/* of3_trimul_fwd for callers that cannot allocate device memory or hand a workspace over (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, results and kernels as of3_trimul_fwd, minus the
+ * workspace: a, b and x live in a scratch array built into the library, OF3_STATIC_SCRATCH_BYTES
+ * per GPU, which every GPU the library runs on holds until the process ends.  The call allocates
+ * and frees nothing.  Problems with of3_trimul_workspace_bytes_for(dtype, B, N, C, CH) above that
+ * size return OF3_ESTATIC before anything is launched (bf16: B*CH*NP*NP <= 2^23, e.g. B = 1,
+ * C = CH = 128, N <= 256; fp32: B*CH*N*N <= 2^22).  All calls on one GPU share that GPU's array:
+ * calls that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered. */
+#define OF3_STATIC_SCRATCH_BYTES (48u << 20)
+int of3_trimul_fwd_static(const void* z, const int64_t z_strides[3], const float* mask,
+                          const int64_t mask_strides[3], const void* ln_in_w, const void* ln_in_b, const void* ln_out_w,
+                          const void* ln_out_b, const void* w_a_p, const void* w_a_g, const void* w_b_p,
+                          const void* w_b_g, const void* w_g, const void* w_z, void* out, int64_t B, int64_t N,
+                          int64_t C, int64_t CH, int outgoing, int add_residual, int dtype, void* stream);
 
 /* ---- triangle attention ------------------------------------------------------------- */
 

@@ -4,9 +4,38 @@
 
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "of3_kernels.h"
+#include "of3_launch.h"
+
+// Built-in scratch of of3_trimul_fwd_static: one copy per GPU the library runs on, held until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress; the device
+// address it yields (one per device) is what kernels and copies are given.
+static __device__ __align__(256) unsigned char scratch[OF3_STATIC_SCRATCH_BYTES];
 
 namespace {
+
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[of3::kMaxDevices];  // device address of `scratch` on each device, null until looked up
+
+// Address of the current device's copy of `scratch` (looked up on the first call on that device).
+hipError_t static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= of3::kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!ptr) return hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return hipSuccess;
+}
 
 thread_local int g_last_hip_error = 0;
 
@@ -99,6 +128,9 @@ const char* of3_status_string(int status) {
       return "workspace too small";
     case OF3_EHIP:
       return "HIP error (see of3_last_hip_error)";
+    case OF3_ESTATIC:
+      return "problem needs more scratch than the library's built-in OF3_STATIC_SCRATCH_BYTES; use the entry "
+             "point that takes a workspace";
     default:
       return "unknown status";
   }
@@ -243,6 +275,24 @@ int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask,
   if (st != OF3_OK) return st;
   return of3_trimul_out(x, z, z_strides, out, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_g, w_z, B, N, C, CH,
                         add_residual, stream);
+}
+
+int of3_trimul_fwd_static(const void* z, const int64_t z_strides[3], const float* mask,
+                          const int64_t mask_strides[3], const void* ln_in_w, const void* ln_in_b, const void* ln_out_w,
+                          const void* ln_out_b, const void* w_a_p, const void* w_a_g, const void* w_b_p,
+                          const void* w_b_g, const void* w_g, const void* w_z, void* out, int64_t B, int64_t N,
+                          int64_t C, int64_t CH, int outgoing, int add_residual, int dtype, void* stream) {
+  const int64_t need = of3_trimul_workspace_bytes_for(dtype, B, N, C, CH);
+  if (need < 0) return OF3_EINVAL;
+  if (need > (int64_t)OF3_STATIC_SCRATCH_BYTES) return OF3_ESTATIC;
+  void* ws = nullptr;
+  hipError_t e = static_scratch(&ws);
+  if (e != hipSuccess) return fail_hip(e);
+  // a, b and x are written in full before they are read (entries beyond N that the kernels read
+  // feed only outputs beyond N, which nothing reads), so what the last call left needs no clearing
+  return of3_trimul_fwd(z, z_strides, mask, mask_strides, ln_in_w, ln_in_b, ln_out_w, ln_out_b, w_a_p, w_a_g, w_b_p,
+                        w_b_g, w_g, w_z, out, B, N, C, CH, outgoing, add_residual, ws, (int64_t)OF3_STATIC_SCRATCH_BYTES,
+                        dtype, stream);
 }
 
 int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {

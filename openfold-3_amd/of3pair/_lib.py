@@ -11,7 +11,8 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 
 from .build import LIB_PATH
 
-OF3_OK, OF3_EINVAL, OF3_ENOSPC, OF3_EHIP = 0, -1, -2, -3
+OF3_OK, OF3_EINVAL, OF3_ENOSPC, OF3_EHIP, OF3_ESTATIC = 0, -1, -2, -3, -4
+OF3_STATIC_SCRATCH_BYTES = 48 << 20
 OF3_DTYPE_F32, OF3_DTYPE_BF16 = 0, 1
 
 _I64x3 = ctypes.POINTER(c_int64)
@@ -29,6 +30,8 @@ SIGNATURES = {
     "of3_trimul_out": (c_int, [c_void_p, c_void_p, _I64x3] + [c_void_p] * 7 + [c_int64] * 4 + [c_int, c_void_p]),
     "of3_trimul_fwd": (c_int, [c_void_p, _I64x3, c_void_p, _I64x3] + [c_void_p] * 11 + [c_int64] * 4
                        + [c_int, c_int, c_void_p, c_int64, c_int, c_void_p]),
+    "of3_trimul_fwd_static": (c_int, [c_void_p, _I64x3, c_void_p, _I64x3] + [c_void_p] * 11 + [c_int64] * 4
+                              + [c_int, c_int, c_int, c_void_p]),
     "of3_triattn_workspace_bytes": (c_int64, [c_int64] * 5),
     "of3_triattn_workspace_bytes_for": (c_int64, [c_int] + [c_int64] * 5),
     "of3_triattn_proj": (c_int, [c_void_p, _I64x3, c_void_p, _I64x3] + [c_void_p] * 11 + [c_int64] * 5
@@ -80,7 +83,7 @@ def check(status: int, what: str):
         return
     lib = load()
     msg = "%s: %s" % (what, lib.of3_status_string(status).decode())
-    if status == OF3_EINVAL:
+    if status in (OF3_EINVAL, OF3_ESTATIC):
         raise ValueError(msg)
     if status == OF3_EHIP:
         msg += " (hipError %d)" % lib.of3_last_hip_error()
