@@ -39,6 +39,14 @@ __device__ __forceinline__ f32x16_t mfma_32x32x16(u32x4_t a, u32x4_t b, f32x16_t
                                                  __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
+// the 8-deep form (two registers per operand: lane l supplies row/column l % 32 and the 4 consecutive
+// k-values of k-half l / 32); same matrix-pipe time as the 16-deep one
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_bits_t;
+__device__ __forceinline__ f32x16_t mfma_32x32x8(u32x2_t a, u32x2_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(bf16x4_bits_t, a),
+                                                  __builtin_bit_cast(bf16x4_bits_t, b), c, 0, 0, 0);
+}
+
 __device__ __forceinline__ f32x16_t zero16() {
   f32x16_t z;
 #pragma unroll

@@ -175,8 +175,12 @@ def test_triattn_proj(transposed, C, D, n, B):
     assert torch.isfinite(k[:, :, :, n:].float()).all() and torch.isfinite(vt[..., n:].float()).all()
 
 
-@pytest.mark.parametrize("D,n,B", [(32, 70, 2), (32, 256, 1), (16, 130, 1)])
-def test_triattn_flash(D, n, B):
+# logit_scale > 1 drives the logits far beyond the range in which a softmax without running maxima is
+# exact (queries shifted up overflow exp2, queries shifted down lose every term): the kernel's second
+# pass has to take over for those work-groups, next to work-groups that never need it
+@pytest.mark.parametrize("D,n,B,logit_scale", [(32, 70, 2, 1.0), (32, 256, 1, 1.0), (16, 130, 1, 1.0),
+                                               (32, 200, 1, 40.0), (16, 70, 1, 40.0)])
+def test_triattn_flash(D, n, B, logit_scale):
     L = lib()
     H = 4
     gen = _gen(53 + n)
@@ -185,8 +189,13 @@ def test_triattn_flash(D, n, B):
     k = bf(_randn(gen, B, n, H, np_, D))
     vt = bf(_randn(gen, B, n, H, D, np_))
     tb = _randn(gen, B, H, n, np_).contiguous()
+    if logit_scale != 1.0:
+        tb[:, 0] *= logit_scale                      # head 0: logits of +-100 and more
+        tb[:, 1, : n // 2] += 3.0 * logit_scale      # head 1: half of the queries far up ...
+        tb[:, 1, n // 2:] -= 5.0 * logit_scale       # ... the others far down; heads 2, 3 stay moderate
     mask = (torch.rand(B, n, n, generator=gen) > 0.3).float().to(DEV)
-    mask[:, 3, :] = 0  # a fully masked row
+    if logit_scale == 1.0:
+        mask[:, 3, :] = 0  # a fully masked row (its -1e9 absorbs moderate logits only: ulp(1.44e9) = 128)
     mb = torch.full((B, n, np_), float("-inf"), device=DEV)
     mb[..., :n] = LOG2E * 1e9 * (mask - 1)
     o = torch.full((B, n, n, H * D), float("nan"), dtype=torch.bfloat16, device=DEV)
