@@ -3,11 +3,14 @@ start + end, residual adds fused) on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--n 768] [--no-cpu]
 
-A step is one block forward, in place, on a z that already lives in HBM.  The workload is
-benchmark configuration 3: N_token = 768, c_z = 128, c_hidden_mul = 128, 4 heads x 32, batch 1,
+A step is one block forward on a z that already lives in HBM; every step reads the same input (the
+result goes to a tensor of the block's own, so the data-dependent branches of the kernels see the
+same data in every step).  The workload is benchmark configuration 3: N_token = 768, c_z = 128, c_hidden_mul = 128, 4 heads x 32, batch 1,
 all-ones mask, bf16, synthetic N(0,1) input and seeded random weights.  Prints one JSON line.
 
-Besides the whole-block time the line carries
+Besides the whole-block time (`value`: wall clock over the K steps; `step_ms_median` / `step_ms_min`:
+one event pair per step in a second loop of K steps; `inplace_ms_per_step`: the same loop run in place
+with inplace_safe, where z drifts from step to step, for comparison) the line carries
   roofline      the triangle-multiplication contraction (the MFMA-bound kernel the target
                 of >= 50 % of bf16 peak is set on): algorithmic 2*B*N^3*C_h flops over its
                 average launch duration, measured here with events on the launch stream;
@@ -29,8 +32,8 @@ Besides the whole-block time the line carries
                 the same N, for orientation; not part of `value`;
   fp32_block_ms  wall clock of the same pair-stack block in fp32 (the reference's default inference
                 precision; of3pair.PairStack on fp32 tensors), for orientation; not part of `value`;
-  cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path)
-                timed once on the host cores for the same workload.
+  cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path) on the host
+                cores for the same workload: one warm-up run, then the median of three.
 """
 from __future__ import annotations
 
@@ -53,8 +56,9 @@ CAL_BYTES = 256 << 20      # size of the calibration copy
 # HBM bytes per launch of the contraction at the headline workload (N=768, B=1), from two
 # counter passes of this command (rocprofv3 --pmc FETCH_SIZE, then --pmc WRITE_SIZE), each
 # scaled by what the same counter reads for the calibration copy; the summaries are kept in
-# profiles/.  None for any other workload.
-MEASURED_TRAFFIC = {("trimul_contract", 768): 539701909}
+# profiles/.  Keyed by (N, tile variant the library picks for that shape): a figure measured
+# on one kernel variant is not reported for another; None for any other workload.
+MEASURED_TRAFFIC = {(768, 1): 539701909}
 
 TRANSITION_N = 4           # hidden width factor of the pair transition (AF3 configuration)
 PAIR_BIAS_HEADS = 16       # heads of the pairformer's single-representation attention
@@ -137,9 +141,9 @@ def main():
     torch.cuda.synchronize()
     del cal_src, cal_dst
 
-    # ---- whole block, in place, inputs resident
+    # ---- whole block, inputs resident, the same input in every step
     def step():
-        block(z, mask, inplace_safe=True)
+        return block(z, mask, inplace_safe=False)
 
     for _ in range(args.warmup):
         step()
@@ -149,6 +153,29 @@ def main():
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # the same K steps once more with one event pair per step: spread of the step time
+    step_marks = []
+    for _ in range(args.steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        step()
+        e1.record()
+        step_marks.append((e0, e1))
+    torch.cuda.synchronize()
+    step_ms = sorted(e0.elapsed_time(e1) for e0, e1 in step_marks)
+    step_ms_median, step_ms_min = step_ms[len(step_ms) // 2], step_ms[0]
+
+    # and in place (the z of step k is the output of step k-1), for comparison
+    z_ip = z.clone()
+    block(z_ip, mask, inplace_safe=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        block(z_ip, mask, inplace_safe=True)
+    torch.cuda.synchronize()
+    inplace_ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    del z_ip
 
     # ---- per-kernel durations: the same block issued kernel by kernel through the stage
     # entry points of the C ABI, every launch bracketed by its own pair of events on the
@@ -276,7 +303,8 @@ def main():
                              "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4)}
     dom = kernels["trimul_contract"]
     roofline = {"kernel": "trimul_contract", "bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": dom["frac"], "traffic": MEASURED_TRAFFIC.get(("trimul_contract", N))}
+                "unit": "TFLOP/s", "frac": dom["frac"],
+                "traffic": MEASURED_TRAFFIC.get((N, args.contract_variant or int(lib.of3_trimul_contract_variant(B, N, CH))))}
 
     # ---- a whole PairFormerBlock through the module interface (pair stack, pair transition, pair
     # bias, attention over s, single transition), wall clock; informative, not part of `value`
@@ -310,21 +338,38 @@ def main():
     torch.cuda.synchronize()
     fp32_block_ms = (time.perf_counter() - t0) * 1e3 / fp32_reps
 
-    # ---- CPU baseline: the oracle on the host cores, one block of the same workload
+    # ---- CPU baseline: the oracle on the host cores, one block of the same workload; one warm-up
+    # run (thread pool, allocator), then the median of three
     cpu = None
     if not args.no_cpu:
         torch.set_num_threads(os.cpu_count() or 1)
         mask_h = torch.ones(B, N, N)
-        t0 = time.perf_counter()
-        with torch.no_grad():
-            orc.pair_stack_block(z_host, mask_h, params, H, row_chunk=32)
-        cpu_ms = (time.perf_counter() - t0) * 1e3
-        cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
-               "sample": "1 block forward, fp32, N=%d, same weights and input (tri-attn in 32-row chunks)" % N}
+        runs = []
+        for rep in range(4):
+            t0 = time.perf_counter()
+            with torch.no_grad():
+                orc.pair_stack_block(z_host, mask_h, params, H, row_chunk=32)
+            if rep > 0:
+                runs.append((time.perf_counter() - t0) * 1e3)
+        cpu_model = "unknown"
+        try:
+            with open("/proc/cpuinfo") as f:
+                for ln in f:
+                    if ln.startswith("model name"):
+                        cpu_model = ln.split(":", 1)[1].strip()
+                        break
+        except OSError:
+            pass
+        cpu = {"value": round(sorted(runs)[1], 1), "unit": "ms", "cores": torch.get_num_threads(), "kind": "port",
+               "cpu": cpu_model, "runs_ms": [round(r, 1) for r in runs],
+               "sample": "1 block forward, fp32, N=%d, same weights and input (tri-attn in 32-row chunks); "
+                         "median of 3 after one warm-up run" % N}
 
     line = {
         "metric": METRIC, "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak",
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "step_ms_median": round(step_ms_median, 4),
+        "step_ms_min": round(step_ms_min, 4), "inplace_ms_per_step": round(inplace_ms_per_step, 4),
+        "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "pair-stack block (trimul out+in, tri-attn start+end, residuals), B=1, N_token=%d, "
                                "c_z=128, c_hidden_mul=128, 4 heads x 32, all-ones mask" % N},

@@ -110,6 +110,11 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream);
 
+/* The tile variant (1..3) that variant = 0 selects for this shape, or OF3_EINVAL.  A pure function of
+ * the shape; lets a caller that records measurements name the kernel they were taken on.  (No
+ * counterpart in the reference: the choice is internal to torch's bmm there, tmu.py:71-97.) */
+int of3_trimul_contract_variant(int64_t B, int64_t N, int64_t CH);
+
 /* out = [z +] (LN_out(x) Wz^T) * sigmoid(LN_in(z) Wg^T); out uses z's strides. */
 int of3_trimul_out(const void* x, const void* z, const int64_t z_strides[3], void* out, const void* ln_in_w,
                    const void* ln_in_b, const void* ln_out_w, const void* ln_out_b, const void* w_g,

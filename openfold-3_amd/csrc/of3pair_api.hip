@@ -48,12 +48,21 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline int64_t align256(int64_t n) { return (n + 255) & ~(int64_t)255; }
 inline int64_t padded(int64_t n) { return (n + 127) / 128 * 128; }
 
+// The kernels count positions, tiles and work-groups in 32-bit integers: every shape whose padded
+// position count B * NP * NP does not fit one is refused before any launch (such a pair tensor
+// would exceed the memory of the device by far).
+inline bool positions_ok(int64_t B, int64_t N) {
+  if (B < 1 || N < 1 || N > (1 << 20) || B > 0x7fffffffll) return false;
+  const int64_t np = padded(N);
+  return np * np <= 0x7fffffffll / B;
+}
+
 inline bool trimul_dims_ok(int64_t B, int64_t N, int64_t C, int64_t CH) {
-  if (B < 1 || N < 1 || N > (1 << 20)) return false;
+  if (!positions_ok(B, N)) return false;
   return (C == 128 && CH == 128) || (C == 64 && CH == 64);
 }
 inline bool triattn_dims_ok(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
-  if (B < 1 || N < 1 || N > (1 << 20)) return false;
+  if (!positions_ok(B, N)) return false;
   if (B * H > 65535 || (N + 3) / 4 > 65535) return false;
   return H == 4 && ((C == 128 && D == 32) || (C == 64 && D == 16));
 }
@@ -66,10 +75,10 @@ inline bool mask_ok(const float* mask, const int64_t s[3]) {
 }
 
 inline bool f32_trimul_dims_ok(int64_t B, int64_t N, int64_t C, int64_t CH) {
-  return B >= 1 && N >= 1 && N <= (1 << 16) && C >= 1 && C <= 256 && CH >= 1 && CH <= 256;
+  return positions_ok(B, N) && N <= (1 << 16) && C >= 1 && C <= 256 && CH >= 1 && CH <= 256;
 }
 inline bool f32_triattn_dims_ok(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
-  return B >= 1 && N >= 1 && N <= (1 << 16) && C >= 1 && C <= 256 && H >= 1 && (D == 16 || D == 32 || D == 64) &&
+  return positions_ok(B, N) && N <= (1 << 16) && C >= 1 && C <= 256 && H >= 1 && (D == 16 || D == 32 || D == 64) &&
          H * D <= 256;
 }
 inline bool f32_strides_ok(const int64_t s[3]) { return s && s[0] >= 0 && s[1] > 0 && s[2] > 0; }
@@ -138,6 +147,11 @@ const char* of3_status_string(int status) {
 
 int64_t of3_padded_n(int64_t n) { return n < 1 ? 0 : padded(n); }
 
+int of3_trimul_contract_variant(int64_t B, int64_t N, int64_t CH) {
+  if (!positions_ok(B, N) || (CH != 128 && CH != 64)) return OF3_EINVAL;
+  return contract_variant_auto(B * CH, padded(N));
+}
+
 int64_t of3_trimul_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t CH) {
   if (!trimul_dims_ok(B, N, C, CH)) return OF3_EINVAL;
   const int64_t Np = padded(N);
@@ -180,7 +194,7 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
 
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream) {
-  if (B < 1 || N < 1 || (CH != 128 && CH != 64) || variant < 0 || variant > 3) return OF3_EINVAL;
+  if (!positions_ok(B, N) || (CH != 128 && CH != 64) || variant < 0 || variant > 3) return OF3_EINVAL;
   if (!a || !b || !x || !aligned16(a) || !aligned16(b) || !aligned16(x)) return OF3_EINVAL;
   const int64_t Np = padded(N);
   if (variant == 0) variant = contract_variant_auto(B * CH, Np);
@@ -456,7 +470,7 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
                        void* out, int64_t B, int64_t N, int64_t C, int64_t HID, int add_residual, int dtype,
                        void* stream) {
   const void* ptrs[] = {x, ln_w, ln_b, w_a, w_b, w_out, out};
-  if (B < 1 || N < 1 || N > (1 << 20) || !mask_ok(mask, mask_strides)) return OF3_EINVAL;
+  if (!positions_ok(B, N) || !mask_ok(mask, mask_strides)) return OF3_EINVAL;
   if (dtype == OF3_DTYPE_F32) {
     if (N > (1 << 16) || C < 1 || C > 256 || HID < 1 || HID > 1024 || !f32_strides_ok(x_strides)) return OF3_EINVAL;
     for (const void* p : ptrs)
@@ -521,8 +535,7 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
 
 int of3_pair_bias_fwd(const void* z, const int64_t z_strides[3], const void* ln_w, const void* ln_b, const void* w,
                       void* out, int64_t B, int64_t N, int64_t C, int64_t H, int dtype, void* stream) {
-  if (B < 1 || N < 1 || N > (1 << 16) || H < 1 || !z || !ln_w || !w || !out) return OF3_EINVAL;
-  if (B * N * ((N + 7) / 8) > 0x7fffffffll) return OF3_EINVAL;
+  if (!positions_ok(B, N) || N > (1 << 16) || H < 1 || !z || !ln_w || !w || !out) return OF3_EINVAL;
   if (dtype == OF3_DTYPE_F32) {
     if (C < 1 || C > 256 || H > 64 || !f32_strides_ok(z_strides)) return OF3_EINVAL;
     if (!aligned4(z) || !aligned4(ln_w) || !aligned4(ln_b) || !aligned4(w) || !aligned4(out)) return OF3_EINVAL;

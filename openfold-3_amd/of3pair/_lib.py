@@ -27,6 +27,7 @@ SIGNATURES = {
     "of3_trimul_workspace_bytes_for": (c_int64, [c_int] + [c_int64] * 4),
     "of3_trimul_proj": (c_int, [c_void_p, _I64x3, c_void_p, _I64x3] + [c_void_p] * 8 + [c_int64] * 4 + [c_int, c_void_p]),
     "of3_trimul_contract": (c_int, [c_void_p] * 3 + [c_int64] * 3 + [c_int, c_void_p]),
+    "of3_trimul_contract_variant": (c_int, [c_int64] * 3),
     "of3_trimul_out": (c_int, [c_void_p, c_void_p, _I64x3] + [c_void_p] * 7 + [c_int64] * 4 + [c_int, c_void_p]),
     "of3_trimul_fwd": (c_int, [c_void_p, _I64x3, c_void_p, _I64x3] + [c_void_p] * 11 + [c_int64] * 4
                        + [c_int, c_int, c_void_p, c_int64, c_int, c_void_p]),

@@ -15,23 +15,30 @@ import torch
 from . import _lib
 
 _workspaces: dict = {}
+_retired: list = []
 
 
 def _workspace(device, nbytes: int) -> torch.Tensor:
-    """Grow-only scratch per device, owned by this Python layer (the library allocates
-    nothing).  Kernels on one stream are ordered, so one buffer per device is shared by all
-    modules; callers using several streams on one device must pass their own workspace."""
-    buf = _workspaces.get(device)
+    """Grow-only scratch per (device, current stream), owned by this Python layer (the library
+    allocates nothing).  Kernels on one stream are ordered, so all modules running on a stream share
+    its buffer; another stream gets a buffer of its own.  A buffer that is outgrown is kept alive
+    until release_workspaces(): a HIP graph captured earlier still replays kernels that point into
+    it, and the caching allocator must not hand that memory to another tensor."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = None
-        _workspaces.pop(device, None)
+        if buf is not None:
+            _retired.append(buf)
         buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
-        _workspaces[device] = buf
+        _workspaces[key] = buf
     return buf
 
 
 def release_workspaces():
+    """Drops every scratch buffer, current and outgrown.  Only when no captured graph that used them
+    will be replayed again."""
     _workspaces.clear()
+    _retired.clear()
 
 
 def _require_gpu(t: torch.Tensor, name: str) -> int:
@@ -167,7 +174,8 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
     """Update of transition.py:256-268 (LayerNorm, SwiGLU, linear_out, mask), or x + update when
     add_residual.  x [*, N, N, C], mask [*, N, N] or None; a_weight / b_weight [n*C, C] are
     SwiGLU's linear_a (through SiLU) and linear_b, out_weight [C, n*C].  With C = 384 (the single
-    representation) x is [*, 384] and mask [*]: any leading dimensions."""
+    representation) x is [*, 384] and mask [*]: any leading dimensions (the transition is
+    position-wise, so a pair tensor of 384 channels takes that route too and gets the same result)."""
     code = _require_gpu(x, "x")
     lib = _lib.load()
     if x.shape[-1] == 384:  # the single representation: position-wise over [*, 384] rows
@@ -221,6 +229,9 @@ def _swiglu_transition_rows(x, mask, norm_weight, norm_bias, a_weight, b_weight,
                                          *[k.data_ptr() for k in keep], out.data_ptr(), rows, C, HID,
                                          int(bool(add_residual)), ws.data_ptr(), ws.numel(), code, _stream(x))
     _lib.check(st, "of3_transition_rows_fwd")
+    if inplace and out is not x:  # the kernel ran on a contiguous copy of a strided x
+        x.copy_(out)
+        return x
     return out
 
 
@@ -340,4 +351,7 @@ def attention_pair_bias(a, z, mask, norm_a_weight, norm_a_bias, norm_z_weight, n
                                         *[t.data_ptr() for t in w], out.data_ptr(), B, N, CS, H, D, float(inf),
                                         1 if add_residual else 0, ws.data_ptr(), ws.numel(), code, _stream(a))
     _lib.check(st, "of3_attn_pair_bias_fwd")
+    if inplace and out is not a:  # the kernel ran on a contiguous copy of a strided a
+        a.copy_(out)
+        return a
     return out

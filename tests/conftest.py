@@ -30,3 +30,12 @@ def pytest_collection_modifyitems(config, items):
     for it in items:
         if "gpu" in it.keywords:
             it.add_marker(skip)
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """After a GPU run: the achieved error figures of every parity comparison, as a text table."""
+    try:
+        import gpu_util
+    except Exception:
+        return
+    gpu_util.write_parity_summary(os.path.join(ROOT, "gpurun_out", "parity_summary.txt"))

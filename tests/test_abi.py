@@ -32,6 +32,7 @@ def test_header_declares_expected_entry_points():
     for required in ("of3_trimul_fwd", "of3_trimul_proj", "of3_trimul_contract", "of3_trimul_out",
                      "of3_triattn_fwd", "of3_triattn_proj", "of3_triattn_flash", "of3_triattn_out",
                      "of3_version", "of3_last_hip_error", "of3_status_string", "of3_padded_n",
+                     "of3_trimul_contract_variant",
                      "of3_trimul_workspace_bytes", "of3_triattn_workspace_bytes",
                      "of3_trimul_workspace_bytes_for", "of3_triattn_workspace_bytes_for",
                      "of3_transition_fwd", "of3_pair_bias_fwd", "of3_layer_norm_fwd", "of3_template_tail_fwd",
@@ -143,6 +144,26 @@ def test_stage_entry_points_validate(lib):
     assert lib.of3_trimul_contract(FAKE, FAKE, FAKE, 1, 64, 128, 9, None) == _lib.OF3_EINVAL   # unknown variant
     assert lib.of3_trimul_contract(FAKE, FAKE, FAKE, 1, 64, 96, 0, None) == _lib.OF3_EINVAL    # unsupported CH
     assert lib.of3_triattn_flash(FAKE, FAKE, FAKE, FAKE, FAKE, None, 1, 64, 4, 32, None) == _lib.OF3_EINVAL
+
+
+def test_shapes_beyond_32_bit_position_counts_are_refused(lib):
+    """B * NP * NP must fit a 32-bit integer (the kernels count positions and tiles in int): larger
+    shapes return OF3_EINVAL before any launch, in the stage entry points as in the fused ones."""
+    from of3pair import _lib
+
+    big_n, big_b = 46464, 40000  # 46464^2 > 2^31 ; 40000 * 256^2 > 2^31
+    assert lib.of3_trimul_contract(FAKE, FAKE, FAKE, 1, big_n, 128, 0, None) == _lib.OF3_EINVAL
+    assert lib.of3_trimul_contract(FAKE, FAKE, FAKE, big_b, 256, 128, 0, None) == _lib.OF3_EINVAL
+    assert lib.of3_triattn_flash(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 1, big_n, 4, 32, None) == _lib.OF3_EINVAL
+    assert lib.of3_triattn_flash(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, big_b, 256, 4, 32, None) == _lib.OF3_EINVAL
+    assert lib.of3_trimul_workspace_bytes(1, big_n, 128, 128) == _lib.OF3_EINVAL
+    assert lib.of3_triattn_workspace_bytes(big_b, 256, 128, 4, 32) == _lib.OF3_EINVAL
+    assert lib.of3_trimul_workspace_bytes_for(_lib.OF3_DTYPE_F32, big_b, 256, 128, 128) == _lib.OF3_EINVAL
+    assert lib.of3_trimul_contract_variant(1, big_n, 128) == _lib.OF3_EINVAL
+    # the largest shapes that pass are still accepted by the size queries
+    assert lib.of3_trimul_workspace_bytes(1, 46336, 128, 128) > 0
+    assert lib.of3_trimul_contract_variant(1, 768, 128) in (1, 2, 3, 4)
+    assert lib.of3_trimul_contract_variant(1, 768, 96) == _lib.OF3_EINVAL
 
 
 def test_check_maps_status_to_exceptions(lib):

@@ -129,3 +129,35 @@ def test_pair_block_in_a_hip_graph_replays_like_eager():
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(out_static, blk(z1, mask))
+
+
+def test_outgrown_workspace_stays_valid_for_a_captured_graph():
+    """A graph captured at a small N keeps pointing into the scratch buffer of its capture; later
+    eager calls at a larger N need more scratch.  The outgrown buffer must stay alive (and the graph's
+    own buffer untouched), so the replay still reproduces the eager result of the small problem."""
+    from of3pair import functional as F3
+
+    lib()
+    torch.cuda.synchronize()
+    F3.release_workspaces()  # earlier tests have grown the scratch already; no graph of theirs is replayed again
+    blk, _ = _block(128, 32, seed=5)
+    z_small = orc.round_bf16(orc.make_pair_input(31, (1,), 40, 128)).to(DEV).to(torch.bfloat16)
+    m_small = torch.ones(1, 40, 40, device=DEV)
+    eager_small = blk(z_small, m_small)
+    torch.cuda.synchronize()
+    z_static = z_small.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static = blk(z_static, m_small)
+    retired_before = len(F3._retired)
+    z_big = orc.round_bf16(orc.make_pair_input(32, (1,), 160, 128)).to(DEV).to(torch.bfloat16)
+    big = blk(z_big, torch.ones(1, 160, 160, device=DEV))  # grows the eager stream's scratch
+    assert torch.isfinite(big).all()
+    assert len(F3._retired) > retired_before, "the outgrown buffer is kept until release_workspaces()"
+    filler = torch.full((64 << 20,), 7, dtype=torch.uint8, device=DEV)  # would land in freed scratch memory
+    for rep in range(2):
+        z_static.copy_(z_small)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, eager_small), "replay %d after the workspace grew" % rep
+    assert int(filler[0]) == 7

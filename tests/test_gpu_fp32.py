@@ -6,7 +6,7 @@ benchmark configuration 1 (N=64, c_z=128, 4 heads x 32, all-ones mask) is the fi
 import pytest
 import torch
 
-from gpu_util import lib  # noqa: F401
+from gpu_util import lib, record_parity  # noqa: F401
 from oracle import pairstack_oracle as orc
 
 import of3pair
@@ -17,6 +17,7 @@ FP32_TOL = 1e-4
 
 
 def _maxerr(name, got, want):
+    record_parity(name, got, want, None, "fp32: max|err| <= 1e-4")
     err = float((got.float().cpu() - want).abs().max())
     print("%s: max|err| = %.3g (max|want| = %.3g)" % (name, err, float(want.abs().max())), flush=True)
     assert err <= FP32_TOL, "%s: %.3g" % (name, err)

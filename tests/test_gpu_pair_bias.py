@@ -4,7 +4,7 @@ the rms error of the oracle's own operations executed in bfloat16.  fp32: max-ab
 import pytest
 import torch
 
-from gpu_util import lib, report  # noqa: F401
+from gpu_util import lib, report, record_parity  # noqa: F401
 from oracle import pairstack_oracle as orc
 
 import of3pair
@@ -17,6 +17,8 @@ DEV = "cuda"
 def _check(name, got, want, rms_rel=5e-3, bf16_ref=None):
     got = got.float().cpu()
     want = want.float()
+    record_parity(name, got, want, bf16_ref, "max|err| <= 2e-2 max|want|, rms_rel <= %.1e%s" % (
+        rms_rel, ", floor <= 1.5" if bf16_ref is not None else ""))
     report(name, got, want, atol=2e-2 * float(want.abs().max()), rtol=0.0)
     erms = float((got - want).pow(2).mean().sqrt())
     assert erms <= rms_rel * float(want.pow(2).mean().sqrt()), "%s: rms error %.3g" % (name, erms)

@@ -17,7 +17,7 @@ import math
 import pytest
 import torch
 
-from gpu_util import lib, report  # noqa: F401  (lib() makes sure the library is built)
+from gpu_util import lib, report, record_parity  # noqa: F401  (lib() makes sure the library is built)
 from oracle import pairstack_oracle as orc
 
 import of3pair
@@ -30,6 +30,8 @@ REL = 2e-2
 def _check(name, got, want, rms_rel=5e-3, bf16_ref=None):
     got = got.float().cpu()
     want = want.float()
+    record_parity(name, got, want, bf16_ref, "max|err| <= 2e-2 max|want|, rms_rel <= %.1e%s" % (
+        rms_rel, ", floor <= 1.5" if bf16_ref is not None else ""))
     rms = float(want.pow(2).mean().sqrt())
     report(name, got, want, atol=REL * float(want.abs().max()), rtol=0.0)
     erms = float((got - want).pow(2).mean().sqrt())

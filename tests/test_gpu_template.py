@@ -7,7 +7,7 @@ of the oracle's own operations executed in bfloat16 where that floor is computed
 import pytest
 import torch
 
-from gpu_util import lib, report, stream  # noqa: F401
+from gpu_util import lib, report, stream, record_parity  # noqa: F401
 from oracle import pairstack_oracle as orc
 
 import of3pair
@@ -27,6 +27,8 @@ STACK_CFG = dict(c_t=64, c_hidden_tri_att=16, c_hidden_tri_mul=64, no_blocks=2, 
 def _check(name, got, want, rms_rel=5e-3, bf16_ref=None):
     got = got.float().cpu()
     want = want.float()
+    record_parity(name, got, want, bf16_ref, "max|err| <= 2e-2 max|want|, rms_rel <= %.1e%s" % (
+        rms_rel, ", floor <= 1.5" if bf16_ref is not None else ""))
     rms = float(want.pow(2).mean().sqrt())
     report(name, got, want, atol=REL * float(want.abs().max()), rtol=0.0)
     erms = float((got - want).pow(2).mean().sqrt())

@@ -367,3 +367,60 @@ def test_attention_pair_bias_invariants():
     o0 = orc.attention_pair_bias(a[:1], torch.zeros(1, n, n, cz), m0, p, h)
     o1 = orc.attention_pair_bias(a[:1], torch.zeros(1, n, n, cz), torch.ones(1, n), p, h)
     assert torch.isfinite(o0).all() and o0.shape == o1.shape
+
+
+def _brute_pair_block(z, mask, p, heads, mask_trans=True):
+    """PairBlock (base_blocks.py:408-480) as a float64 composition of the brute-force pieces."""
+    w = z.double().numpy()
+    w = w + bf.trimul_update(w, mask, orc._sub(p, "tri_mul_out."), True)
+    w = w + bf.trimul_update(w, mask, orc._sub(p, "tri_mul_in."), False)
+    w = w + bf.triattn_update(w, mask, orc._sub(p, "tri_att_start."), heads, starting=True)
+    w = w + bf.triattn_update(w, mask, orc._sub(p, "tri_att_end."), heads, starting=False)
+    return w + bf.transition_update(w, mask if mask_trans else None, orc._sub(p, "pair_transition."))
+
+
+@pytest.mark.parametrize("mask_trans", [True, False])
+def test_pair_block_matches_bruteforce_composition(mask_trans):
+    """orc.pair_block = the four triangle updates, then z + transition(z, mask or None): the order
+    of the modules, the residual adds and the _mask_trans switch against an independent float64
+    composition."""
+    n, c, hd, heads = 5, 8, 4, 2
+    p = orc.make_block_params(7, c, 8, hd, heads)
+    gen = torch.Generator().manual_seed(71)
+    p.update({"pair_transition." + k: v for k, v in orc.make_transition_params(gen, c, 2).items()})
+    z = orc.make_pair_input(8, (), n, c)
+    mask = orc.tail_padding_mask((), n, 1)
+    got = orc.pair_block(z, mask, p, heads, mask_trans=mask_trans).double().numpy()
+    want = _brute_pair_block(z, mask, p, heads, mask_trans)
+    assert np.abs(got - want).max() < 5e-4
+    # the switch matters on this input (masked positions keep the transition's update without it)
+    other = _brute_pair_block(z, mask, p, heads, not mask_trans)
+    assert np.abs(want - other).max() > 1e-2
+
+
+@pytest.mark.parametrize("mask_trans", [True, False])
+def test_pairformer_block_matches_bruteforce_composition(mask_trans):
+    """orc.pairformer_block (pairformer.py:176-213): z through the PairBlock first, then
+    s += attn_pair_bias(s, z_new, single_mask), s += single_transition(s, single_mask or None).
+    A composition that fed the old z into the attention, dropped a residual or swapped the two
+    single-representation updates differs by far more than the bound."""
+    n, cs, cz, hd, heads, cb, hb = 5, 12, 8, 4, 2, 3, 4
+    p = orc.make_pairformer_block_params(5, cs, cz, 8, hd, heads, cb, hb, 2)
+    gen = torch.Generator().manual_seed(72)
+    s = torch.randn(n, cs, generator=gen)
+    z = orc.make_pair_input(9, (), n, cz)
+    single_mask = torch.tensor([1, 1, 1, 0, 1.0])
+    pair_mask = single_mask[:, None] * single_mask[None, :]
+    s_got, z_got = orc.pairformer_block(s, z, single_mask, pair_mask, p, heads, hb, mask_trans=mask_trans)
+    zw = _brute_pair_block(z, pair_mask, orc._sub(p, "pair_stack."), heads, mask_trans)
+    sw = s.double().numpy()
+    sw = sw + bf.attention_pair_bias(sw, zw, single_mask, orc._sub(p, "attn_pair_bias."), hb)
+    sw = sw + bf.transition_update(sw, single_mask if mask_trans else None, orc._sub(p, "single_transition."))
+    assert np.abs(z_got.double().numpy() - zw).max() < 5e-4
+    assert np.abs(s_got.double().numpy() - sw).max() < 5e-4
+    # the attention must see the updated z: with the input z the result moves visibly
+    s_old = s.double().numpy() + bf.attention_pair_bias(s.double().numpy(), z.double().numpy(), single_mask,
+                                                        orc._sub(p, "attn_pair_bias."), hb)
+    s_new = s.double().numpy() + bf.attention_pair_bias(s.double().numpy(), zw, single_mask,
+                                                        orc._sub(p, "attn_pair_bias."), hb)
+    assert np.abs(s_old - s_new).max() > 1e-3
