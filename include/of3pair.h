@@ -106,11 +106,11 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
 
 /* x[b][c][i][j] = sum_k a[b][c][i][k] * b[b][c][j][k] over the padded planes; a, b in the
  * k-panel layout above, x row-major [B][CH][NP][NP].
- * variant: 0 = automatic; 1 / 2 / 3 = 256x192 / 256x128 / 256x256 output tiles. */
+ * variant: 0 = automatic; 1 / 2 / 3 / 4 = 256x192 / 256x128 / 256x256 / 384x192 output tiles. */
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream);
 
-/* The tile variant (1..3) that variant = 0 selects for this shape, or OF3_EINVAL.  A pure function of
+/* The tile variant (1..4) that variant = 0 selects for this shape, or OF3_EINVAL.  A pure function of
  * the shape; lets a caller that records measurements name the kernel they were taken on.  (No
  * counterpart in the reference: the choice is internal to torch's bmm there, tmu.py:71-97.) */
 int of3_trimul_contract_variant(int64_t B, int64_t N, int64_t CH);

@@ -101,17 +101,19 @@ inline const of3::bf16_t* bf(const void* p) { return static_cast<const of3::bf16
 inline of3::bf16_t* bf(void* p) { return static_cast<of3::bf16_t*>(p); }
 
 inline int contract_variant_auto(int64_t planes, int64_t Np) {
-  // Cheapest of the three output tile shapes for this problem on the 256 CUs of an MI355X:
+  // Cheapest of the four output tile shapes for this problem on the 256 CUs of an MI355X:
   // rounds of persistent work-groups x padded tile area, with a small bonus for the wider
-  // tiles, which move fewer operand bytes per flop.  (768: 256x192 gives every work-group
-  // exactly 6 tiles; 512, 1024, 2048: 256x256 divides the plane without waste.)
-  const int64_t bn[3] = {192, 128, 256};
-  const double eff[3] = {0.97, 0.90, 1.00};
+  // tiles, which move fewer operand bytes per flop.  (768: 384x192 gives every work-group
+  // exactly 4 tiles and every XCD whole planes per round; 512, 1024, 2048: 256x256 divides the
+  // plane without waste.)
+  const int64_t bm[4] = {256, 256, 256, 384};
+  const int64_t bn[4] = {192, 128, 256, 192};
+  const double eff[4] = {0.97, 0.90, 1.00, 1.00};
   int best = 1;
   double best_cost = 0;
-  for (int v = 0; v < 3; ++v) {
-    const int64_t tiles = planes * ((Np + 255) / 256) * ((Np + bn[v] - 1) / bn[v]);
-    const double cost = (double)((tiles + 255) / 256) * (256.0 * bn[v]) / eff[v];
+  for (int v = 0; v < 4; ++v) {
+    const int64_t tiles = planes * ((Np + bm[v] - 1) / bm[v]) * ((Np + bn[v] - 1) / bn[v]);
+    const double cost = (double)((tiles + 255) / 256) * (double)(bm[v] * bn[v]) / eff[v];
     if (v == 0 || cost < best_cost) {
       best = v + 1;
       best_cost = cost;
@@ -194,7 +196,7 @@ int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask
 
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream) {
-  if (!positions_ok(B, N) || (CH != 128 && CH != 64) || variant < 0 || variant > 3) return OF3_EINVAL;
+  if (!positions_ok(B, N) || (CH != 128 && CH != 64) || variant < 0 || variant > 4) return OF3_EINVAL;
   if (!a || !b || !x || !aligned16(a) || !aligned16(b) || !aligned16(x)) return OF3_EINVAL;
   const int64_t Np = padded(N);
   if (variant == 0) variant = contract_variant_auto(B * CH, Np);

@@ -35,6 +35,8 @@
 #include "of3_kernels.h"
 #include "of3_launch.h"
 
+#include <type_traits>
+
 namespace of3 {
 
 namespace {
@@ -330,6 +332,260 @@ hipError_t launch_contract(const bf16_t* a, const bf16_t* b, bf16_t* x, int plan
   return hipGetLastError();
 }
 
+
+// ---- eight-wave organisation: 384 x 192 output tiles ------------------------------------------
+// A plane of 768 x 768 is 2 x 4 = 8 such tiles, so the 32 work-groups of an XCD finish whole planes
+// together (4 per round) and no operand panel is fetched from HBM by two rounds; a tile moves 14 %
+// fewer operand bytes from L2 per flop than a 256 x 192 one.  Eight waves (4 along j x 2 along i),
+// each a 96 x 96 sub-tile (144 accumulator registers), two per SIMD; the ring has three stages of
+// 36 KB.  Both sides keep their natural row order; a lane therefore holds runs of 4 consecutive j,
+// which the epilogue writes as 8-byte pieces into a wave-private [32 i][96 j] staging block (chunk
+// index XOR (i / 4) % 4 within each group of four: conflict-free for the writers) and reads back as
+// whole 192-byte row segments.
+// A stage is 24 + 12 direct-to-LDS instructions: three j-side ones per wave, two i-side ones for
+// waves 0..3 and one for waves 4..7 (a wave-uniform difference, so every wait stays a constant).
+template <int kNS>
+__global__ __launch_bounds__(512, 1) void contract8_kernel(const bf16_t* __restrict__ pm,  // j side planes (b)
+                                                           const bf16_t* __restrict__ pn,  // i side planes (a)
+                                                           bf16_t* __restrict__ x, int Np, int tiles_m, int tiles_n,
+                                                           int total_tiles, int tiles_per_xcd) {
+  constexpr int BM = 384, BN = 192;
+  constexpr int WM = 96, WN = 96;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int ROWS = BM + BN;
+  constexpr int STAGE = ROWS * 4;
+  constexpr int MI = BM / 16 / 8;           // 3 j-side instructions per wave
+  constexpr int NI_LO = 2, NI_HI = 1;       // i-side instructions of waves 0..3 / 4..7
+  constexpr int IPW_LO = MI + NI_LO, IPW_HI = MI + NI_HI;
+  constexpr int NMMA = TM * TN;
+  constexpr int EPI_ROW = 12;               // 16-byte slots per staging row
+  constexpr int EPI_WAVE = 32 * EPI_ROW;    // slots per wave
+  constexpr int STORES = 6 * TN;            // output stores of a wave per tile
+  static_assert(IPW_LO <= NMMA, "a stage's loads are issued between the MFMAs of one k-step");
+  static_assert((kNS - 2) * IPW_LO + STORES < 64, "vmcnt budget");
+
+  extern __shared__ u32x4_t lds[];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool lo_wave = wave < 4;
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+
+  const int xcd = blockIdx.x & 7, slot_in_xcd = blockIdx.x >> 3, wgs_per_xcd = gridDim.x >> 3;
+  const int xcd_first = xcd * tiles_per_xcd;
+  int xcd_count = total_tiles - xcd_first;
+  xcd_count = xcd_count < 0 ? 0 : (xcd_count > tiles_per_xcd ? tiles_per_xcd : xcd_count);
+  const int my_tiles = slot_in_xcd < xcd_count ? (xcd_count - slot_in_xcd + wgs_per_xcd - 1) / wgs_per_xcd : 0;
+  if (my_tiles == 0) return;
+  const int per_plane = tiles_m * tiles_n;
+  const int nk = Np / kBK;
+  const size_t panel_bytes = (size_t)Np * kBK * 2;
+
+  auto tile_coords = [&](int t_local, int& plane, int& tm, int& tn) {
+    const int logical = xcd_first + slot_in_xcd + t_local * wgs_per_xcd;
+    plane = logical / per_plane;
+    const int rem = logical - plane * per_plane;
+    tm = rem / tiles_n;
+    tn = rem - tm * tiles_n;
+  };
+
+  // row block (16 rows) that instruction n of this wave fills, counted within its side
+  auto block_row = [&](int n) {
+    if (n < MI) return 16 * (wave * MI + n);
+    return lo_wave ? 16 * (wave * NI_LO + (n - MI)) : 16 * (4 * NI_LO + (wave - 4));
+  };
+  const int lrow = lane >> 2, lchunk = lane & 3;
+  const uint32_t off[2] = {(uint32_t)(lrow * 64 + 16 * (lchunk ^ key_n(lrow))),
+                           (uint32_t)(lrow * 64 + 16 * (lchunk ^ key_n(lrow + 16)))};
+  const char* dma_base[IPW_LO];
+  int issue_tile = 0, issue_kb = 0, issue_left = nk, issue_buf = 0;
+  auto dma_setup_tile = [&](int t_local) {
+    int plane, tm, tn;
+    tile_coords(t_local < my_tiles ? t_local : my_tiles - 1, plane, tm, tn);  // past the end: reload the last tile
+    const size_t plane_off = (size_t)plane * Np * Np * 2;
+    const int rows_m_left = Np - tm * BM, rows_n_left = Np - tn * BN;
+#pragma unroll
+    for (int n = 0; n < IPW_LO; ++n) {
+      const int rb = block_row(n);
+      const int left = n < MI ? rows_m_left : rows_n_left;
+      const int rbc = rb + 16 <= left ? rb : left - 16;  // whole blocks stay inside the plane
+      const bf16_t* side = n < MI ? pm : pn;
+      const int first = n < MI ? tm * BM : tn * BN;
+      dma_base[n] = reinterpret_cast<const char*>(side) + plane_off + (size_t)(first + rbc) * (kBK * 2);
+    }
+    issue_kb = ((tm + tn) & 3) % nk;
+    issue_left = nk;
+  };
+  auto issue_one = [&](int n) {  // n is a constant at every call site; the fifth one belongs to waves 0..3 only
+    if (n == IPW_LO - 1 && !lo_wave) return;
+    u32x4_t* buf = lds + issue_buf * STAGE;
+    const char* src = dma_base[n] + (size_t)issue_kb * panel_bytes;
+    const int rb = block_row(n);
+    __builtin_amdgcn_global_load_lds((const void OF3_GLOBAL_AS*)(src + off[(rb >> 4) & 1]),
+                                     (void OF3_LDS_AS*)(buf + ((n < MI ? 0 : BM) + rb) * 4), 16, 0, 0);
+  };
+  auto issue_advance = [&]() {
+    issue_buf = issue_buf + 1 == kNS ? 0 : issue_buf + 1;
+    issue_kb = issue_kb + 1 == nk ? 0 : issue_kb + 1;
+    if (--issue_left == 0) dma_setup_tile(++issue_tile);
+  };
+  // "at most `stages` whole stages of this wave's loads (plus `extra` stores) still outstanding"
+  auto wait_stages = [&](auto stages, auto extra) {
+    constexpr int S = decltype(stages)::value, E = decltype(extra)::value;
+    if (lo_wave) wait_vmcnt<S * IPW_LO + E>();
+    else wait_vmcnt<S * IPW_HI + E>();
+  };
+
+  int am_slot[TM], bn_slot[TN];
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt) {
+    const int row = wm0 + 32 * mt + l32;
+    am_slot[mt] = row * 4 + (lh ^ key_n(row));
+  }
+#pragma unroll
+  for (int nt = 0; nt < TN; ++nt) {
+    const int row = wn0 + 32 * nt + l32;
+    bn_slot[nt] = (BM + row) * 4 + (lh ^ key_n(row));
+  }
+  auto fetch = [&](const u32x4_t* buf, int ks, u32x4_t (&af)[TM], u32x4_t (&bfr)[TN]) {
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt) af[mt] = buf[am_slot[mt] ^ (2 * ks)];
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) bfr[nt] = buf[bn_slot[nt] ^ (2 * ks)];
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) acc[mt][nt] = zero16();
+  auto mma_and_issue = [&](const u32x4_t (&af)[TM], const u32x4_t (&bfr)[TN]) {
+    int n = 0;
+#pragma unroll
+    for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < TN; ++nt) {
+        acc[mt][nt] = mfma_32x32x16(af[mt], bfr[nt], acc[mt][nt]);
+        if (n < IPW_LO) issue_one(n++);
+      }
+    issue_advance();
+  };
+
+  dma_setup_tile(0);
+#pragma unroll
+  for (int s = 0; s < kNS; ++s) {
+#pragma unroll
+    for (int n = 0; n < IPW_LO; ++n) issue_one(n);
+    issue_advance();
+  }
+  wait_stages(std::integral_constant<int, kNS - 1>{}, std::integral_constant<int, 0>{});
+  compiler_fence();
+  __builtin_amdgcn_s_barrier();
+  compiler_fence();
+
+  u32x4_t a0[TM], b0[TN], a1[TM], b1[TN];
+  fetch(lds, 0, a0, b0);
+
+  int cur_buf = 0;
+  bool stores_pending = false;
+  for (int t_local = 0; t_local < my_tiles; ++t_local) {
+    for (int kb = 0; kb < nk; ++kb) {
+      const u32x4_t* cur = lds + cur_buf * STAGE;
+      acc[0][0] = mfma_32x32x16(a0[0], b0[0], acc[0][0]);
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(cur, 1, a1, b1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < TN; ++nt)
+          if (mt + nt > 0) acc[mt][nt] = mfma_32x32x16(a0[mt], b0[nt], acc[mt][nt]);
+      __builtin_amdgcn_sched_barrier(0);
+
+      // as in the four-wave kernel: stage s is in registers, stage s+1 must have landed in every
+      // wave, the newest kNS-2 stages (and a finished tile's stores, for its first stages) may
+      // stay in flight
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): a1/b1 have arrived
+      if (stores_pending && kb < kNS - 1)
+        wait_stages(std::integral_constant<int, kNS - 2>{}, std::integral_constant<int, STORES>{});
+      else
+        wait_stages(std::integral_constant<int, kNS - 2>{}, std::integral_constant<int, 0>{});
+      compiler_fence();
+      __builtin_amdgcn_s_barrier();
+      compiler_fence();
+      __builtin_amdgcn_sched_barrier(0);
+
+      cur_buf = cur_buf + 1 == kNS ? 0 : cur_buf + 1;
+      fetch(lds + cur_buf * STAGE, 0, a0, b0);
+      mma_and_issue(a1, b1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- tile finished: 32-row blocks through the wave's staging area, 192-byte row segments out
+    int plane, tm, tn;
+    tile_coords(t_local, plane, tm, tn);
+    bf16_t* xo = x + (size_t)plane * Np * Np;
+    u32x2_t* epi2 = reinterpret_cast<u32x2_t*>(lds + kNS * STAGE + wave * EPI_WAVE);
+    const u32x4_t* epi4 = lds + kNS * STAGE + wave * EPI_WAVE;
+    const int jbase = tm * BM + wm0;
+    int n_stores = 0;
+#pragma unroll
+    for (int nt = 0; nt < TN; ++nt) {
+#pragma unroll
+      for (int mt = 0; mt < TM; ++mt) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {  // registers 4g..4g+3: j-local = 32*mt + 8*g + 4*lh + (0..3) of row i = l32
+          const u32x2_t v = {pack_bf16(acc[mt][nt][4 * g], acc[mt][nt][4 * g + 1]),
+                             pack_bf16(acc[mt][nt][4 * g + 2], acc[mt][nt][4 * g + 3])};
+          epi2[(l32 * EPI_ROW + 4 * mt + (g ^ ((l32 >> 2) & 3))) * 2 + lh] = v;
+        }
+        acc[mt][nt] = zero16();
+      }
+      const int i0 = tn * BN + wn0 + 32 * nt;
+      const bool whole = i0 + 32 <= Np && jbase + WM <= Np;  // wave-uniform
+#pragma unroll
+      for (int rr = 0; rr < 6; ++rr) {
+        const int idx = 64 * rr + lane, row = idx / 12, chunk = idx - 12 * row;
+        const u32x4_t v = epi4[row * EPI_ROW + (chunk ^ ((row >> 2) & 3))];
+        if (whole || (i0 + row < Np && jbase + 8 * chunk < Np))
+          *reinterpret_cast<u32x4_t*>(xo + (size_t)(i0 + row) * Np + jbase + 8 * chunk) = v;
+      }
+      if (whole) n_stores += 6;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // only a complete set of unconditional stores is accounted for exactly; otherwise the next
+    // waits simply cover them too
+    stores_pending = (n_stores == STORES);
+  }
+  wait_vmcnt<0>();
+}
+
+template <int kNS>
+hipError_t launch_contract8(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, hipStream_t stream) {
+  constexpr int BM = 384, BN = 192;
+  auto kern = contract8_kernel<kNS>;
+  const size_t smem = ((size_t)kNS * (BM + BN) * 4 + 8 * 32 * 12) * sizeof(u32x4_t);  // ring + epilogue staging
+  static int cache[kMaxDevices];
+  int cus = 0;
+  hipError_t e = per_device(
+      cache,
+      [&](int dev, int* v) {
+        hipError_t s = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        return s != hipSuccess ? s : cu_count(dev, v);
+      },
+      &cus);
+  if (e != hipSuccess) return e;
+  const int tiles_m = (Np + BM - 1) / BM, tiles_n = (Np + BN - 1) / BN;
+  const int total = planes * tiles_m * tiles_n;
+  const int tiles_per_xcd = (total + 7) / 8;
+  int grid = (cus / 8) * 8;
+  if (grid < 8) grid = 8;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), smem, stream, b, a, x, Np, tiles_m, tiles_n, total, tiles_per_xcd);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
@@ -341,6 +597,8 @@ hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, i
       return launch_contract<128, 4>(a, b, x, planes, Np, stream);
     case 3:
       return launch_contract<256, 4>(a, b, x, planes, Np, stream);
+    case 4:
+      return launch_contract8<3>(a, b, x, planes, Np, stream);
     default:
       return hipErrorInvalidValue;
   }

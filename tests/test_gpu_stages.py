@@ -36,7 +36,7 @@ def _to_panels(t):
     return t.reshape(*lead, rows, k // 32, 32).transpose(-2, -3).contiguous()
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("n", [128, 384, 640, 768])
 def test_contract(variant, n):
     L = lib()
