@@ -5,7 +5,8 @@ attention.py:366-413), here with a single implementation and no dispatch.
 All functions run on the current CUDA(HIP) stream of the tensors' device, are forward-only
 and accept bf16 or fp32 pair tensors shaped [*, N, N, C] (any number of leading batch
 dimensions, a transposed view in the two N dimensions is fine and is not copied).  bf16 runs
-the bf16 MFMA kernels; fp32 (the reference's default inference precision) runs the library's
+the bf16 MFMA kernels (built for the AF3 widths; any other width runs on the fp32 kernels and is
+rounded to bf16 at the end); fp32 (the reference's default inference precision) runs the library's
 fp32 kernels (slower, the precision path); parameters are converted to the tensor's dtype.
 """
 from __future__ import annotations
@@ -50,6 +51,18 @@ def _require_gpu(t: torch.Tensor, name: str) -> int:
     if t.dtype == torch.float32:
         return _lib.OF3_DTYPE_F32
     raise ValueError("%s must be bfloat16 or float32 (got %s)" % (name, t.dtype))
+
+
+def _through_fp32(fn, x, inplace, *args, **kwargs):
+    """A bf16 call whose channel widths the bf16 MFMA kernels do not serve (they are built for the
+    AF3 widths) runs on the library's fp32 kernels instead: the activations are widened on the
+    device, every operation is the fp32 one, the result is rounded to bf16 once at the end.  Still
+    the HIP path; slower, and closer to an fp32 evaluation than the reference's bf16 path is."""
+    out = fn(x.float(), *args, inplace=False, **kwargs).to(torch.bfloat16)
+    if inplace:
+        x.copy_(out)
+        return x
+    return out
 
 
 def _flatten_pair(z: torch.Tensor):
@@ -126,6 +139,10 @@ def triangle_multiplicative_update(z, mask, norm_in_weight, norm_in_bias, norm_o
     B, N, _, C = z4.shape
     CH = a_p_weight.shape[0]
     nbytes = lib.of3_trimul_workspace_bytes_for(code, B, N, C, CH)
+    if nbytes < 0 and code == _lib.OF3_DTYPE_BF16 and lib.of3_trimul_workspace_bytes_for(_lib.OF3_DTYPE_F32, B, N, C, CH) >= 0:
+        return _through_fp32(triangle_multiplicative_update, z, inplace, mask, norm_in_weight, norm_in_bias,
+                             norm_out_weight, norm_out_bias, a_p_weight, a_g_weight, b_p_weight, b_g_weight,
+                             g_out_weight, p_out_weight, outgoing=outgoing, add_residual=add_residual)
     if nbytes < 0:
         raise ValueError("triangle multiplication: bf16 supports (c_z, c_hidden) = (128,128) or (64,64), fp32 any "
                          "widths up to 256; got (%d,%d) in %s" % (C, CH, z.dtype))
@@ -154,6 +171,10 @@ def triangle_attention(x, mask, norm_weight, norm_bias, bias_weight, q_weight, k
     H = int(no_heads)
     D = q_weight.shape[0] // H
     nbytes = lib.of3_triattn_workspace_bytes_for(code, B, N, C, H, D)
+    if nbytes < 0 and code == _lib.OF3_DTYPE_BF16 and lib.of3_triattn_workspace_bytes_for(_lib.OF3_DTYPE_F32, B, N, C, H, D) >= 0:
+        return _through_fp32(triangle_attention, x, inplace, mask, norm_weight, norm_bias, bias_weight, q_weight,
+                             k_weight, v_weight, g_weight, o_weight, no_heads=no_heads, inf=inf,
+                             add_residual=add_residual)
     if nbytes < 0:
         raise ValueError("triangle attention: bf16 supports 4 heads with (c_in, c_head) = (128,32) or (64,16), fp32 "
                          "head widths 16/32/64; got c_in=%d heads=%d c_head=%d in %s" % (C, H, D, x.dtype))
@@ -193,6 +214,9 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
         st = lib.of3_transition_fwd(x4.data_ptr(), _lib.strides3(x4.stride()[:3]), mptr, mstr,
                                     *[k.data_ptr() for k in keep], out4.data_ptr(), B, N, C, HID,
                                     int(bool(add_residual)), code, _stream(x))
+    if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and C <= 256 and HID <= 1024:
+        return _through_fp32(swiglu_transition, x, inplace, mask, norm_weight, norm_bias, a_weight, b_weight, out_weight,
+                             add_residual=add_residual)
     if st == _lib.OF3_EINVAL:
         raise ValueError("pair transition: bf16 supports c_in 64 or 128 with a hidden width n*c_in that is a multiple "
                          "of 32 and at least 128, fp32 c_in <= 256 and n*c_in <= 1024; got c_in=%d hidden=%d in %s"

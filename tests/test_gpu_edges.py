@@ -161,3 +161,25 @@ def test_outgrown_workspace_stays_valid_for_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(out_static, eager_small), "replay %d after the workspace grew" % rep
     assert int(filler[0]) == 7
+
+
+def test_bf16_widths_outside_the_mfma_kernels_run_on_the_fp32_kernels():
+    """The bf16 MFMA kernels serve the AF3 widths; a bf16 pair tensor of any other width (here
+    c_z = 96, c_hidden_mul = 40, 3 heads of 16, transition n = 2) is widened on the device, runs on
+    the fp32 kernels and is rounded to bf16 at the end: same interface, in-place contract included."""
+    lib()
+    c, ch, d, heads, n = 96, 40, 16, 3, 37
+    p = _round_params(orc.make_block_params(61, c, ch, d, heads))
+    gen = torch.Generator().manual_seed(62)
+    p.update({"pair_transition." + k: orc.round_bf16(v) for k, v in orc.make_transition_params(gen, c, 2).items()})
+    blk = _load(of3pair.PairBlock(c, ch, d, heads, "swiglu", 2, 0.0, False, 1e9), p)
+    z = orc.round_bf16(orc.make_pair_input(63, (2,), n, c))
+    mask = orc.tail_padding_mask((2,), n, torch.tensor([5, 0]))
+    zg = z.to(DEV).to(torch.bfloat16)
+    got = blk(zg, mask.to(DEV))
+    assert got.dtype == torch.bfloat16 and torch.equal(zg.float().cpu(), z)
+    want = orc.pair_block(z, mask, p, heads)
+    _check("odd-width bf16 block", got, want, rms_rel=1.2e-2)
+    res = blk(zg, mask.to(DEV), inplace_safe=True)
+    assert res.data_ptr() == zg.data_ptr()
+    assert torch.equal(res, got)

@@ -145,11 +145,11 @@ def test_transition_full_size_at_sampled_rows(n, rows):
 
 def test_transition_rejects_unsupported():
     lib()
-    x = torch.zeros(1, 8, 8, 32, device=DEV, dtype=torch.bfloat16)  # c_in = 32 has no bf16 kernel
-    w = torch.zeros(128, 32, device=DEV, dtype=torch.bfloat16)
+    x = torch.zeros(1, 8, 8, 32, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(2048, 32, device=DEV, dtype=torch.bfloat16)  # hidden width beyond what any kernel serves
     with pytest.raises(ValueError):
         F3.swiglu_transition(x, None, torch.ones(32, device=DEV), torch.zeros(32, device=DEV), w, w,
-                             torch.zeros(32, 128, device=DEV))
+                             torch.zeros(32, 2048, device=DEV))
 
 
 @pytest.mark.parametrize("mask_trans", [True, False])
