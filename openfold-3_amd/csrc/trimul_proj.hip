@@ -132,6 +132,10 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
     float mval[TPW];
 #pragma unroll
     for (int tt = 0; tt < TPW; ++tt) mval[tt] = (kfirst + tt < N && r < N) ? (p.mask ? mraw[tt] : 1.f) : 0.f;
+    bool not_one = false;
+#pragma unroll
+    for (int tt = 0; tt < TPW; ++tt) not_one |= mval[tt] != 1.f;
+    const bool masked = __builtin_amdgcn_ballot_w64(not_one) != 0;  // wave-uniform
 
     // ---- LayerNorm phase: wave w normalises positions [16w, 16w+16) of the tile
     float lw[8], lb[8];
@@ -164,8 +168,15 @@ __global__ __launch_bounds__(512) void trimul_proj_kernel(TrimulProjArgs p, int 
         accg = mfma_32x32x16(wg[s], bop, accg);
         accp = mfma_32x32x16(wp[s], bop, accp);
       }
+      // mask * sigmoid(gate) * projection; a wave whose positions all carry mask 1 (the usual tile)
+      // skips the multiplication by 1
+      if (masked) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) res[tt][v] = (mval[tt] * sigmoidf_fast(accg[v])) * accp[v];
+        for (int v = 0; v < 16; ++v) res[tt][v] = (mval[tt] * sigmoidf_fast(accg[v])) * accp[v];
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) res[tt][v] = sigmoidf_fast(accg[v]) * accp[v];
+      }
     }
     // stores: register v of a lane is channel 32*ot + 8*(v/4) + 4*lh + v%4; k-panel layout
     // plane[k / 32][row][k % 32].  r < Np always (Np is a multiple of 128): rows between N and
