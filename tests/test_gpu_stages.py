@@ -213,6 +213,48 @@ def test_triattn_flash(D, n, B, logit_scale):
     report("flash o", o, want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_triattn_flash_random_shapes(seed):
+    """Seeded random shapes, mask densities and logit ranges: ragged N around the 32-key and 128-query
+    tile sizes, work-groups that finish in the first pass next to ones that need the second."""
+    import random
+
+    L = lib()
+    rnd = random.Random(1000 + seed)
+    H = 4
+    D = rnd.choice([16, 32])
+    n = rnd.choice([1, 2, 31, 32, 33, 63, 65, 127, 128, 129, 160, 191, 193, 255, 257]) if seed < 8 else rnd.randint(1, 300)
+    B = rnd.choice([1, 2])
+    scale = rnd.choice([1.0, 1.0, 8.0, 30.0])
+    density = rnd.choice([1.0, 0.9, 0.5])
+    gen = _gen(7000 + seed)
+    np_ = L.of3_padded_n(n)
+    q = bf(_randn(gen, B, n, H, np_, D))
+    k = bf(_randn(gen, B, n, H, np_, D))
+    vt = bf(_randn(gen, B, n, H, D, np_))
+    tb = (_randn(gen, B, H, n, np_) * scale).contiguous()
+    mask = (torch.rand(B, n, n, generator=gen) < density).float().to(DEV)
+    if scale == 1.0 and n > 3:
+        mask[:, n // 2, :] = 0  # a fully masked row (moderate logits only: -1e9 absorbs |logit| < 64)
+    else:
+        mask[:, :, 0] = 1       # every row keeps a key, so the softmax does not hinge on the absorption
+    mb = torch.full((B, n, np_), float("-inf"), device=DEV)
+    mb[..., :n] = LOG2E * 1e9 * (mask - 1)
+    o = torch.full((B, n, n, H * D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    print("flash random", seed, "D", D, "n", n, "B", B, "scale", scale, "density", density, flush=True)
+    vtp = _to_panels(vt)
+    st = L.of3_triattn_flash(q.data_ptr(), k.data_ptr(), vtp.data_ptr(), tb.data_ptr(), mb.data_ptr(), o.data_ptr(),
+                             B, n, H, D, stream())
+    assert st == 0, L.of3_status_string(st)
+    torch.cuda.synchronize()
+    qf, kf, vf = q[:, :, :, :n].float(), k[:, :, :, :n].float(), vt[..., :n].float()
+    s = torch.einsum("bihqd,bihkd->bihqk", qf, kf)
+    s = (s + mb[:, :, None, None, :n]) + tb[:, None, :, :, :n]
+    p = torch.softmax(s * math.log(2.0), dim=-1)
+    want = torch.einsum("bihqk,bihdk->biqhd", p, vf).reshape(B, n, n, H * D)
+    report("flash o (random shapes)", o, want, atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("transposed,add_residual", [(False, 0), (True, 1)])
 @pytest.mark.parametrize("C,D,n,B", [(128, 32, 70, 2), (64, 16, 130, 1)])
 def test_triattn_out(transposed, add_residual, C, D, n, B):
