@@ -33,9 +33,12 @@ def pytest_collection_modifyitems(config, items):
 
 
 def pytest_sessionfinish(session, exitstatus):
-    """After a GPU run: the achieved error figures of every parity comparison, as a text table."""
+    """After a GPU run: the achieved error figures of every parity comparison, as a text table, into
+    the file OF3_PARITY_SUMMARY names."""
     try:
         import gpu_util
     except Exception:
         return
-    gpu_util.write_parity_summary(os.path.join(ROOT, "gpurun_out", "parity_summary.txt"))
+    path = os.environ.get("OF3_PARITY_SUMMARY")
+    if path:
+        gpu_util.write_parity_summary(path)

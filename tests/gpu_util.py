@@ -58,9 +58,9 @@ PARITY_RECORDS = []
 
 
 def record_parity(name, got, want, bf16_ref=None, bound=None):
-    """Keeps the achieved error figures of one comparison; tests/conftest.py writes them to
-    gpurun_out/parity_summary.txt when the session ends (a copy of one full GPU run is tracked under
-    profiles/).  `bound` describes the assertion the figures were held against."""
+    """Keeps the achieved error figures of one comparison; when the session ends, tests/conftest.py
+    writes them to the file the environment variable OF3_PARITY_SUMMARY names (nothing is written
+    without it).  `bound` describes the assertion the figures were held against."""
     got, want = got.float().cpu(), want.float().cpu()
     err = (got - want).abs()
     rms_want = float(want.pow(2).mean().sqrt())
@@ -80,7 +80,7 @@ def record_parity(name, got, want, bf16_ref=None, bound=None):
 def write_parity_summary(path):
     if not PARITY_RECORDS:
         return
-    os.makedirs(os.path.dirname(path), exist_ok=True)
+    os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
     with open(path, "w") as f:
         f.write("# achieved errors of the GPU parity tests (HIP path vs fp32 CPU oracle), one line per compared tensor\n")
         f.write("# max_rel = max|err| / max|want| ; rms_rel = rms(err) / rms(want) ; floor = rms(err) / rms error of the\n")
