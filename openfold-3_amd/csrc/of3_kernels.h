@@ -196,10 +196,16 @@ struct TrimulF32Args {
   const float *ln_in_w, *ln_in_b, *ln_out_w, *ln_out_b;
   const float *w_ap, *w_ag, *w_bp, *w_bg, *w_g, *w_z;
   float *a, *b, *x;                  // workspace, [B][CH][N][N] each
+  void* wsplit;                      // workspace, trimul_wsplit_bytes(C, CH) bytes, 16-byte aligned; may be null
   float* out;
   int B, N, C, CH, add_residual;
 };
 hipError_t trimul_fwd_f32(const TrimulF32Args& args, hipStream_t stream);
+// room for the six weight matrices split into three bf16 terms each, rows padded to multiples of 32
+inline long wsplit_elems(long rows, long K) { return (rows + 31) / 32 * 32 * K; }
+inline size_t trimul_wsplit_bytes(long C, long CH) {
+  return (size_t)6 * (4 * wsplit_elems(CH, C) + wsplit_elems(C, C) + wsplit_elems(C, CH));
+}
 
 struct TriattnF32Args {
   const float* x;
@@ -209,11 +215,15 @@ struct TriattnF32Args {
   float *q, *k, *v;                  // workspace, [B][N][H][N][D] each
   float *tb;                         // workspace, [B][H][N][N]
   float *o;                          // workspace, [B][N][N][H*D]
+  void* wsplit;                      // workspace, triattn_wsplit_bytes(C, H, D) bytes, 16-byte aligned; may be null
   float* out;
   int B, N, C, H, D, add_residual;
   float inf;
 };
 hipError_t triattn_fwd_f32(const TriattnF32Args& args, hipStream_t stream);
+inline size_t triattn_wsplit_bytes(long C, long H, long D) {
+  return (size_t)6 * (4 * wsplit_elems(H * D, C) + wsplit_elems(C, H * D) + wsplit_elems(H, C));
+}
 
 struct TransitionF32Args {
   const float* x;

@@ -163,7 +163,8 @@ int64_t of3_trimul_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t CH) 
 int64_t of3_trimul_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t CH) {
   if (dtype == OF3_DTYPE_BF16) return of3_trimul_workspace_bytes(B, N, C, CH);
   if (dtype != OF3_DTYPE_F32 || !f32_trimul_dims_ok(B, N, C, CH)) return OF3_EINVAL;
-  return 3 * align256(B * CH * N * N * 4);
+  // a, b, x and the weights split into three bf16 terms
+  return 3 * align256(B * CH * N * N * 4) + align256((int64_t)of3::trimul_wsplit_bytes(C, CH));
 }
 
 int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
@@ -265,6 +266,7 @@ int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask,
     a.a = reinterpret_cast<float*>(ws);
     a.b = reinterpret_cast<float*>(ws + part);
     a.x = reinterpret_cast<float*>(ws + 2 * part);
+    a.wsplit = ws + 3 * part;
     a.out = static_cast<float*>(out);
     a.B = (int)B;
     a.N = (int)N;
@@ -321,7 +323,9 @@ int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, 
 int64_t of3_triattn_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
   if (dtype == OF3_DTYPE_BF16) return of3_triattn_workspace_bytes(B, N, C, H, D);
   if (dtype != OF3_DTYPE_F32 || !f32_triattn_dims_ok(B, N, C, H, D)) return OF3_EINVAL;
-  return 4 * align256(B * N * N * H * D * 4) + align256(B * H * N * N * 4);
+  // q, k, v, o, the triangle bias and the weights split into three bf16 terms
+  return 4 * align256(B * N * N * H * D * 4) + align256(B * H * N * N * 4) +
+         align256((int64_t)of3::triattn_wsplit_bytes(C, H, D));
 }
 
 int of3_triattn_proj(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
@@ -435,6 +439,7 @@ int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask
     a.v = reinterpret_cast<float*>(ws + 2 * part);
     a.o = reinterpret_cast<float*>(ws + 3 * part);
     a.tb = reinterpret_cast<float*>(ws + 4 * part);
+    a.wsplit = ws + 4 * part + align256(B * H * N * N * 4);
     a.out = static_cast<float*>(out);
     a.B = (int)B;
     a.N = (int)N;

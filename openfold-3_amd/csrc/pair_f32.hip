@@ -32,6 +32,11 @@ constexpr float kEps = 1e-5f;
 
 constexpr float kLog2eF32 = 1.4426950408889634f;
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+// the matrix-pipe kernels: the hardware's exp2 and reciprocal (1 ulp each; the rounding of x * log2(e)
+// adds |x| * 2^-24 relative), a sixth of the instructions
+__device__ __forceinline__ float sigmoid_hw_f32(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * kLog2eF32));
+}
 
 // LayerNorm of kP positions (32 lanes each) from global rows into shared xn[kP][C].
 // src(pos) returns the pointer to the C channels of position pos or nullptr (out of range).
@@ -143,6 +148,190 @@ __device__ __forceinline__ void linear_tiles(const float* xs, int ldx, const flo
   }
 }
 
+
+// ---- linear layers with fp32 operands split into three bf16 terms -------------------------------
+// x = xh + xm + xl with xh = bf16(x), xm = bf16(x - xh), xl = bf16(x - xh - xm): both differences are
+// exact in fp32, so the three terms carry 24 significant bits of x.  A product then is
+//     x w = xh wh + xh wm + xm wh + xh wl + xl wh + xm wm + (three terms below 2^-24 |x w|),
+// six bf16 MFMA products (exact, summed in fp32) at a sixteenth of the cost of an fp32 MFMA product each:
+// 2.7 times less matrix time for the accuracy of an fp32 product.  The activations are split once per
+// tile when the LayerNorm writes them to LDS; the weights once per call into the workspace, in the
+// order the MFMA A/B operands are read: the 16 bytes lane l needs for step s of row tile t sit at
+// ((t * steps + s) * 64 + l) * 16, so a wave's operand read is one contiguous kilobyte (read straight
+// from the row-major matrix the same operand touches 32 cache lines, and the passes are bound by that).
+struct Split3 {
+  bf16_t h, m, l;
+};
+__device__ __forceinline__ Split3 split3(float v) {
+  Split3 s;
+  s.h = to_bf16(v);
+  const float r1 = v - bf16_to_f32(s.h);
+  s.m = to_bf16(r1);
+  s.l = to_bf16(r1 - bf16_to_f32(s.m));
+  return s;
+}
+
+// LDS tile of tp positions in three planes [tp][ld] bf16 (ld = K + 8: rows 16 bytes apart in the bank map)
+struct TileX3 {
+  bf16_t* h;
+  int ld, plane;  // plane = tp * ld elements: m = h + plane, l = h + 2 * plane
+  __device__ __forceinline__ void store(int pos, int c, float v) const {
+    const Split3 s = split3(v);
+    h[pos * ld + c] = s.h;
+    h[plane + pos * ld + c] = s.m;
+    h[2 * plane + pos * ld + c] = s.l;
+  }
+};
+__device__ __forceinline__ TileX3 make_tile_x3(void* base, int K, int tp) {
+  TileX3 t;
+  t.h = static_cast<bf16_t*>(base);
+  t.ld = K + 8;
+  t.plane = tp * t.ld;
+  return t;
+}
+__host__ __device__ constexpr size_t tile_bytes_x3(int K, int tp) { return (size_t)3 * tp * (K + 8) * sizeof(bf16_t); }
+
+// split, operand-ordered copy of a weight matrix [rows][K]: three planes of ceil(rows / 32) * 32 * K bf16
+struct WeightX3 {
+  const bf16_t* h;
+  long plane;
+};
+__host__ __device__ constexpr long packed_elems(long rows, long K) { return (rows + 31) / 32 * 32 * K; }
+
+__global__ __launch_bounds__(kThreads) void split_weights_f32(const float* __restrict__ src, bf16_t* __restrict__ dst,
+                                                              int rows, int K) {
+  // one thread per (row tile, step, lane): its 8 consecutive k-values
+  const int steps = K / 16;
+  const long item = (long)blockIdx.x * kThreads + threadIdx.x;
+  const long n_items = (long)((rows + 31) / 32) * steps * 64;
+  if (item >= n_items) return;
+  const int lane = (int)(item & 63), l32 = lane & 31, lh = lane >> 5;
+  const long ts = item >> 6;
+  const int s = (int)(ts % steps), t = (int)(ts / steps);
+  int row = 32 * t + l32;
+  row = row < rows ? row : rows - 1;  // rows past the end repeat the last one (their results are dropped)
+  const long plane = packed_elems(rows, K);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const Split3 v = split3(src[(size_t)row * K + 16 * s + 8 * lh + e]);
+    dst[item * 8 + e] = v.h;
+    dst[plane + item * 8 + e] = v.m;
+    dst[2 * plane + item * 8 + e] = v.l;
+  }
+}
+
+// LayerNorm of 32 * XT positions into a split tile, a row per 32 lanes, at most 256 channels.  A row
+// is read once and kept in registers (the reads of four rows are in flight together); the arithmetic
+// is that of layer_norm_tile.  extra(pos, y) sees the normalised row: lane l holds channels l + 32 e.
+template <int XT, typename Src, typename Extra>
+__device__ __forceinline__ void layer_norm_tile_x3(Src src, const float* __restrict__ w, const float* __restrict__ bsh,
+                                                   int C, const TileX3& t, Extra extra) {
+  constexpr int kGroups = kThreads / 32, ITERS = 32 * XT / kGroups;
+  static_assert(ITERS % 4 == 0, "rows in batches of four");
+  const int l = threadIdx.x & 31, grp = threadIdx.x >> 5;
+  float wv[8], bv[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int c = l + 32 * e;
+    wv[e] = c < C ? w[c] : 0.f;
+    bv[e] = c < C ? bsh[c] : 0.f;
+  }
+  for (int it0 = 0; it0 < ITERS; it0 += 4) {
+    float val[4][8];
+    bool has[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float* row = src(grp + (it0 + u) * kGroups);
+      has[u] = row != nullptr;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) val[u][e] = (row && l + 32 * e < C) ? row[l + 32 * e] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int pos = grp + (it0 + u) * kGroups;
+      float s = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += val[u][e];  // channels past C hold 0
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, 32);
+      const float mean = s / (float)C;
+      float q = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float d = val[u][e] - mean;
+        q += l + 32 * e < C ? d * d : 0.f;
+      }
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 32);
+      const float rstd = 1.0f / sqrtf(q / (float)C + kEps);
+      float y[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        y[e] = has[u] ? (val[u][e] - mean) * rstd * wv[e] + bv[e] : 0.f;
+        if (l + 32 * e < C) t.store(pos, l + 32 * e, y[e]);
+      }
+      extra(pos, y);
+    }
+  }
+}
+struct NoExtra {
+  __device__ __forceinline__ void operator()(int, const float (&)[8]) const {}
+};
+
+// linear_tiles on split operands for XT tiles of 32 positions at once (a weight operand is read once
+// for all of them): K % 16 == 0, o0 a multiple of 32; lane (row or column l32, half lh) supplies the 8
+// consecutive k-values 16 s + 8 lh .. + 7 of step s, one 16-byte read per term and operand.  The
+// result layout of acc[n][xt] is that of linear_tiles for positions 32 xt .. 32 xt + 31.
+template <int NW, int XT, bool OUT_ROWS>
+__device__ __forceinline__ void linear_tiles_x3(const TileX3& xs, const WeightX3 (&W)[NW], int o0, int K,
+                                                f32x16_t (&acc)[NW][XT]) {
+  const int lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int steps = K / 16;
+  const u32x4_t* xh = reinterpret_cast<const u32x4_t*>(xs.h + l32 * xs.ld + 8 * lh);
+  const int xplane = xs.plane / 8, xtile = 32 * xs.ld / 8;  // in 16-byte units
+  const u32x4_t* wh[NW];
+  long wplane[NW];
+#pragma unroll
+  for (int n = 0; n < NW; ++n) {
+    wh[n] = reinterpret_cast<const u32x4_t*>(W[n].h) + (size_t)(o0 >> 5) * steps * 64 + lane;
+    wplane[n] = W[n].plane / 8;
+#pragma unroll
+    for (int xt = 0; xt < XT; ++xt) acc[n][xt] = zero16();
+  }
+  for (int s = 0; s < steps; ++s) {
+    u32x4_t x_h[XT], x_m[XT], x_l[XT];
+#pragma unroll
+    for (int xt = 0; xt < XT; ++xt) {
+      x_h[xt] = xh[xt * xtile + 2 * s];
+      x_m[xt] = xh[xplane + xt * xtile + 2 * s];
+      x_l[xt] = xh[2 * xplane + xt * xtile + 2 * s];
+    }
+#pragma unroll
+    for (int n = 0; n < NW; ++n) {
+      const u32x4_t w_h = wh[n][64 * s], w_m = wh[n][wplane[n] + 64 * s], w_l = wh[n][2 * wplane[n] + 64 * s];
+#pragma unroll
+      for (int xt = 0; xt < XT; ++xt) {
+        // smallest terms first
+        if (OUT_ROWS) {
+          acc[n][xt] = mfma_32x32x16(w_l, x_h[xt], acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(w_h, x_l[xt], acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(w_m, x_m[xt], acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(w_m, x_h[xt], acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(w_h, x_m[xt], acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(w_h, x_h[xt], acc[n][xt]);
+        } else {
+          acc[n][xt] = mfma_32x32x16(x_h[xt], w_l, acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(x_l[xt], w_h, acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(x_m[xt], w_m, acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(x_h[xt], w_m, acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(x_m[xt], w_h, acc[n][xt]);
+          acc[n][xt] = mfma_32x32x16(x_h[xt], w_h, acc[n][xt]);
+        }
+      }
+    }
+  }
+}
+
 // ---- triangle multiplication -----------------------------------------------------------------
 struct TrimulF32 {
   const float *z, *mask;
@@ -150,6 +339,7 @@ struct TrimulF32 {
   PairView zc;              // canonical view (output pass)
   const float *ln_in_w, *ln_in_b, *ln_out_w, *ln_out_b;
   const float *w_ap, *w_ag, *w_bp, *w_bg, *w_g, *w_z;
+  WeightX3 s_ap, s_ag, s_bp, s_bg, s_g, s_z;  // split copies (the *_x3 kernels only)
   float *a, *b, *x, *out;
   int B, N, C, CH, add_residual;
 };
@@ -366,7 +556,7 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_mm_f32(TrimulF32 p, int 
     for (int v = 0; v < 16; ++v) {
       const int c = o0 + acc_row(v, lh);
       // mask * sigmoid(gate) * projection, in the reference's order of multiplication
-      if (c < CH && k < N) dst[(((size_t)b * CH + c) * N + r) * N + k] = m * sigmoid_f32(acc[0][v]) * acc[1][v];
+      if (c < CH && k < N) dst[(((size_t)b * CH + c) * N + r) * N + k] = m * sigmoid_hw_f32(acc[0][v]) * acc[1][v];
     }
   }
 }
@@ -406,11 +596,154 @@ __global__ __launch_bounds__(kThreads) void trimul_out_mm_f32(TrimulF32 p, int g
     for (int v = 0; v < 16; ++v) {
       const int j = j0 + acc_row(v, lh);
       if (co < C && j < N) {
-        float res = lin[0][v] * sigmoid_f32(gate[0][v]);
+        float res = lin[0][v] * sigmoid_hw_f32(gate[0][v]);
         const size_t o = b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k + co;
         if (p.add_residual) res = p.z[o] + res;
         p.out[o] = res;
       }
+    }
+  }
+}
+
+// The same two passes on split operands (channel counts that are multiples of 16), 32 * XT positions
+// per work-group.  WIDE: more than 128 channels on either side (two output tiles per wave).
+template <int XT>
+__global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int groups) {
+  extern __shared__ float smem[];
+  constexpr int TPX = 32 * XT;
+  const int N = p.N, C = p.C, CH = p.CH;
+  const TileX3 xn = make_tile_x3(smem, C, TPX);
+  float* msk = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + tile_bytes_x3(C, TPX));  // [TPX]
+  const int g = blockIdx.x % groups, r = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int k0 = g * TPX;
+  layer_norm_tile_x3<XT>(
+      [&](int pos) -> const float* {
+        const int k = k0 + pos;
+        return k < N ? p.z + b * p.zv.stride_b + r * p.zv.stride_r + k * p.zv.stride_k : nullptr;
+      },
+      p.ln_in_w, p.ln_in_b, C, xn, NoExtra{});
+  if (threadIdx.x < TPX) {
+    const int k = k0 + threadIdx.x;
+    msk[threadIdx.x] = (k < N && p.mask) ? p.mask[b * p.mv.stride_b + r * p.mv.stride_r + k * p.mv.stride_k] : 1.f;
+  }
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int n_ot = (CH + 31) / 32;
+  for (int t = wave; t < 2 * n_ot; t += kThreads / 64) {
+    const int pair = t / n_ot, o0 = 32 * (t - pair * n_ot);
+    const WeightX3 W[2] = {pair ? p.s_bg : p.s_ag, pair ? p.s_bp : p.s_ap};
+    f32x16_t acc[2][XT];
+    linear_tiles_x3<2, XT, true>(xn, W, o0, C, acc);
+    float* dst = pair ? p.b : p.a;
+#pragma unroll
+    for (int xt = 0; xt < XT; ++xt) {
+      const int k = k0 + 32 * xt + l32;
+      const float m = msk[32 * xt + l32];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int c = o0 + acc_row(v, lh);
+        if (c < CH && k < N)
+          dst[(((size_t)b * CH + c) * N + r) * N + k] = m * sigmoid_hw_f32(acc[0][xt][v]) * acc[1][xt][v];
+      }
+    }
+  }
+}
+
+// Output pass.  The gate is computed first and kept in registers, so that LayerNorm(x) can take the
+// place of LayerNorm(z) in LDS.  x is read channel-major straight into registers: thread (position
+// pos = tid % TPX, channel group cg = tid / TPX) holds channels cg + CG e; the statistics of a
+// position are summed over the channel groups through LDS.
+template <int XT, bool WIDE>
+__global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int groups) {
+  extern __shared__ float smem[];
+  constexpr int TPX = 32 * XT, CG = kThreads / TPX, XE = (WIDE ? 256 : 128) / CG, MAXT = WIDE ? 2 : 1;
+  const int N = p.N, C = p.C, CH = p.CH;
+  char* base = reinterpret_cast<char*>(smem);
+  const TileX3 zn = make_tile_x3(base, C, TPX);   // LayerNorm(z), then
+  const TileX3 xo = make_tile_x3(base, CH, TPX);  // LayerNorm(x) in the same memory
+  const size_t tile_max = tile_bytes_x3(C > CH ? C : CH, TPX);
+  float* red_s = reinterpret_cast<float*>(base + tile_max);  // [CG][TPX]
+  float* red_q = red_s + kThreads;                           // [CG][TPX]
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * TPX;
+  const int xpos = threadIdx.x % TPX, cg = threadIdx.x / TPX;
+  const bool xin = j0 + xpos < N;
+  float xv[XE];
+  {
+    const float* xp = p.x + (((size_t)b * CH + cg) * N + i) * N + j0 + xpos;
+#pragma unroll
+    for (int e = 0; e < XE; ++e) xv[e] = (xin && cg + CG * e < CH) ? xp[(size_t)CG * e * N * N] : 0.f;
+  }
+  layer_norm_tile_x3<XT>(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.z + b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k : nullptr;
+      },
+      p.ln_in_w, p.ln_in_b, C, zn, NoExtra{});
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int n_ot = (C + 31) / 32;
+  f32x16_t gate[MAXT][1][XT];
+#pragma unroll
+  for (int u = 0; u < MAXT; ++u) {
+    const int t = wave + u * (kThreads / 64);
+    if (t < n_ot) {
+      const WeightX3 Wg[1] = {p.s_g};
+      linear_tiles_x3<1, XT, false>(zn, Wg, 32 * t, C, gate[u]);
+    }
+  }
+  // LayerNorm over the channels of x
+  {
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < XE; ++e) s += xv[e];
+    red_s[threadIdx.x] = s;
+  }
+  __syncthreads();  // also: every wave has finished reading zn
+  float mean = 0.f;
+#pragma unroll
+  for (int c = 0; c < CG; ++c) mean += red_s[c * TPX + xpos];
+  mean /= (float)CH;
+  {
+    float q = 0.f;
+#pragma unroll
+    for (int e = 0; e < XE; ++e) {
+      const float d = xv[e] - mean;
+      q += cg + CG * e < CH ? d * d : 0.f;
+    }
+    red_q[threadIdx.x] = q;
+  }
+  __syncthreads();
+  float var = 0.f;
+#pragma unroll
+  for (int c = 0; c < CG; ++c) var += red_q[c * TPX + xpos];
+  const float rstd = 1.0f / sqrtf(var / (float)CH + kEps);
+#pragma unroll
+  for (int e = 0; e < XE; ++e) {
+    const int c = cg + CG * e;
+    if (c < CH) xo.store(xpos, c, xin ? (xv[e] - mean) * rstd * p.ln_out_w[c] + p.ln_out_b[c] : 0.f);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < MAXT; ++u) {
+    const int t = wave + u * (kThreads / 64);
+    if (t < n_ot) {
+      const int o0 = 32 * t, co = o0 + l32;
+      const WeightX3 Wz[1] = {p.s_z};
+      f32x16_t lin[1][XT];
+      linear_tiles_x3<1, XT, false>(xo, Wz, o0, CH, lin);
+#pragma unroll
+      for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int j = j0 + 32 * xt + acc_row(v, lh);
+          if (co < C && j < N) {
+            float res = lin[0][xt][v] * sigmoid_hw_f32(gate[u][0][xt][v]);
+            const size_t o = b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k + co;
+            if (p.add_residual) res = p.z[o] + res;
+            p.out[o] = res;
+          }
+        }
     }
   }
 }
@@ -420,6 +753,7 @@ struct TriattnF32 {
   const float *x, *mask;
   PairView xv, mv;
   const float *ln_w, *ln_b, *w_q, *w_k, *w_v, *w_b, *w_g, *w_o;
+  WeightX3 s_q, s_k, s_v, s_b, s_g, s_o;  // split copies (the *_x3 kernels only)
   float *q, *k, *v, *tb, *o, *out;
   int B, N, C, H, D, add_residual;
   float inf;
@@ -527,7 +861,7 @@ __global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int
     for (int v = 0; v < 16; ++v) {
       const int pos = acc_row(v, lh), j = j0 + pos;
       if (hd < HD)
-        og[pos * ldh + hd] = j < N ? p.o[(((size_t)b * N + i) * N + j) * HD + hd] * sigmoid_f32(gate[0][v]) : 0.f;
+        og[pos * ldh + hd] = j < N ? p.o[(((size_t)b * N + i) * N + j) * HD + hd] * sigmoid_hw_f32(gate[0][v]) : 0.f;
     }
   }
   __syncthreads();
@@ -546,6 +880,127 @@ __global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int
         p.out[o] = res;
       }
     }
+  }
+}
+
+// The two position-wise passes of the attention on split operands (channel counts that are multiples
+// of 16), 32 * XT positions per work-group.  The H rows of the triangle bias are too few for a matrix
+// tile: they are fp32 dot products taken on the normalised row while it is in registers.
+template <int XT>
+__global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, int groups) {
+  extern __shared__ float smem[];
+  constexpr int TPX = 32 * XT;
+  const int N = p.N, C = p.C, H = p.H, D = p.D, HD = H * D;
+  const TileX3 xn = make_tile_x3(smem, C, TPX);
+  float* tbs = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + tile_bytes_x3(C, TPX));  // [H][TPX]
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * TPX;
+  const int l = threadIdx.x & 31;
+  layer_norm_tile_x3<XT>(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+      },
+      p.ln_w, p.ln_b, C, xn, [&](int pos, const float(&y)[8]) {
+        for (int h = 0; h < H; ++h) {
+          float d = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (l + 32 * e < C) d += y[e] * p.w_b[h * C + l + 32 * e];
+#pragma unroll
+          for (int o = 16; o > 0; o >>= 1) d += __shfl_xor(d, o, 32);
+          if (l == 0) tbs[h * TPX + pos] = d;
+        }
+      });
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < H * TPX; idx += kThreads) {
+    const int h = idx / TPX, j = j0 + idx % TPX;
+    if (j < N) p.tb[(((size_t)b * H + h) * N + i) * N + j] = tbs[idx];
+  }
+  const float scale = 1.0f / sqrtf((float)D);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  for (int t = wave; t < (HD + 31) / 32; t += kThreads / 64) {
+    const int o0 = 32 * t, hd = o0 + l32, h = hd / D, d = hd - h * D;
+    const WeightX3 W[3] = {p.s_q, p.s_k, p.s_v};
+    f32x16_t acc[3][XT];
+    linear_tiles_x3<3, XT, false>(xn, W, o0, C, acc);
+#pragma unroll
+    for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int j = j0 + 32 * xt + acc_row(v, lh);
+        if (hd < HD && j < N) {
+          const size_t o = ((((size_t)b * N + i) * H + h) * N + j) * D + d;
+          p.q[o] = acc[0][xt][v] * scale;  // q / sqrt(c) after the projection (attention.py:283-284)
+          p.k[o] = acc[1][xt][v];
+          p.v[o] = acc[2][xt][v];
+        }
+      }
+  }
+}
+
+// Output pass: the gate stays in registers until every wave has finished with LayerNorm(x), then the
+// gated attention output takes its place in LDS.
+template <int XT, bool WIDE>
+__global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int groups) {
+  extern __shared__ float smem[];
+  constexpr int TPX = 32 * XT, MAXT = WIDE ? 2 : 1;
+  const int N = p.N, C = p.C, HD = p.H * p.D;
+  const TileX3 xn = make_tile_x3(smem, C, TPX);
+  const TileX3 og = make_tile_x3(smem, HD, TPX);  // gated attention output, in the same memory
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * TPX;
+  layer_norm_tile_x3<XT>(
+      [&](int pos) -> const float* {
+        const int j = j0 + pos;
+        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+      },
+      p.ln_w, p.ln_b, C, xn, NoExtra{});
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int n_gt = (HD + 31) / 32;
+  f32x16_t gate[MAXT][1][XT];
+#pragma unroll
+  for (int u = 0; u < MAXT; ++u) {
+    const int t = wave + u * (kThreads / 64);
+    if (t < n_gt) {
+      const WeightX3 W[1] = {p.s_g};
+      linear_tiles_x3<1, XT, false>(xn, W, 32 * t, C, gate[u]);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < MAXT; ++u) {
+    const int t = wave + u * (kThreads / 64), hd = 32 * t + l32;
+    if (t < n_gt && hd < HD) {
+#pragma unroll
+      for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int pos = 32 * xt + acc_row(v, lh), j = j0 + pos;
+          og.store(pos, hd,
+                   j < N ? p.o[(((size_t)b * N + i) * N + j) * HD + hd] * sigmoid_hw_f32(gate[u][0][xt][v]) : 0.f);
+        }
+    }
+  }
+  __syncthreads();
+  for (int t = wave; t < (C + 31) / 32; t += kThreads / 64) {
+    const int o0 = 32 * t, co = o0 + l32;
+    const WeightX3 W[1] = {p.s_o};
+    f32x16_t acc[1][XT];
+    linear_tiles_x3<1, XT, false>(og, W, o0, HD, acc);
+#pragma unroll
+    for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int j = j0 + 32 * xt + acc_row(v, lh);
+        if (co < C && j < N) {
+          float res = acc[0][xt][v];
+          const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
+          if (p.add_residual) res = p.x[o] + res;
+          p.out[o] = res;
+        }
+      }
   }
 }
 
@@ -791,7 +1246,7 @@ __global__ __launch_bounds__(kThreads) void transition_mm_f32(TransitionF32 p, i
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const float a = acc[0][v];
-          hid[acc_row(v, lh) * ldh + hd] = (a * sigmoid_f32(a)) * acc[1][v];
+          hid[acc_row(v, lh) * ldh + hd] = (a * sigmoid_hw_f32(a)) * acc[1][v];
         }
       }
     }
@@ -929,9 +1384,13 @@ bool aligned16(std::initializer_list<const void*> ptrs) {
 // the largest tiles exceed the default dynamic LDS limit: raised to max_bytes once per device and
 // kernel (slot = index of the kernel's cache)
 constexpr size_t kLdsLimit = 160 * 1024;
+#ifndef OF3_X3_XT
+#define OF3_X3_XT 1
+#endif
+constexpr int kXT = OF3_X3_XT;  // 32-position tiles per work-group of the split-operand passes
 template <typename Kern>
 hipError_t allow_lds(Kern kern, int slot, size_t max_bytes = 3 * (size_t)kTP * (kMaxC + 4) * sizeof(float)) {
-  static int cache[4][kMaxDevices];
+  static int cache[16][kMaxDevices];
   int done = 0;
   return per_device(
       cache[slot],
@@ -1008,7 +1467,34 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
                   aligned16({a.w_ap, a.w_ag, a.w_bp, a.w_bg, a.w_g, a.w_z});
   const int mgroups = (a.N + kTP - 1) / kTP;
   const unsigned mblocks = (unsigned)((long)a.B * a.N * mgroups);
-  if (mm) {
+  // split-operand kernels for the position-wise passes: channel counts in multiples of 16 and room for
+  // the split weights
+  const bool x3 = a.C % 16 == 0 && a.CH % 16 == 0 && a.wsplit && aligned16({a.wsplit});
+  const int xgroups = (a.N + 32 * kXT - 1) / (32 * kXT);
+  const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
+  if (x3) {
+    bf16_t* w = static_cast<bf16_t*>(a.wsplit);
+    auto split = [&](const float* src, int rows, int K, WeightX3& dst) {
+      dst.h = w;
+      dst.plane = packed_elems(rows, K);
+      const long items = dst.plane / 8;
+      hipLaunchKernelGGL(split_weights_f32, dim3((unsigned)((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream,
+                         src, w, rows, K);
+      w += 3 * dst.plane;
+    };
+    split(a.w_ap, a.CH, a.C, p.s_ap);
+    split(a.w_ag, a.CH, a.C, p.s_ag);
+    split(a.w_bp, a.CH, a.C, p.s_bp);
+    split(a.w_bg, a.CH, a.C, p.s_bg);
+    split(a.w_g, a.C, a.C, p.s_g);
+    split(a.w_z, a.C, a.CH, p.s_z);
+    hipError_t e = allow_lds(trimul_proj_x3_f32<kXT>, 4, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, false>, 5, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, true>, 6, kLdsLimit);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(trimul_proj_x3_f32<kXT>, dim3(xblocks), dim3(kThreads),
+                       tile_bytes_x3(a.C, 32 * kXT) + 32 * kXT * sizeof(float), stream, p, xgroups);
+  } else if (mm) {
     hipError_t e = allow_lds(trimul_proj_mm_f32, 0);
     if (e == hipSuccess) e = allow_lds(trimul_out_mm_f32, 1);
     if (e != hipSuccess) return e;
@@ -1019,7 +1505,7 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   }
   // the contraction has no shape or alignment condition of its own; the FMA kernel stays with the
   // FMA passes so that odd shapes run one family of kernels
-  if (mm) {
+  if (mm || x3) {
     const unsigned t = (unsigned)((a.N + 127) / 128);
     hipLaunchKernelGGL(trimul_contract_mm_f32, dim3(t, t, (unsigned)(a.B * a.CH)), dim3(kThreads), 0, stream, p.a, p.b,
                        p.x, a.N);
@@ -1028,7 +1514,14 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
     hipLaunchKernelGGL(trimul_contract_f32, dim3(t, t, (unsigned)(a.B * a.CH)), dim3(kThreads), 0, stream, p.a, p.b,
                        p.x, a.N);
   }
-  if (mm)
+  if (x3) {
+    const size_t lds = tile_bytes_x3(a.C > a.CH ? a.C : a.CH, 32 * kXT) + 2 * kThreads * sizeof(float);
+    if (a.C > 128 || a.CH > 128)
+      hipLaunchKernelGGL((trimul_out_x3_f32<kXT, true>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    else
+      hipLaunchKernelGGL((trimul_out_x3_f32<kXT, false>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+  }
+  else if (mm)
     hipLaunchKernelGGL(trimul_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + 2 * tile_bytes(a.CH), stream,
                        p, mgroups);
   else
@@ -1071,7 +1564,33 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   const bool mm = a.C % 8 == 0 && (a.H * a.D) % 8 == 0 && aligned16({a.w_q, a.w_k, a.w_v, a.w_b, a.w_g, a.w_o});
   const int mgroups = (a.N + kTP - 1) / kTP;
   const unsigned mblocks = (unsigned)((long)a.B * a.N * mgroups);
-  if (mm) {
+  const bool x3 = a.C % 16 == 0 && (a.H * a.D) % 16 == 0 && a.wsplit && aligned16({a.wsplit});
+  const int xgroups = (a.N + 32 * kXT - 1) / (32 * kXT);
+  const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
+  if (x3) {
+    bf16_t* w = static_cast<bf16_t*>(a.wsplit);
+    auto split = [&](const float* src, int rows, int K, WeightX3& dst) {
+      dst.h = w;
+      dst.plane = packed_elems(rows, K);
+      const long items = dst.plane / 8;
+      hipLaunchKernelGGL(split_weights_f32, dim3((unsigned)((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream,
+                         src, w, rows, K);
+      w += 3 * dst.plane;
+    };
+    const int HD = a.H * a.D;
+    split(a.w_q, HD, a.C, p.s_q);
+    split(a.w_k, HD, a.C, p.s_k);
+    split(a.w_v, HD, a.C, p.s_v);
+    split(a.w_g, HD, a.C, p.s_g);
+    split(a.w_o, a.C, HD, p.s_o);
+    split(a.w_b, a.H, a.C, p.s_b);
+    hipError_t e = allow_lds(triattn_proj_x3_f32<kXT>, 7, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, false>, 8, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, true>, 9, kLdsLimit);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(triattn_proj_x3_f32<kXT>, dim3(xblocks), dim3(kThreads),
+                       tile_bytes_x3(a.C, 32 * kXT) + (size_t)a.H * 32 * kXT * sizeof(float), stream, p, xgroups);
+  } else if (mm) {
     hipError_t e = allow_lds(triattn_proj_mm_f32, 2);
     if (e == hipSuccess) e = allow_lds(triattn_out_mm_f32, 3);
     if (e != hipSuccess) return e;
@@ -1087,7 +1606,15 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     hipLaunchKernelGGL(triattn_core_f32<64>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
   else
     return hipErrorInvalidValue;
-  if (mm)
+  if (x3) {
+    const int HD = a.H * a.D;
+    const size_t lds = tile_bytes_x3(a.C > HD ? a.C : HD, 32 * kXT);
+    if (a.C > 128 || HD > 128)
+      hipLaunchKernelGGL((triattn_out_x3_f32<kXT, true>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    else
+      hipLaunchKernelGGL((triattn_out_x3_f32<kXT, false>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+  }
+  else if (mm)
     hipLaunchKernelGGL(triattn_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + tile_bytes(a.H * a.D), stream,
                        p, mgroups);
   else

@@ -102,7 +102,7 @@ def test_trimul_fwd_rejects_bad_arguments(lib):
     assert call(dtype=7) == _lib.OF3_EINVAL                        # unknown dtype code
     # fp32 has its own (larger) workspace and looser shape rules; never call it with a workable argument set here
     need32 = lib.of3_trimul_workspace_bytes_for(_lib.OF3_DTYPE_F32, 1, 64, 128, 128)
-    assert need32 == 3 * 128 * 64 * 64 * 4
+    assert need32 == 3 * 128 * 64 * 64 * 4 + 6 * (5 * 128 * 128 + 128 * 128)  # a, b, x + the weights split in three
     assert call(dtype=_lib.OF3_DTYPE_F32, ws_bytes=need32 - 1) == _lib.OF3_ENOSPC
     assert call(dtype=_lib.OF3_DTYPE_F32, C=300, CH=300) == _lib.OF3_EINVAL
     assert call(dtype=_lib.OF3_DTYPE_F32, z=FAKE + 2, ws_bytes=need32) == _lib.OF3_EINVAL
@@ -128,7 +128,7 @@ def test_triattn_fwd_rejects_bad_arguments(lib):
 
     assert call(dtype=7) == _lib.OF3_EINVAL
     need32 = lib.of3_triattn_workspace_bytes_for(_lib.OF3_DTYPE_F32, 1, 64, 128, 4, 32)
-    assert need32 == 4 * 64 * 64 * 128 * 4 + 4 * 64 * 64 * 4
+    assert need32 == 4 * 64 * 64 * 128 * 4 + 4 * 64 * 64 * 4 + 6 * (5 * 128 * 128 + 32 * 128)  # + the split weights (4 bias rows padded to 32)
     assert call(dtype=_lib.OF3_DTYPE_F32, ws_bytes=need32 - 1) == _lib.OF3_ENOSPC
     assert call(dtype=_lib.OF3_DTYPE_F32, D=24, ws_bytes=need32) == _lib.OF3_EINVAL
     assert call(H=8) == _lib.OF3_EINVAL
