@@ -216,13 +216,19 @@ struct TriattnF32Args {
   float *tb;                         // workspace, [B][H][N][N]
   float *o;                          // workspace, [B][N][N][H*D]
   void* wsplit;                      // workspace, triattn_wsplit_bytes(C, H, D) bytes, 16-byte aligned; may be null
+  void* qkv_split;                   // workspace, triattn_qkv_split_bytes(B, N, H, D) bytes, 16-byte aligned, may
+                                     // overlap q, k, v; may be null
   float* out;
   int B, N, C, H, D, add_residual;
   float inf;
 };
 hipError_t triattn_fwd_f32(const TriattnF32Args& args, hipStream_t stream);
 inline size_t triattn_wsplit_bytes(long C, long H, long D) {
-  return (size_t)6 * (4 * wsplit_elems(H * D, C) + wsplit_elems(C, H * D) + wsplit_elems(H, C));
+  return (size_t)6 * (4 * wsplit_elems(H * D, C) + wsplit_elems(C, H * D));
+}
+// q, k and v^T in three bf16 terms each, rows padded to whole 32-position tiles
+inline size_t triattn_qkv_split_bytes(long B, long N, long H, long D) {
+  return (size_t)18 * B * N * H * ((N + 31) / 32 * 32) * D;
 }
 
 struct TransitionF32Args {

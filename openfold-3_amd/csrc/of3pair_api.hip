@@ -81,6 +81,10 @@ inline bool f32_triattn_dims_ok(int64_t B, int64_t N, int64_t C, int64_t H, int6
   return positions_ok(B, N) && N <= (1 << 16) && C >= 1 && C <= 256 && H >= 1 && (D == 16 || D == 32 || D == 64) &&
          H * D <= 256;
 }
+inline int64_t f32_triattn_qkv_bytes(int64_t B, int64_t N, int64_t H, int64_t D) {
+  const int64_t fp32 = 3 * align256(B * N * N * H * D * 4), split = align256((int64_t)of3::triattn_qkv_split_bytes(B, N, H, D));
+  return fp32 > split ? fp32 : split;
+}
 inline bool f32_strides_ok(const int64_t s[3]) { return s && s[0] >= 0 && s[1] > 0 && s[2] > 0; }
 inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
@@ -323,8 +327,9 @@ int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, 
 int64_t of3_triattn_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
   if (dtype == OF3_DTYPE_BF16) return of3_triattn_workspace_bytes(B, N, C, H, D);
   if (dtype != OF3_DTYPE_F32 || !f32_triattn_dims_ok(B, N, C, H, D)) return OF3_EINVAL;
-  // q, k, v, o, the triangle bias and the weights split into three bf16 terms
-  return 4 * align256(B * N * N * H * D * 4) + align256(B * H * N * N * 4) +
+  // q, k, v (fp32, or split into three bf16 terms in whole 32-position tiles), o, the triangle bias
+  // and the weights split into three bf16 terms
+  return f32_triattn_qkv_bytes(B, N, H, D) + align256(B * N * N * H * D * 4) + align256(B * H * N * N * 4) +
          align256((int64_t)of3::triattn_wsplit_bytes(C, H, D));
 }
 
@@ -437,9 +442,11 @@ int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask
     a.q = reinterpret_cast<float*>(ws);
     a.k = reinterpret_cast<float*>(ws + part);
     a.v = reinterpret_cast<float*>(ws + 2 * part);
-    a.o = reinterpret_cast<float*>(ws + 3 * part);
-    a.tb = reinterpret_cast<float*>(ws + 4 * part);
-    a.wsplit = ws + 4 * part + align256(B * H * N * N * 4);
+    const int64_t qkv = f32_triattn_qkv_bytes(B, N, H, D);
+    a.qkv_split = ws;  // in place of q, k, v
+    a.o = reinterpret_cast<float*>(ws + qkv);
+    a.tb = reinterpret_cast<float*>(ws + qkv + part);
+    a.wsplit = ws + qkv + part + align256(B * H * N * N * 4);
     a.out = static_cast<float*>(out);
     a.B = (int)B;
     a.N = (int)N;

@@ -171,6 +171,21 @@ __device__ __forceinline__ Split3 split3(float v) {
   return s;
 }
 
+// eight values at once, as three MFMA operands of 8 bf16
+__device__ __forceinline__ void split8(const float (&x)[8], u32x4_t& h, u32x4_t& m, u32x4_t& l) {
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float a = x[2 * w], b = x[2 * w + 1];
+    const uint32_t ph = pack_bf16(a, b);
+    const float ra = a - __uint_as_float(ph << 16), rb = b - __uint_as_float(ph & 0xffff0000u);
+    const uint32_t pm = pack_bf16(ra, rb);
+    const float sa = ra - __uint_as_float(pm << 16), sb = rb - __uint_as_float(pm & 0xffff0000u);
+    h[w] = ph;
+    m[w] = pm;
+    l[w] = pack_bf16(sa, sb);
+  }
+}
+
 // LDS tile of tp positions in three planes [tp][ld] bf16 (ld = K + 8: rows 16 bytes apart in the bank map)
 struct TileX3 {
   bf16_t* h;
@@ -753,8 +768,14 @@ struct TriattnF32 {
   const float *x, *mask;
   PairView xv, mv;
   const float *ln_w, *ln_b, *w_q, *w_k, *w_v, *w_b, *w_g, *w_o;
-  WeightX3 s_q, s_k, s_v, s_b, s_g, s_o;  // split copies (the *_x3 kernels only)
+  WeightX3 s_q, s_k, s_v, s_g, s_o;  // split copies (the *_x3 kernels only)
   float *q, *k, *v, *tb, *o, *out;
+  // q, k and v^T split into three bf16 terms and stored as MFMA operands (the split-operand core only):
+  // the 16 bytes of lane l for step s of 32-position tile t of (b, i, h) are slot
+  // (((b N + i) H + h) * Jp / 32 + t) * 2 + s) * 64 + l of a plane, planes qkv_plane elements apart
+  bf16_t *qs, *ks, *vs;
+  long qkv_plane;
+  int Jp;  // N rounded up to whole 32-position tiles
   int B, N, C, H, D, add_residual;
   float inf;
 };
@@ -886,7 +907,13 @@ __global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int
 // The two position-wise passes of the attention on split operands (channel counts that are multiples
 // of 16), 32 * XT positions per work-group.  The H rows of the triangle bias are too few for a matrix
 // tile: they are fp32 dot products taken on the normalised row while it is in registers.
-template <int XT>
+// SPLIT (head width 32): q, k and v leave as operands of the split-operand core instead of fp32 arrays.
+// A 32-column tile of the projections is one head.  q and k are computed with the head channels in
+// the accumulator rows and the positions in the lanes, v the other way round: in both cases registers
+// 8 s .. 8 s + 7 of a lane are its operand for step s (q, k: head channels 16 s + 4 lh + r and
+// 16 s + 8 + 4 lh + r, the same for both, so the order inside the dot product does not matter;
+// v: the keys the core's S^T accumulator holds in the same registers).
+template <int XT, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, int groups) {
   extern __shared__ float smem[];
   constexpr int TPX = 32 * XT;
@@ -920,22 +947,61 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
   const float scale = 1.0f / sqrtf((float)D);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
   for (int t = wave; t < (HD + 31) / 32; t += kThreads / 64) {
-    const int o0 = 32 * t, hd = o0 + l32, h = hd / D, d = hd - h * D;
-    const WeightX3 W[3] = {p.s_q, p.s_k, p.s_v};
-    f32x16_t acc[3][XT];
-    linear_tiles_x3<3, XT, false>(xn, W, o0, C, acc);
+    const int o0 = 32 * t;
+    if (SPLIT) {
+      // positions past N were normalised to zero rows: their q, k and v are zeros, and are stored
+      const size_t slot0 = ((((size_t)b * N + i) * H + t) * (p.Jp / 32) + j0 / 32) * 128 + lane;
+      const long plane = p.qkv_plane / 8;
+      auto store = [&](bf16_t* dst, const f32x16_t& acc, int xt, float mul) {
+        if (j0 + 32 * xt >= p.Jp) return;  // a tile past the padded row (XT > 1 only)
+        u32x4_t* d4 = reinterpret_cast<u32x4_t*>(dst) + slot0 + xt * 128;
 #pragma unroll
-    for (int xt = 0; xt < XT; ++xt)
+        for (int st = 0; st < 2; ++st) {
+          float x[8];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int j = j0 + 32 * xt + acc_row(v, lh);
-        if (hd < HD && j < N) {
-          const size_t o = ((((size_t)b * N + i) * H + h) * N + j) * D + d;
-          p.q[o] = acc[0][xt][v] * scale;  // q / sqrt(c) after the projection (attention.py:283-284)
-          p.k[o] = acc[1][xt][v];
-          p.v[o] = acc[2][xt][v];
+          for (int e = 0; e < 8; ++e) x[e] = acc[8 * st + e] * mul;
+          u32x4_t h, m, lo;
+          split8(x, h, m, lo);
+          d4[st * 64] = h;
+          d4[plane + st * 64] = m;
+          d4[2 * plane + st * 64] = lo;
+        }
+      };
+      {
+        const WeightX3 W[2] = {p.s_q, p.s_k};
+        f32x16_t acc[2][XT];
+        linear_tiles_x3<2, XT, true>(xn, W, o0, C, acc);
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt) {
+          store(p.qs, acc[0][xt], xt, scale);  // q / sqrt(c) after the projection (attention.py:283-284)
+          store(p.ks, acc[1][xt], xt, 1.f);
         }
       }
+      {
+        const WeightX3 W[1] = {p.s_v};
+        f32x16_t acc[1][XT];
+        linear_tiles_x3<1, XT, false>(xn, W, o0, C, acc);
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt) store(p.vs, acc[0][xt], xt, 1.f);
+      }
+    } else {
+      const int hd = o0 + l32, h = hd / D, d = hd - h * D;
+      const WeightX3 W[3] = {p.s_q, p.s_k, p.s_v};
+      f32x16_t acc[3][XT];
+      linear_tiles_x3<3, XT, false>(xn, W, o0, C, acc);
+#pragma unroll
+      for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int j = j0 + 32 * xt + acc_row(v, lh);
+          if (hd < HD && j < N) {
+            const size_t o = ((((size_t)b * N + i) * H + h) * N + j) * D + d;
+            p.q[o] = acc[0][xt][v] * scale;  // q / sqrt(c) after the projection (attention.py:283-284)
+            p.k[o] = acc[1][xt][v];
+            p.v[o] = acc[2][xt][v];
+          }
+        }
+    }
   }
 }
 
@@ -1001,6 +1067,201 @@ __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int
           p.out[o] = res;
         }
       }
+  }
+}
+
+// Attention core on split operands, head width 32.  Work-group = 8 waves = 4 consecutive rows i x 2
+// halves of one (head, 128-query range); a wave owns 64 queries (two 32-query tiles) of one row.
+//   S^T = K Q^T  (rows = keys, columns = queries), six bf16 products per k-step, started from the
+//                triangle bias: the accumulator is loaded with it, and the mask bias is added after
+//   O^T = V^T P^T, the weights split in registers straight from the S^T accumulator into B operands
+// Per 32-key tile the work-group brings in the bias slice of its query range (it does not depend on
+// i: shared by the four rows) and each row's K and V^T operands (shared by the row's two waves),
+// global -> registers one tile ahead, registers -> the idle half of a double buffer in LDS, one
+// barrier per tile.  Online softmax; the mask bias carries -inf for keys past N.
+constexpr int kXRows = 4;
+constexpr int kXTbLd = 36;  // floats per query row of the bias slice: 16-byte reads of 16 lanes cover all banks
+constexpr size_t kCoreX3Lds = 2 * 128 * kXTbLd * sizeof(float) + 2 * kXRows * 12 * 64 * 16 + 2 * kXRows * 32 * sizeof(float);
+
+__global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_qc, int n_rg, int total, int per_xcd) {
+  constexpr int QT = 2;
+  extern __shared__ u32x4_t lds4[];
+  float* tb_lds = reinterpret_cast<float*>(lds4);           // [2][128][kXTbLd]
+  u32x4_t* kv_lds = lds4 + 2 * 128 * kXTbLd / 4;            // [2][kXRows][12][64]: K step 0, 1 (h m l each), V^T step 0, 1
+  float* mb_lds = reinterpret_cast<float*>(kv_lds + 2 * kXRows * 12 * 64);  // [2][kXRows][32]
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int row = wave >> 1, qh = wave & 1;
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int N = p.N, H = p.H, nt = p.Jp / 32;
+  const int logical = xcd_logical_block(blockIdx.x, per_xcd);
+  if (logical >= total) return;  // the whole work-group leaves together
+  const int qc = logical % n_qc, rg = (logical / n_qc) % n_rg, bh = logical / (n_qc * n_rg);
+  const int i_raw = rg * kXRows + row;
+  const bool row_valid = i_raw < N;  // wave-uniform; idle waves still take part in the loads and barriers
+  const int i = row_valid ? i_raw : N - 1;
+  const int b = bh / H, h = bh % H;
+  const int q0 = qc * 128 + 64 * qh;
+  const size_t bih = ((size_t)b * N + i) * H + h;
+  const long plane = p.qkv_plane / 8;  // in 16-byte slots
+  const u32x4_t* Q = reinterpret_cast<const u32x4_t*>(p.qs) + bih * nt * 128 + lane;
+  // this wave's share of its row's tile: the K operands (first wave of the row) or the V^T operands
+  const u32x4_t* KV = reinterpret_cast<const u32x4_t*>(qh ? p.vs : p.ks) + bih * nt * 128 + lane;
+  const float* tbp = p.tb + ((size_t)b * H + h) * N * N;
+  const int nkt = (N + 31) / 32;
+
+  u32x4_t qop[QT][2][3];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int jt = q0 / 32 + qt < nt ? q0 / 32 + qt : nt - 1;  // tiles past the end: computed, not stored
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int pl = 0; pl < 3; ++pl) qop[qt][st][pl] = Q[pl * plane + (jt * 2 + st) * 64];
+  }
+
+  u32x4_t kv_r[6];
+  float tb_r[2][4];
+  float mb_r = 0.f;
+  const bool tb_vec = (N & 3) == 0;  // rows of the bias are 16-byte aligned
+  auto fetch = [&](int kt) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int pl = 0; pl < 3; ++pl) kv_r[st * 3 + pl] = KV[pl * plane + (kt * 2 + st) * 64];
+    // bias slice [128 queries][32 keys] in 16-byte chunks: thread t takes chunks t and t + 512
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int chunk = tid + 512 * u, q = qc * 128 + (chunk >> 3), k = kt * 32 + 4 * (chunk & 7);
+      const float* src = tbp + (size_t)q * N + k;
+      if (tb_vec) {
+        const float4 v = (q < N && k < N) ? *reinterpret_cast<const float4*>(src) : make_float4(0.f, 0.f, 0.f, 0.f);
+        tb_r[u][0] = v.x, tb_r[u][1] = v.y, tb_r[u][2] = v.z, tb_r[u][3] = v.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) tb_r[u][e] = (q < N && k + e < N) ? src[e] : 0.f;
+      }
+    }
+    if (qh == 0 && lane < 32) {
+      const int k = kt * 32 + lane;
+      float mv = 1.f;
+      if (k < N && p.mask) mv = p.mask[b * p.mv.stride_b + i * p.mv.stride_r + k * p.mv.stride_k];
+      mb_r = k < N ? p.inf * (mv - 1.f) : -__builtin_inff();
+    }
+  };
+  auto stash = [&](int buf) {
+    u32x4_t* kvb = kv_lds + ((buf * kXRows + row) * 12 + 6 * qh) * 64 + lane;
+#pragma unroll
+    for (int e = 0; e < 6; ++e) kvb[e * 64] = kv_r[e];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int chunk = tid + 512 * u;
+      *reinterpret_cast<float4*>(tb_lds + (buf * 128 + (chunk >> 3)) * kXTbLd + 4 * (chunk & 7)) =
+          make_float4(tb_r[u][0], tb_r[u][1], tb_r[u][2], tb_r[u][3]);
+    }
+    if (qh == 0 && lane < 32) mb_lds[(buf * kXRows + row) * 32 + lane] = mb_r;
+  };
+
+  f32x16_t oacc[QT];
+  float m_run[QT], l_run[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    oacc[qt] = zero16();
+    m_run[qt] = -__builtin_inff();
+    l_run[qt] = 0.f;
+  }
+
+  fetch(0);
+  stash(0);
+  if (nkt > 1) fetch(1);
+  __syncthreads();
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int buf = kt & 1;
+    const u32x4_t* kvb = kv_lds + (buf * kXRows + row) * 12 * 64 + lane;
+    u32x4_t kop[2][3];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int pl = 0; pl < 3; ++pl) kop[st][pl] = kvb[(st * 3 + pl) * 64];
+    float mbv[16];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const float4 v = *reinterpret_cast<const float4*>(mb_lds + (buf * kXRows + row) * 32 + 8 * a + 4 * lh);
+      mbv[4 * a] = v.x, mbv[4 * a + 1] = v.y, mbv[4 * a + 2] = v.z, mbv[4 * a + 3] = v.w;
+    }
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      f32x16_t s;
+      const float* tbl = tb_lds + (buf * 128 + 64 * qh + 32 * qt + l32) * kXTbLd + 4 * lh;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const float4 v = *reinterpret_cast<const float4*>(tbl + 8 * a);
+        s[4 * a] = v.x, s[4 * a + 1] = v.y, s[4 * a + 2] = v.z, s[4 * a + 3] = v.w;
+      }
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {  // smallest terms first
+        s = mfma_32x32x16(kop[st][2], qop[qt][st][0], s);
+        s = mfma_32x32x16(kop[st][0], qop[qt][st][2], s);
+        s = mfma_32x32x16(kop[st][1], qop[qt][st][1], s);
+        s = mfma_32x32x16(kop[st][1], qop[qt][st][0], s);
+        s = mfma_32x32x16(kop[st][0], qop[qt][st][1], s);
+        s = mfma_32x32x16(kop[st][0], qop[qt][st][0], s);
+      }
+      float cmax = -__builtin_inff();
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        s[v] += mbv[v];
+        cmax = fmaxf(cmax, s[v]);
+      }
+      cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));  // the other half of the query's keys
+      const float m_new = fmaxf(m_run[qt], cmax);    // finite: every tile holds a key below N
+      const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_new) * kLog2eF32);
+      m_run[qt] = m_new;
+      float lsum = 0.f;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        s[v] = __builtin_amdgcn_exp2f((s[v] - m_new) * kLog2eF32);
+        lsum += s[v];
+      }
+      l_run[qt] = l_run[qt] * alpha + lsum;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) oacc[qt][v] *= alpha;
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = s[8 * st + e];
+        u32x4_t ph, pm, pl;
+        split8(x, ph, pm, pl);
+        const u32x4_t vh = kvb[(6 + st * 3) * 64], vm = kvb[(7 + st * 3) * 64], vl = kvb[(8 + st * 3) * 64];
+        oacc[qt] = mfma_32x32x16(vl, ph, oacc[qt]);
+        oacc[qt] = mfma_32x32x16(vh, pl, oacc[qt]);
+        oacc[qt] = mfma_32x32x16(vm, pm, oacc[qt]);
+        oacc[qt] = mfma_32x32x16(vm, ph, oacc[qt]);
+        oacc[qt] = mfma_32x32x16(vh, pm, oacc[qt]);
+        oacc[qt] = mfma_32x32x16(vh, ph, oacc[qt]);
+      }
+    }
+    if (kt + 1 < nkt) {
+      stash(buf ^ 1);
+      if (kt + 2 < nkt) fetch(kt + 2);
+    }
+    __syncthreads();
+  }
+
+  if (row_valid) {
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      const int q = q0 + 32 * qt + l32;
+      const float l_tot = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
+      if (q >= N) continue;
+      const float inv = 1.0f / l_tot;
+      float* dst = p.o + ((((size_t)b * N + i) * N + q) * H + h) * 32 + 4 * lh;
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+        *reinterpret_cast<float4*>(dst + 8 * a) = make_float4(oacc[qt][4 * a] * inv, oacc[qt][4 * a + 1] * inv,
+                                                              oacc[qt][4 * a + 2] * inv, oacc[qt][4 * a + 3] * inv);
+    }
   }
 }
 
@@ -1565,6 +1826,13 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   const int mgroups = (a.N + kTP - 1) / kTP;
   const unsigned mblocks = (unsigned)((long)a.B * a.N * mgroups);
   const bool x3 = a.C % 16 == 0 && (a.H * a.D) % 16 == 0 && a.wsplit && aligned16({a.wsplit});
+  // head width 32: q, k and v leave the projection pass as split operands of the split-operand core
+  const bool core_x3 = x3 && a.D == 32 && a.qkv_split && aligned16({a.qkv_split});
+  p.Jp = (a.N + 31) / 32 * 32;
+  p.qkv_plane = (long)a.B * a.N * a.H * p.Jp * 32;
+  p.qs = static_cast<bf16_t*>(a.qkv_split);
+  p.ks = p.qs + 3 * p.qkv_plane;
+  p.vs = p.qs + 6 * p.qkv_plane;
   const int xgroups = (a.N + 32 * kXT - 1) / (32 * kXT);
   const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
   if (x3) {
@@ -1583,13 +1851,17 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     split(a.w_v, HD, a.C, p.s_v);
     split(a.w_g, HD, a.C, p.s_g);
     split(a.w_o, a.C, HD, p.s_o);
-    split(a.w_b, a.H, a.C, p.s_b);
-    hipError_t e = allow_lds(triattn_proj_x3_f32<kXT>, 7, kLdsLimit);
+    hipError_t e = allow_lds(triattn_proj_x3_f32<kXT, false>, 7, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, true>, 10, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, false>, 8, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, true>, 9, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_core_x3_f32, 0, kLdsLimit);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(triattn_proj_x3_f32<kXT>, dim3(xblocks), dim3(kThreads),
-                       tile_bytes_x3(a.C, 32 * kXT) + (size_t)a.H * 32 * kXT * sizeof(float), stream, p, xgroups);
+    const size_t lds = tile_bytes_x3(a.C, 32 * kXT) + (size_t)a.H * 32 * kXT * sizeof(float);
+    if (core_x3)
+      hipLaunchKernelGGL((triattn_proj_x3_f32<kXT, true>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    else
+      hipLaunchKernelGGL((triattn_proj_x3_f32<kXT, false>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
   } else if (mm) {
     hipError_t e = allow_lds(triattn_proj_mm_f32, 2);
     if (e == hipSuccess) e = allow_lds(triattn_out_mm_f32, 3);
@@ -1598,7 +1870,14 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   } else {
     hipLaunchKernelGGL(triattn_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
   }
-  if (a.D == 32)
+  if (core_x3) {
+    const int n_qc = (a.N + 127) / 128, n_rg = (a.N + kXRows - 1) / kXRows;
+    const long total = (long)n_qc * n_rg * a.B * a.H;
+    if (total > 0x7fffffffL - 8) return hipErrorInvalidValue;
+    const int per_xcd = (int)((total + 7) / 8);
+    hipLaunchKernelGGL(triattn_core_x3_f32, dim3(per_xcd * 8), dim3(512), kCoreX3Lds, stream, p, n_qc, n_rg, (int)total,
+                       per_xcd);
+  } else if (a.D == 32)
     hipLaunchKernelGGL(triattn_core_f32<32>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
   else if (a.D == 16)
     hipLaunchKernelGGL(triattn_core_f32<16>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);

@@ -47,7 +47,8 @@ def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
 @pytest.mark.parametrize("starting", [True, False])
 @pytest.mark.parametrize("c,d,heads,n,batch,masked", [(128, 32, 4, 64, (1,), False), (64, 16, 4, 45, (2,), True),
                                                      (48, 64, 2, 37, (), True), (36, 16, 3, 21, (), True),
-                                                     (64, 32, 2, 150, (), True)])  # more than one 128-query group
+                                                     (64, 32, 2, 150, (), True),  # more than one 128-query group
+                                                     (128, 32, 4, 44, (2,), True), (32, 32, 1, 129, (), False)])
 def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
     lib()
     gen = torch.Generator().manual_seed(400 + n)
