@@ -196,6 +196,17 @@ struct TileX3 {
     h[plane + pos * ld + c] = s.m;
     h[2 * plane + pos * ld + c] = s.l;
   }
+  // two adjacent channels c (even) and c + 1 in one 4-byte write per plane
+  __device__ __forceinline__ void store2(int pos, int c, float v0, float v1) const {
+    const uint32_t ph = pack_bf16(v0, v1);
+    const float r0 = v0 - __uint_as_float(ph << 16), r1 = v1 - __uint_as_float(ph & 0xffff0000u);
+    const uint32_t pm = pack_bf16(r0, r1);
+    const float s0 = r0 - __uint_as_float(pm << 16), s1 = r1 - __uint_as_float(pm & 0xffff0000u);
+    uint32_t* d = reinterpret_cast<uint32_t*>(h + pos * ld + c);
+    d[0] = ph;
+    d[plane / 2] = pm;
+    d[plane] = pack_bf16(s0, s1);
+  }
 };
 __device__ __forceinline__ TileX3 make_tile_x3(void* base, int K, int tp) {
   TileX3 t;
@@ -235,21 +246,29 @@ __global__ __launch_bounds__(kThreads) void split_weights_f32(const float* __res
   }
 }
 
-// LayerNorm of 32 * XT positions into a split tile, a row per 32 lanes, at most 256 channels.  A row
-// is read once and kept in registers (the reads of four rows are in flight together); the arithmetic
-// is that of layer_norm_tile.  extra(pos, y) sees the normalised row: lane l holds channels l + 32 e.
-template <int XT, typename Src, typename Extra>
+// LayerNorm of 32 * XT positions into a split tile, a row per 32 lanes, at most 256 channels (a
+// multiple of 16).  Lane l holds channels 2 l + 64 e and 2 l + 64 e + 1, e < 4.  A row is read once
+// and kept in registers (the reads of four rows are in flight together).  extra(pos, y) sees the
+// normalised row: y[2 e + i] is channel 2 l + 64 e + i.
+// FAST: the channel count is a multiple of 64 (whole wave-uniform steps instead of lane masks) and
+// the rows are 8-byte aligned (one read per pair).
+template <int XT, bool FAST, typename Src, typename Extra>
 __device__ __forceinline__ void layer_norm_tile_x3(Src src, const float* __restrict__ w, const float* __restrict__ bsh,
                                                    int C, const TileX3& t, Extra extra) {
   constexpr int kGroups = kThreads / 32, ITERS = 32 * XT / kGroups;
   static_assert(ITERS % 4 == 0, "rows in batches of four");
   const int l = threadIdx.x & 31, grp = threadIdx.x >> 5;
+  const int nE = C / 64;
+  auto ok = [&](int e) { return FAST ? e < nE : 2 * l + 64 * e < C; };
   float wv[8], bv[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int c = l + 32 * e;
-    wv[e] = c < C ? w[c] : 0.f;
-    bv[e] = c < C ? bsh[c] : 0.f;
+  for (int e = 0; e < 4; ++e) {
+    const int c = 2 * l + 64 * e;
+    wv[2 * e] = wv[2 * e + 1] = bv[2 * e] = bv[2 * e + 1] = 0.f;
+    if (ok(e)) {
+      wv[2 * e] = w[c], wv[2 * e + 1] = w[c + 1];
+      bv[2 * e] = bsh[c], bv[2 * e + 1] = bsh[c + 1];
+    }
   }
   for (int it0 = 0; it0 < ITERS; it0 += 4) {
     float val[4][8];
@@ -259,7 +278,17 @@ __device__ __forceinline__ void layer_norm_tile_x3(Src src, const float* __restr
       const float* row = src(grp + (it0 + u) * kGroups);
       has[u] = row != nullptr;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) val[u][e] = (row && l + 32 * e < C) ? row[l + 32 * e] : 0.f;
+      for (int e = 0; e < 4; ++e) {
+        val[u][2 * e] = val[u][2 * e + 1] = 0.f;
+        if (row && ok(e)) {
+          if (FAST) {
+            const float2 v = *reinterpret_cast<const float2*>(row + 2 * l + 64 * e);
+            val[u][2 * e] = v.x, val[u][2 * e + 1] = v.y;
+          } else {
+            val[u][2 * e] = row[2 * l + 64 * e], val[u][2 * e + 1] = row[2 * l + 64 * e + 1];
+          }
+        }
+      }
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -272,18 +301,21 @@ __device__ __forceinline__ void layer_norm_tile_x3(Src src, const float* __restr
       const float mean = s / (float)C;
       float q = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float d = val[u][e] - mean;
-        q += l + 32 * e < C ? d * d : 0.f;
-      }
+      for (int e = 0; e < 4; ++e)
+        if (ok(e)) {
+          const float d0 = val[u][2 * e] - mean, d1 = val[u][2 * e + 1] - mean;
+          q += d0 * d0;
+          q += d1 * d1;
+        }
 #pragma unroll
       for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 32);
       const float rstd = 1.0f / sqrtf(q / (float)C + kEps);
       float y[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        y[e] = has[u] ? (val[u][e] - mean) * rstd * wv[e] + bv[e] : 0.f;
-        if (l + 32 * e < C) t.store(pos, l + 32 * e, y[e]);
+      for (int e = 0; e < 4; ++e) {
+        y[2 * e] = has[u] ? (val[u][2 * e] - mean) * rstd * wv[2 * e] + bv[2 * e] : 0.f;
+        y[2 * e + 1] = has[u] ? (val[u][2 * e + 1] - mean) * rstd * wv[2 * e + 1] + bv[2 * e + 1] : 0.f;
+        if (ok(e)) t.store2(pos, 2 * l + 64 * e, y[2 * e], y[2 * e + 1]);
       }
       extra(pos, y);
     }
@@ -621,8 +653,10 @@ __global__ __launch_bounds__(kThreads) void trimul_out_mm_f32(TrimulF32 p, int g
 }
 
 // The same two passes on split operands (channel counts that are multiples of 16), 32 * XT positions
-// per work-group.  WIDE: more than 128 channels on either side (two output tiles per wave).
-template <int XT>
+// per work-group.  WIDE: more than 128 channels on either side (two output tiles per wave).  FAST:
+// channel counts in multiples of 64 and 8-byte aligned rows; a work-group whose positions all lie
+// below N then stores without lane conditions, from one address per lane plus wave-uniform offsets.
+template <int XT, bool FAST>
 __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int groups) {
   extern __shared__ float smem[];
   constexpr int TPX = 32 * XT;
@@ -631,7 +665,8 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
   float* msk = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + tile_bytes_x3(C, TPX));  // [TPX]
   const int g = blockIdx.x % groups, r = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
   const int k0 = g * TPX;
-  layer_norm_tile_x3<XT>(
+  const bool whole = k0 + TPX <= N;
+  layer_norm_tile_x3<XT, FAST>(
       [&](int pos) -> const float* {
         const int k = k0 + pos;
         return k < N ? p.z + b * p.zv.stride_b + r * p.zv.stride_r + k * p.zv.stride_k : nullptr;
@@ -642,8 +677,10 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
     msk[threadIdx.x] = (k < N && p.mask) ? p.mask[b * p.mv.stride_b + r * p.mv.stride_r + k * p.mv.stride_k] : 1.f;
   }
   __syncthreads();
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
+            lh = lane >> 5;
   const int n_ot = (CH + 31) / 32;
+  const size_t NN = (size_t)N * N;
   for (int t = wave; t < 2 * n_ot; t += kThreads / 64) {
     const int pair = t / n_ot, o0 = 32 * (t - pair * n_ot);
     const WeightX3 W[2] = {pair ? p.s_bg : p.s_ag, pair ? p.s_bp : p.s_ap};
@@ -654,11 +691,18 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
     for (int xt = 0; xt < XT; ++xt) {
       const int k = k0 + 32 * xt + l32;
       const float m = msk[32 * xt + l32];
+      if (FAST && whole) {
+        float* lp = dst + (((size_t)b * CH + o0) * N + r) * N + (size_t)(4 * lh) * NN + k;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int c = o0 + acc_row(v, lh);
-        if (c < CH && k < N)
-          dst[(((size_t)b * CH + c) * N + r) * N + k] = m * sigmoid_hw_f32(acc[0][xt][v]) * acc[1][xt][v];
+        for (int v = 0; v < 16; ++v)
+          lp[(size_t)(8 * (v >> 2) + (v & 3)) * NN] = m * sigmoid_hw_f32(acc[0][xt][v]) * acc[1][xt][v];
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int c = o0 + acc_row(v, lh);
+          if (c < CH && k < N)
+            dst[(((size_t)b * CH + c) * N + r) * N + k] = m * sigmoid_hw_f32(acc[0][xt][v]) * acc[1][xt][v];
+        }
       }
     }
   }
@@ -666,12 +710,12 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
 
 // Output pass.  The gate is computed first and kept in registers, so that LayerNorm(x) can take the
 // place of LayerNorm(z) in LDS.  x is read channel-major straight into registers: thread (position
-// pos = tid % TPX, channel group cg = tid / TPX) holds channels cg + CG e; the statistics of a
-// position are summed over the channel groups through LDS.
-template <int XT, bool WIDE>
+// pos = tid % TPX, channel group cg = tid / TPX) holds the channel pairs 2 cg + 2 CG e, + 1; the
+// statistics of a position are summed over the channel groups through LDS.
+template <int XT, bool WIDE, bool FAST>
 __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int groups) {
   extern __shared__ float smem[];
-  constexpr int TPX = 32 * XT, CG = kThreads / TPX, XE = (WIDE ? 256 : 128) / CG, MAXT = WIDE ? 2 : 1;
+  constexpr int TPX = 32 * XT, CG = kThreads / TPX, XP = (WIDE ? 128 : 64) / CG, MAXT = WIDE ? 2 : 1;
   const int N = p.N, C = p.C, CH = p.CH;
   char* base = reinterpret_cast<char*>(smem);
   const TileX3 zn = make_tile_x3(base, C, TPX);   // LayerNorm(z), then
@@ -681,22 +725,29 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
   float* red_q = red_s + kThreads;                           // [CG][TPX]
   const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
   const int j0 = g * TPX;
+  const bool whole = j0 + TPX <= N;
   const int xpos = threadIdx.x % TPX, cg = threadIdx.x / TPX;
   const bool xin = j0 + xpos < N;
-  float xv[XE];
+  const size_t NN = (size_t)N * N;
+  float xv[2 * XP];
   {
-    const float* xp = p.x + (((size_t)b * CH + cg) * N + i) * N + j0 + xpos;
+    const float* xp = p.x + (((size_t)b * CH + 2 * cg) * N + i) * N + j0 + xpos;
 #pragma unroll
-    for (int e = 0; e < XE; ++e) xv[e] = (xin && cg + CG * e < CH) ? xp[(size_t)CG * e * N * N] : 0.f;
+    for (int e = 0; e < XP; ++e) {
+      const bool in = xin && 2 * cg + 2 * CG * e < CH;
+      xv[2 * e] = in ? xp[(size_t)(2 * CG * e) * NN] : 0.f;
+      xv[2 * e + 1] = in ? xp[(size_t)(2 * CG * e + 1) * NN] : 0.f;
+    }
   }
-  layer_norm_tile_x3<XT>(
+  layer_norm_tile_x3<XT, FAST>(
       [&](int pos) -> const float* {
         const int j = j0 + pos;
         return j < N ? p.z + b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k : nullptr;
       },
       p.ln_in_w, p.ln_in_b, C, zn, NoExtra{});
   __syncthreads();
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
+            lh = lane >> 5;
   const int n_ot = (C + 31) / 32;
   f32x16_t gate[MAXT][1][XT];
 #pragma unroll
@@ -711,7 +762,7 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
   {
     float s = 0.f;
 #pragma unroll
-    for (int e = 0; e < XE; ++e) s += xv[e];
+    for (int e = 0; e < 2 * XP; ++e) s += xv[e];
     red_s[threadIdx.x] = s;
   }
   __syncthreads();  // also: every wave has finished reading zn
@@ -722,10 +773,12 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
   {
     float q = 0.f;
 #pragma unroll
-    for (int e = 0; e < XE; ++e) {
-      const float d = xv[e] - mean;
-      q += cg + CG * e < CH ? d * d : 0.f;
-    }
+    for (int e = 0; e < XP; ++e)
+      if (2 * cg + 2 * CG * e < CH) {
+        const float d0 = xv[2 * e] - mean, d1 = xv[2 * e + 1] - mean;
+        q += d0 * d0;
+        q += d1 * d1;
+      }
     red_q[threadIdx.x] = q;
   }
   __syncthreads();
@@ -734,9 +787,11 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
   for (int c = 0; c < CG; ++c) var += red_q[c * TPX + xpos];
   const float rstd = 1.0f / sqrtf(var / (float)CH + kEps);
 #pragma unroll
-  for (int e = 0; e < XE; ++e) {
-    const int c = cg + CG * e;
-    if (c < CH) xo.store(xpos, c, xin ? (xv[e] - mean) * rstd * p.ln_out_w[c] + p.ln_out_b[c] : 0.f);
+  for (int e = 0; e < XP; ++e) {
+    const int c = 2 * cg + 2 * CG * e;
+    if (c < CH)
+      xo.store2(xpos, c, xin ? (xv[2 * e] - mean) * rstd * p.ln_out_w[c] + p.ln_out_b[c] : 0.f,
+                xin ? (xv[2 * e + 1] - mean) * rstd * p.ln_out_w[c + 1] + p.ln_out_b[c + 1] : 0.f);
   }
   __syncthreads();
 #pragma unroll
@@ -748,17 +803,31 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
       f32x16_t lin[1][XT];
       linear_tiles_x3<1, XT, false>(xo, Wz, o0, CH, lin);
 #pragma unroll
-      for (int xt = 0; xt < XT; ++xt)
+      for (int xt = 0; xt < XT; ++xt) {
+        if (FAST && whole) {
+          const size_t lo = b * p.zc.stride_b + i * p.zc.stride_r + (size_t)(j0 + 32 * xt + 4 * lh) * p.zc.stride_k + co;
+          const float* zp = p.z + lo;
+          float* op = p.out + lo;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int j = j0 + 32 * xt + acc_row(v, lh);
-          if (co < C && j < N) {
+          for (int v = 0; v < 16; ++v) {
+            const size_t vo = (size_t)(8 * (v >> 2) + (v & 3)) * p.zc.stride_k;
             float res = lin[0][xt][v] * sigmoid_hw_f32(gate[u][0][xt][v]);
-            const size_t o = b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k + co;
-            if (p.add_residual) res = p.z[o] + res;
-            p.out[o] = res;
+            if (p.add_residual) res = zp[vo] + res;
+            op[vo] = res;
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int j = j0 + 32 * xt + acc_row(v, lh);
+            if (co < C && j < N) {
+              float res = lin[0][xt][v] * sigmoid_hw_f32(gate[u][0][xt][v]);
+              const size_t o = b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k + co;
+              if (p.add_residual) res = p.z[o] + res;
+              p.out[o] = res;
+            }
           }
         }
+      }
     }
   }
 }
@@ -913,7 +982,7 @@ __global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int
 // 8 s .. 8 s + 7 of a lane are its operand for step s (q, k: head channels 16 s + 4 lh + r and
 // 16 s + 8 + 4 lh + r, the same for both, so the order inside the dot product does not matter;
 // v: the keys the core's S^T accumulator holds in the same registers).
-template <int XT, bool SPLIT>
+template <int XT, bool SPLIT, bool FAST>
 __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, int groups) {
   extern __shared__ float smem[];
   constexpr int TPX = 32 * XT;
@@ -923,17 +992,21 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
   const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
   const int j0 = g * TPX;
   const int l = threadIdx.x & 31;
-  layer_norm_tile_x3<XT>(
+  layer_norm_tile_x3<XT, FAST>(
       [&](int pos) -> const float* {
         const int j = j0 + pos;
         return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
       },
       p.ln_w, p.ln_b, C, xn, [&](int pos, const float(&y)[8]) {
         for (int h = 0; h < H; ++h) {
+          const float* wb = p.w_b + h * C + 2 * l;
           float d = 0.f;
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (l + 32 * e < C) d += y[e] * p.w_b[h * C + l + 32 * e];
+          for (int e = 0; e < 4; ++e)
+            if (FAST ? 64 * e < C : 2 * l + 64 * e < C) {
+              d += y[2 * e] * wb[64 * e];
+              d += y[2 * e + 1] * wb[64 * e + 1];
+            }
 #pragma unroll
           for (int o = 16; o > 0; o >>= 1) d += __shfl_xor(d, o, 32);
           if (l == 0) tbs[h * TPX + pos] = d;
@@ -945,7 +1018,8 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
     if (j < N) p.tb[(((size_t)b * H + h) * N + i) * N + j] = tbs[idx];
   }
   const float scale = 1.0f / sqrtf((float)D);
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
+            lh = lane >> 5;
   for (int t = wave; t < (HD + 31) / 32; t += kThreads / 64) {
     const int o0 = 32 * t;
     if (SPLIT) {
@@ -1007,7 +1081,7 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
 
 // Output pass: the gate stays in registers until every wave has finished with LayerNorm(x), then the
 // gated attention output takes its place in LDS.
-template <int XT, bool WIDE>
+template <int XT, bool WIDE, bool FAST>
 __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int groups) {
   extern __shared__ float smem[];
   constexpr int TPX = 32 * XT, MAXT = WIDE ? 2 : 1;
@@ -1016,14 +1090,16 @@ __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int
   const TileX3 og = make_tile_x3(smem, HD, TPX);  // gated attention output, in the same memory
   const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
   const int j0 = g * TPX;
-  layer_norm_tile_x3<XT>(
+  layer_norm_tile_x3<XT, FAST>(
       [&](int pos) -> const float* {
         const int j = j0 + pos;
         return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
       },
       p.ln_w, p.ln_b, C, xn, NoExtra{});
   __syncthreads();
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
+            lh = lane >> 5;
+  const bool whole = j0 + TPX <= N;
   const int n_gt = (HD + 31) / 32;
   f32x16_t gate[MAXT][1][XT];
 #pragma unroll
@@ -1040,13 +1116,21 @@ __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int
     const int t = wave + u * (kThreads / 64), hd = 32 * t + l32;
     if (t < n_gt && hd < HD) {
 #pragma unroll
-      for (int xt = 0; xt < XT; ++xt)
+      for (int xt = 0; xt < XT; ++xt) {
+        if (whole) {
+          const float* op = p.o + (((size_t)b * N + i) * N + j0 + 32 * xt + 4 * lh) * HD + hd;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int pos = 32 * xt + acc_row(v, lh), j = j0 + pos;
-          og.store(pos, hd,
-                   j < N ? p.o[(((size_t)b * N + i) * N + j) * HD + hd] * sigmoid_hw_f32(gate[u][0][xt][v]) : 0.f);
+          for (int v = 0; v < 16; ++v)
+            og.store(32 * xt + acc_row(v, lh), hd, op[(8 * (v >> 2) + (v & 3)) * HD] * sigmoid_hw_f32(gate[u][0][xt][v]));
+        } else {
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int pos = 32 * xt + acc_row(v, lh), j = j0 + pos;
+            og.store(pos, hd,
+                     j < N ? p.o[(((size_t)b * N + i) * N + j) * HD + hd] * sigmoid_hw_f32(gate[u][0][xt][v]) : 0.f);
+          }
         }
+      }
     }
   }
   __syncthreads();
@@ -1056,17 +1140,31 @@ __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int
     f32x16_t acc[1][XT];
     linear_tiles_x3<1, XT, false>(og, W, o0, HD, acc);
 #pragma unroll
-    for (int xt = 0; xt < XT; ++xt)
+    for (int xt = 0; xt < XT; ++xt) {
+      if (FAST && whole) {
+        const size_t lo = b * p.xv.stride_b + i * p.xv.stride_r + (size_t)(j0 + 32 * xt + 4 * lh) * p.xv.stride_k + co;
+        const float* xp = p.x + lo;
+        float* op = p.out + lo;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int j = j0 + 32 * xt + acc_row(v, lh);
-        if (co < C && j < N) {
+        for (int v = 0; v < 16; ++v) {
+          const size_t vo = (size_t)(8 * (v >> 2) + (v & 3)) * p.xv.stride_k;
           float res = acc[0][xt][v];
-          const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
-          if (p.add_residual) res = p.x[o] + res;
-          p.out[o] = res;
+          if (p.add_residual) res = xp[vo] + res;
+          op[vo] = res;
+        }
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int j = j0 + 32 * xt + acc_row(v, lh);
+          if (co < C && j < N) {
+            float res = acc[0][xt][v];
+            const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
+            if (p.add_residual) res = p.x[o] + res;
+            p.out[o] = res;
+          }
         }
       }
+    }
   }
 }
 
@@ -1642,6 +1740,8 @@ bool aligned16(std::initializer_list<const void*> ptrs) {
   return true;
 }
 
+inline bool even_strides(const PairView& v) { return ((v.stride_b | v.stride_r | v.stride_k) & 1) == 0; }
+
 // the largest tiles exceed the default dynamic LDS limit: raised to max_bytes once per device and
 // kernel (slot = index of the kernel's cache)
 constexpr size_t kLdsLimit = 160 * 1024;
@@ -1731,6 +1831,9 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   // split-operand kernels for the position-wise passes: channel counts in multiples of 16 and room for
   // the split weights
   const bool x3 = a.C % 16 == 0 && a.CH % 16 == 0 && a.wsplit && aligned16({a.wsplit});
+  // channel counts in multiples of 64 and rows of z on 8-byte boundaries in both frames
+  const bool fast = a.C % 64 == 0 && a.CH % 64 == 0 && (reinterpret_cast<uintptr_t>(a.z) & 7u) == 0 &&
+                    even_strides(a.z_view) && even_strides(a.z_canonical);
   const int xgroups = (a.N + 32 * kXT - 1) / (32 * kXT);
   const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
   if (x3) {
@@ -1749,12 +1852,18 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
     split(a.w_bg, a.CH, a.C, p.s_bg);
     split(a.w_g, a.C, a.C, p.s_g);
     split(a.w_z, a.C, a.CH, p.s_z);
-    hipError_t e = allow_lds(trimul_proj_x3_f32<kXT>, 4, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, false>, 5, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, true>, 6, kLdsLimit);
+    hipError_t e = allow_lds(trimul_proj_x3_f32<kXT, false>, 4, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, true>, 11, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, false, false>, 5, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, true, false>, 6, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, false, true>, 12, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, true, true>, 13, kLdsLimit);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(trimul_proj_x3_f32<kXT>, dim3(xblocks), dim3(kThreads),
-                       tile_bytes_x3(a.C, 32 * kXT) + 32 * kXT * sizeof(float), stream, p, xgroups);
+    const size_t lds = tile_bytes_x3(a.C, 32 * kXT) + 32 * kXT * sizeof(float);
+    if (fast)
+      hipLaunchKernelGGL((trimul_proj_x3_f32<kXT, true>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    else
+      hipLaunchKernelGGL((trimul_proj_x3_f32<kXT, false>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
   } else if (mm) {
     hipError_t e = allow_lds(trimul_proj_mm_f32, 0);
     if (e == hipSuccess) e = allow_lds(trimul_out_mm_f32, 1);
@@ -1777,10 +1886,10 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   }
   if (x3) {
     const size_t lds = tile_bytes_x3(a.C > a.CH ? a.C : a.CH, 32 * kXT) + 2 * kThreads * sizeof(float);
-    if (a.C > 128 || a.CH > 128)
-      hipLaunchKernelGGL((trimul_out_x3_f32<kXT, true>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
-    else
-      hipLaunchKernelGGL((trimul_out_x3_f32<kXT, false>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    const bool wide = a.C > 128 || a.CH > 128;
+    auto kern = wide ? (fast ? trimul_out_x3_f32<kXT, true, true> : trimul_out_x3_f32<kXT, true, false>)
+                     : (fast ? trimul_out_x3_f32<kXT, false, true> : trimul_out_x3_f32<kXT, false, false>);
+    hipLaunchKernelGGL(kern, dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
   }
   else if (mm)
     hipLaunchKernelGGL(trimul_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + 2 * tile_bytes(a.CH), stream,
@@ -1826,6 +1935,8 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   const int mgroups = (a.N + kTP - 1) / kTP;
   const unsigned mblocks = (unsigned)((long)a.B * a.N * mgroups);
   const bool x3 = a.C % 16 == 0 && (a.H * a.D) % 16 == 0 && a.wsplit && aligned16({a.wsplit});
+  const bool fast = a.C % 64 == 0 && (a.H * a.D) % 64 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 7u) == 0 &&
+                    even_strides(a.x_view);
   // head width 32: q, k and v leave the projection pass as split operands of the split-operand core
   const bool core_x3 = x3 && a.D == 32 && a.qkv_split && aligned16({a.qkv_split});
   p.Jp = (a.N + 31) / 32 * 32;
@@ -1851,17 +1962,20 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     split(a.w_v, HD, a.C, p.s_v);
     split(a.w_g, HD, a.C, p.s_g);
     split(a.w_o, a.C, HD, p.s_o);
-    hipError_t e = allow_lds(triattn_proj_x3_f32<kXT, false>, 7, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, true>, 10, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, false>, 8, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, true>, 9, kLdsLimit);
+    auto proj = core_x3 ? (fast ? triattn_proj_x3_f32<kXT, true, true> : triattn_proj_x3_f32<kXT, true, false>)
+                        : (fast ? triattn_proj_x3_f32<kXT, false, true> : triattn_proj_x3_f32<kXT, false, false>);
+    hipError_t e = allow_lds(triattn_proj_x3_f32<kXT, false, false>, 7, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, true, false>, 10, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, false, true>, 11, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, true, true>, 12, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, false, false>, 8, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, true, false>, 9, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, false, true>, 13, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, true, true>, 14, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(triattn_core_x3_f32, 0, kLdsLimit);
     if (e != hipSuccess) return e;
     const size_t lds = tile_bytes_x3(a.C, 32 * kXT) + (size_t)a.H * 32 * kXT * sizeof(float);
-    if (core_x3)
-      hipLaunchKernelGGL((triattn_proj_x3_f32<kXT, true>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
-    else
-      hipLaunchKernelGGL((triattn_proj_x3_f32<kXT, false>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    hipLaunchKernelGGL(proj, dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
   } else if (mm) {
     hipError_t e = allow_lds(triattn_proj_mm_f32, 2);
     if (e == hipSuccess) e = allow_lds(triattn_out_mm_f32, 3);
@@ -1888,10 +2002,10 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   if (x3) {
     const int HD = a.H * a.D;
     const size_t lds = tile_bytes_x3(a.C > HD ? a.C : HD, 32 * kXT);
-    if (a.C > 128 || HD > 128)
-      hipLaunchKernelGGL((triattn_out_x3_f32<kXT, true>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
-    else
-      hipLaunchKernelGGL((triattn_out_x3_f32<kXT, false>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    const bool wide = a.C > 128 || HD > 128;
+    auto kern = wide ? (fast ? triattn_out_x3_f32<kXT, true, true> : triattn_out_x3_f32<kXT, true, false>)
+                     : (fast ? triattn_out_x3_f32<kXT, false, true> : triattn_out_x3_f32<kXT, false, false>);
+    hipLaunchKernelGGL(kern, dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
   }
   else if (mm)
     hipLaunchKernelGGL(triattn_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + tile_bytes(a.H * a.D), stream,

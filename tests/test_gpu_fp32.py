@@ -30,7 +30,8 @@ def _load(module, params):
 
 @pytest.mark.parametrize("outgoing", [True, False])
 @pytest.mark.parametrize("c,ch,n,batch,masked", [(128, 128, 64, (1,), False), (64, 64, 45, (2,), True), (96, 40, 33, (), True),
-                                                  (36, 20, 19, (), True)])  # channel counts off the multiples of 8: the plain FMA kernels
+                                                  (36, 20, 19, (), True),  # channel counts off the multiples of 8: the plain FMA kernels
+                                                  (48, 80, 29, (2,), True), (256, 64, 40, (), False)])  # multiples of 16, not of 64; more than 128 channels
 def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
     lib()
     gen = torch.Generator().manual_seed(300 + n)
