@@ -151,6 +151,22 @@ __device__ __forceinline__ int tile_slot(int pos, int chunk) {
   return pos * NCH + (chunk ^ key);
 }
 
+// ---- global -> LDS loads without registers ------------------------------------------------------
+#define OF3_LDS_AS __attribute__((address_space(3)))
+
+// raw buffer descriptor over [base, base + bytes): 32-bit offsets, no swizzling; reads beyond the
+// range return zeros
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_rsrc(const void* base, size_t bytes) {
+  const int n = bytes > 0x7fffffffu ? 0x7fffffff : (int)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
+}
+__device__ __forceinline__ void compiler_fence() { __asm__ volatile("" ::: "memory"); }
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {  // vmcnt(N) only (gfx9 encoding, N < 16)
+  static_assert(N >= 0 && N < 16, "low field only");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+}
+
 // XCD-aware block index: hardware deals consecutive workgroup ids round-robin to the 8
 // XCDs; this returns a logical id such that ids [x*per, (x+1)*per) all run on XCD x, so
 // that neighbouring logical ids share one L2.  Caller launches `8*per` blocks and skips

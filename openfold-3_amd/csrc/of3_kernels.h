@@ -213,7 +213,7 @@ struct TriattnF32Args {
   PairView x_view, mask_view;        // module frame
   const float *ln_w, *ln_b, *w_q, *w_k, *w_v, *w_b, *w_g, *w_o;
   float *q, *k, *v;                  // workspace, [B][N][H][N][D] each
-  float *tb;                         // workspace, [B][H][N][N]
+  float *tb;                         // workspace, [B][H][N][N rounded up to a multiple of 32]
   float *o;                          // workspace, [B][N][N][H*D]
   void* wsplit;                      // workspace, triattn_wsplit_bytes(C, H, D) bytes, 16-byte aligned; may be null
   void* qkv_split;                   // workspace, triattn_qkv_split_bytes(B, N, H, D) bytes, 16-byte aligned, may

@@ -85,6 +85,8 @@ inline int64_t f32_triattn_qkv_bytes(int64_t B, int64_t N, int64_t H, int64_t D)
   const int64_t fp32 = 3 * align256(B * N * N * H * D * 4), split = align256((int64_t)of3::triattn_qkv_split_bytes(B, N, H, D));
   return fp32 > split ? fp32 : split;
 }
+// the triangle bias, rows padded to whole 32-key tiles
+inline int64_t f32_triattn_tb_bytes(int64_t B, int64_t N, int64_t H) { return align256(B * H * N * ((N + 31) / 32 * 32) * 4); }
 inline bool f32_strides_ok(const int64_t s[3]) { return s && s[0] >= 0 && s[1] > 0 && s[2] > 0; }
 inline bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
 
@@ -329,7 +331,7 @@ int64_t of3_triattn_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t
   if (dtype != OF3_DTYPE_F32 || !f32_triattn_dims_ok(B, N, C, H, D)) return OF3_EINVAL;
   // q, k, v (fp32, or split into three bf16 terms in whole 32-position tiles), o, the triangle bias
   // and the weights split into three bf16 terms
-  return f32_triattn_qkv_bytes(B, N, H, D) + align256(B * N * N * H * D * 4) + align256(B * H * N * N * 4) +
+  return f32_triattn_qkv_bytes(B, N, H, D) + align256(B * N * N * H * D * 4) + f32_triattn_tb_bytes(B, N, H) +
          align256((int64_t)of3::triattn_wsplit_bytes(C, H, D));
 }
 
@@ -446,7 +448,7 @@ int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask
     a.qkv_split = ws;  // in place of q, k, v
     a.o = reinterpret_cast<float*>(ws + qkv);
     a.tb = reinterpret_cast<float*>(ws + qkv + part);
-    a.wsplit = ws + qkv + part + align256(B * H * N * N * 4);
+    a.wsplit = ws + qkv + part + f32_triattn_tb_bytes(B, N, H);
     a.out = static_cast<float*>(out);
     a.B = (int)B;
     a.N = (int)N;

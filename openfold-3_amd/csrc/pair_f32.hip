@@ -1015,7 +1015,12 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
   __syncthreads();
   for (int idx = threadIdx.x; idx < H * TPX; idx += kThreads) {
     const int h = idx / TPX, j = j0 + idx % TPX;
-    if (j < N) p.tb[(((size_t)b * H + h) * N + i) * N + j] = tbs[idx];
+    if (SPLIT) {
+      // rows padded to whole 32-position tiles; positions past N were normalised to zero rows and store 0
+      if (j < p.Jp) p.tb[(((size_t)b * H + h) * N + i) * p.Jp + j] = tbs[idx];
+    } else if (j < N) {
+      p.tb[(((size_t)b * H + h) * N + i) * N + j] = tbs[idx];
+    }
   }
   const float scale = 1.0f / sqrtf((float)D);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
@@ -1171,27 +1176,32 @@ __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int
 // Attention core on split operands, head width 32.  Work-group = 8 waves = 4 consecutive rows i x 2
 // halves of one (head, 128-query range); a wave owns 64 queries (two 32-query tiles) of one row.
 //   S^T = K Q^T  (rows = keys, columns = queries), six bf16 products per k-step, started from the
-//                triangle bias: the accumulator is loaded with it, and the mask bias is added after
+//                triangle bias (the accumulator is loaded with it); the mask bias of a key tile rides
+//                on one more k-step, A = [hi, mid, lo, 0 ...] of the key's bias split exactly into
+//                three bf16 terms, B = [1, 1, 1, 0 ...], taken only by tiles with a masked or padded key
 //   O^T = V^T P^T, the weights split in registers straight from the S^T accumulator into B operands
 // Per 32-key tile the work-group brings in the bias slice of its query range (it does not depend on
-// i: shared by the four rows) and each row's K and V^T operands (shared by the row's two waves),
-// global -> registers one tile ahead, registers -> the idle half of a double buffer in LDS, one
-// barrier per tile.  Online softmax; the mask bias carries -inf for keys past N.
+// i: shared by the four rows) and each row's K and V^T operands (shared by the row's two waves) with
+// direct-to-LDS buffer loads, one tile ahead, into double buffers: no registers are held for data in
+// flight, and the only wait is one vmcnt(0) + barrier per key tile, a whole tile of arithmetic after
+// the loads were issued.  The bias slice is XOR-swizzled on the global side (a lane picks which
+// 16-byte chunk it fetches for its fixed LDS slot).  Online softmax; keys past N carry a mask bias
+// of -inf.
 constexpr int kXRows = 4;
-constexpr int kXTbLd = 36;  // floats per query row of the bias slice: 16-byte reads of 16 lanes cover all banks
-constexpr size_t kCoreX3Lds = 2 * 128 * kXTbLd * sizeof(float) + 2 * kXRows * 12 * 64 * 16 + 2 * kXRows * 32 * sizeof(float);
+constexpr int kXTbSlots = 128 * 8;                     // bias slice [128 queries][32 keys] fp32 in 16-byte slots
+constexpr int kXKvSlots = 12 * 64;                     // K step 0, 1 (h m l each), then V^T step 0, 1
+constexpr size_t kCoreX3Lds = (size_t)(2 * kXTbSlots + 2 * kXRows * kXKvSlots) * 16;
 
 __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_qc, int n_rg, int total, int per_xcd) {
   constexpr int QT = 2;
   extern __shared__ u32x4_t lds4[];
-  float* tb_lds = reinterpret_cast<float*>(lds4);           // [2][128][kXTbLd]
-  u32x4_t* kv_lds = lds4 + 2 * 128 * kXTbLd / 4;            // [2][kXRows][12][64]: K step 0, 1 (h m l each), V^T step 0, 1
-  float* mb_lds = reinterpret_cast<float*>(kv_lds + 2 * kXRows * 12 * 64);  // [2][kXRows][32]
+  u32x4_t* tb_lds = lds4;                   // [2][kXTbSlots]
+  u32x4_t* kv_lds = lds4 + 2 * kXTbSlots;   // [kXRows][2][kXKvSlots]
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int row = wave >> 1, qh = wave & 1;
   const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
-  const int N = p.N, H = p.H, nt = p.Jp / 32;
+  const int N = p.N, H = p.H, Jp = p.Jp, nt = Jp / 32;
   const int logical = xcd_logical_block(blockIdx.x, per_xcd);
   if (logical >= total) return;  // the whole work-group leaves together
   const int qc = logical % n_qc, rg = (logical / n_qc) % n_rg, bh = logical / (n_qc * n_rg);
@@ -1203,10 +1213,8 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
   const size_t bih = ((size_t)b * N + i) * H + h;
   const long plane = p.qkv_plane / 8;  // in 16-byte slots
   const u32x4_t* Q = reinterpret_cast<const u32x4_t*>(p.qs) + bih * nt * 128 + lane;
-  // this wave's share of its row's tile: the K operands (first wave of the row) or the V^T operands
-  const u32x4_t* KV = reinterpret_cast<const u32x4_t*>(qh ? p.vs : p.ks) + bih * nt * 128 + lane;
-  const float* tbp = p.tb + ((size_t)b * H + h) * N * N;
-  const int nkt = (N + 31) / 32;
+  const float* tbp = p.tb + ((size_t)b * H + h) * N * Jp;  // rows padded to Jp, zeros past N
+  const int nkt = nt;
 
   u32x4_t qop[QT][2][3];
 #pragma unroll
@@ -1218,46 +1226,60 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
       for (int pl = 0; pl < 3; ++pl) qop[qt][st][pl] = Q[pl * plane + (jt * 2 + st) * 64];
   }
 
-  u32x4_t kv_r[6];
-  float tb_r[2][4];
-  float mb_r = 0.f;
-  const bool tb_vec = (N & 3) == 0;  // rows of the bias are 16-byte aligned
-  auto fetch = [&](int kt) {
+  // bias slice: instruction n of wave w fills slots 64 (2 w + n) .. + 63; slot t holds chunk
+  // (t & 7) ^ ((q >> 1) & 7) of query q = t >> 3 of the work-group's range
+  uint32_t tb_off[2];
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    const int t = 64 * (2 * wave + n) + lane;
+    const int qloc = t >> 3, chunk = (t & 7) ^ ((qloc >> 1) & 7);
+    int qrow = qc * 128 + qloc;
+    qrow = qrow < N ? qrow : N - 1;
+    tb_off[n] = (uint32_t)(((size_t)qrow * Jp + 4 * chunk) * sizeof(float));
+  }
+  // this wave's share of its row's tile: the K operands (first wave of the row) or the V^T operands,
+  // one descriptor per term (a plane can be larger than a descriptor's range)
+  const bf16_t* kvp = (qh ? p.vs : p.ks) + bih * Jp * 32;
+  const __amdgpu_buffer_rsrc_t kv_rsrc[3] = {buffer_rsrc(kvp, (size_t)Jp * 64),
+                                             buffer_rsrc(kvp + p.qkv_plane, (size_t)Jp * 64),
+                                             buffer_rsrc(kvp + 2 * p.qkv_plane, (size_t)Jp * 64)};
+  const __amdgpu_buffer_rsrc_t tb_rsrc = buffer_rsrc(tbp, (size_t)N * Jp * sizeof(float));
+  const uint32_t lane_off = lane * 16;
+  u32x4_t* kv_row = kv_lds + row * (2 * kXKvSlots);
+  auto issue_loads = [&](int kt, int buf) {  // buf is a constant at every call site
+    u32x4_t* tdst = tb_lds + buf * kXTbSlots + 128 * wave;
+    u32x4_t* kdst = kv_row + buf * kXKvSlots + 6 * 64 * qh;
+#pragma unroll
+    for (int n = 0; n < 2; ++n)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(tb_rsrc, (void OF3_LDS_AS*)(tdst + 64 * n), 16, tb_off[n],
+                                               kt * (32 * (int)sizeof(float)), 0, 0);
 #pragma unroll
     for (int st = 0; st < 2; ++st)
 #pragma unroll
-      for (int pl = 0; pl < 3; ++pl) kv_r[st * 3 + pl] = KV[pl * plane + (kt * 2 + st) * 64];
-    // bias slice [128 queries][32 keys] in 16-byte chunks: thread t takes chunks t and t + 512
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int chunk = tid + 512 * u, q = qc * 128 + (chunk >> 3), k = kt * 32 + 4 * (chunk & 7);
-      const float* src = tbp + (size_t)q * N + k;
-      if (tb_vec) {
-        const float4 v = (q < N && k < N) ? *reinterpret_cast<const float4*>(src) : make_float4(0.f, 0.f, 0.f, 0.f);
-        tb_r[u][0] = v.x, tb_r[u][1] = v.y, tb_r[u][2] = v.z, tb_r[u][3] = v.w;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) tb_r[u][e] = (q < N && k + e < N) ? src[e] : 0.f;
-      }
-    }
-    if (qh == 0 && lane < 32) {
-      const int k = kt * 32 + lane;
-      float mv = 1.f;
-      if (k < N && p.mask) mv = p.mask[b * p.mv.stride_b + i * p.mv.stride_r + k * p.mv.stride_k];
-      mb_r = k < N ? p.inf * (mv - 1.f) : -__builtin_inff();
-    }
+      for (int pl = 0; pl < 3; ++pl)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(kv_rsrc[pl], (void OF3_LDS_AS*)(kdst + (st * 3 + pl) * 64), 16, lane_off,
+                                                 (kt * 2 + st) * 1024, 0, 0);
   };
-  auto stash = [&](int buf) {
-    u32x4_t* kvb = kv_lds + ((buf * kXRows + row) * 12 + 6 * qh) * 64 + lane;
-#pragma unroll
-    for (int e = 0; e < 6; ++e) kvb[e * 64] = kv_r[e];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int chunk = tid + 512 * u;
-      *reinterpret_cast<float4*>(tb_lds + (buf * 128 + (chunk >> 3)) * kXTbLd + 4 * (chunk & 7)) =
-          make_float4(tb_r[u][0], tb_r[u][1], tb_r[u][2], tb_r[u][3]);
-    }
-    if (qh == 0 && lane < 32) mb_lds[(buf * kXRows + row) * 32 + lane] = mb_r;
+  // mask value of key 32 kt + l32 (clamped to a real key; some bias value when there is no mask: not used)
+  const float* mrow = p.mask ? p.mask + b * p.mv.stride_b + i * p.mv.stride_r : tbp;
+  const long mstep = p.mask ? p.mv.stride_k : 1;
+  auto load_mask = [&](int kt) {
+    const int k = kt * 32 + l32 < N ? kt * 32 + l32 : N - 1;
+    return mrow[k * mstep];
+  };
+  auto mask_bias = [&](int kt, float mv) {
+    return kt * 32 + l32 < N ? (p.mask ? p.inf * (mv - 1.f) : 0.f) : -__builtin_inff();
+  };
+  // the mask-bias k-step on the 8-deep MFMA (two registers per operand): lanes 0..31 hold k = 0..3
+  auto mask_step = [&](float mb, f32x16_t acc) {
+    const bool lo = lh == 0;
+    const uint32_t hi_bits = __float_as_uint(mb) & 0xffff0000u;
+    const float r1 = __builtin_isinf(mb) ? 0.f : mb - __uint_as_float(hi_bits);  // exact
+    const uint32_t mid_bits = __float_as_uint(r1) & 0xffff0000u;
+    const float r2 = r1 - __uint_as_float(mid_bits);  // exact, at most 8 significant bits
+    const u32x2_t a_op = {lo ? ((hi_bits >> 16) | mid_bits) : 0u, lo ? (__float_as_uint(r2) >> 16) : 0u};
+    const u32x2_t b_op = {lo ? 0x3F803F80u : 0u, lo ? 0x3F80u : 0u};
+    return mfma_32x32x8(a_op, b_op, acc);
   };
 
   f32x16_t oacc[QT];
@@ -1268,34 +1290,27 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
     m_run[qt] = -__builtin_inff();
     l_run[qt] = 0.f;
   }
+  const int tb_key = (l32 >> 1) & 7;
 
-  fetch(0);
-  stash(0);
-  if (nkt > 1) fetch(1);
-  __syncthreads();
-  for (int kt = 0; kt < nkt; ++kt) {
-    const int buf = kt & 1;
-    const u32x4_t* kvb = kv_lds + (buf * kXRows + row) * 12 * 64 + lane;
+  auto tile = [&](int buf, float mb) {
+    const bool has_mb = __builtin_amdgcn_ballot_w64(mb != 0.f) != 0;
+    const u32x4_t* kvb = kv_row + buf * kXKvSlots + lane;
+    const u32x4_t* tbuf = tb_lds + buf * kXTbSlots + (64 * qh + l32) * 8;
     u32x4_t kop[2][3];
 #pragma unroll
     for (int st = 0; st < 2; ++st)
 #pragma unroll
       for (int pl = 0; pl < 3; ++pl) kop[st][pl] = kvb[(st * 3 + pl) * 64];
-    float mbv[16];
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      const float4 v = *reinterpret_cast<const float4*>(mb_lds + (buf * kXRows + row) * 32 + 8 * a + 4 * lh);
-      mbv[4 * a] = v.x, mbv[4 * a + 1] = v.y, mbv[4 * a + 2] = v.z, mbv[4 * a + 3] = v.w;
-    }
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
       f32x16_t s;
-      const float* tbl = tb_lds + (buf * 128 + 64 * qh + 32 * qt + l32) * kXTbLd + 4 * lh;
 #pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const float4 v = *reinterpret_cast<const float4*>(tbl + 8 * a);
-        s[4 * a] = v.x, s[4 * a + 1] = v.y, s[4 * a + 2] = v.z, s[4 * a + 3] = v.w;
+      for (int a = 0; a < 4; ++a) {  // registers 4 a .. 4 a + 3: keys 8 a + 4 lh .. + 3 = chunk 2 a + lh
+        const u32x4_t t = tbuf[qt * 256 + ((2 * a + lh) ^ tb_key)];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[4 * a + e] = __uint_as_float(t[e]);
       }
+      if (has_mb) s = mask_step(mb, s);
 #pragma unroll
       for (int st = 0; st < 2; ++st) {  // smallest terms first
         s = mfma_32x32x16(kop[st][2], qop[qt][st][0], s);
@@ -1305,12 +1320,9 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
         s = mfma_32x32x16(kop[st][0], qop[qt][st][1], s);
         s = mfma_32x32x16(kop[st][0], qop[qt][st][0], s);
       }
-      float cmax = -__builtin_inff();
+      float cmax = s[0];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        s[v] += mbv[v];
-        cmax = fmaxf(cmax, s[v]);
-      }
+      for (int v = 1; v < 16; ++v) cmax = fmaxf(cmax, s[v]);
       cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));  // the other half of the query's keys
       const float m_new = fmaxf(m_run[qt], cmax);    // finite: every tile holds a key below N
       const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_new) * kLog2eF32);
@@ -1340,12 +1352,26 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
         oacc[qt] = mfma_32x32x16(vh, ph, oacc[qt]);
       }
     }
-    if (kt + 1 < nkt) {
-      stash(buf ^ 1);
-      if (kt + 2 < nkt) fetch(kt + 2);
-    }
-    __syncthreads();
+  };
+
+  float mv_next = load_mask(0);
+  issue_loads(0, 0);
+  auto step = [&](int kt, int buf) {  // buf is a constant at both call sites: LDS addresses are immediates
+    wait_vmcnt<0>();               // this wave's loads of tile kt (and its mask values) have landed ...
+    __builtin_amdgcn_s_barrier();  // ... and everybody's; nobody reads tile kt - 1's buffers any more
+    compiler_fence();
+    const float mb = mask_bias(kt, mv_next);
+    const int ktn = kt + 1 < nkt ? kt + 1 : nkt - 1;
+    mv_next = load_mask(ktn);
+    issue_loads(ktn, buf ^ 1);
+    tile(buf, mb);
+    compiler_fence();
+  };
+  for (int kt = 0; kt < nkt; kt += 2) {
+    step(kt, 0);
+    if (kt + 1 < nkt) step(kt + 1, 1);
   }
+  wait_vmcnt<0>();  // the loads issued past the end must not outlive the work-group's LDS
 
   if (row_valid) {
 #pragma unroll
@@ -1938,8 +1964,9 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   const bool fast = a.C % 64 == 0 && (a.H * a.D) % 64 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 7u) == 0 &&
                     even_strides(a.x_view);
   // head width 32: q, k and v leave the projection pass as split operands of the split-operand core
-  const bool core_x3 = x3 && a.D == 32 && a.qkv_split && aligned16({a.qkv_split});
   p.Jp = (a.N + 31) / 32 * 32;
+  // (the core addresses the bias of one (batch, head) with 32-bit byte offsets)
+  const bool core_x3 = x3 && a.D == 32 && a.qkv_split && aligned16({a.qkv_split}) && (long)a.N * p.Jp * 4 <= 0x7fffffffL;
   p.qkv_plane = (long)a.B * a.N * a.H * p.Jp * 32;
   p.qs = static_cast<bf16_t*>(a.qkv_split);
   p.ks = p.qs + 3 * p.qkv_plane;

@@ -42,23 +42,7 @@ namespace of3 {
 
 namespace {
 
-#define OF3_GLOBAL_AS __attribute__((address_space(1)))
-#define OF3_LDS_AS __attribute__((address_space(3)))
-
-
-// raw buffer descriptor over [base, base + bytes): 32-bit offsets, no swizzling; reads beyond the
-// range return zeros
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_rsrc(const void* base, size_t bytes) {
-  const int n = bytes > 0x7fffffffu ? 0x7fffffff : (int)bytes;
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, n, 0x00020000);
-}
 __device__ __forceinline__ float xhalf(float v) { return __shfl_xor(v, 32, 64); }
-__device__ __forceinline__ void compiler_fence() { __asm__ volatile("" ::: "memory"); }
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {  // vmcnt(N) only (gfx9 encoding, N < 16)
-  static_assert(N >= 0 && N < 16, "low field only");
-  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
-}
 
 // swizzle keys of the K / V^T tiles in LDS: rows are read in the order rowperm16(lane), i.e.
 // {x..x+3, x+16..x+19, x+4..x+7, x+20..x+23} per 16 lanes; (row & 1, key) must differ inside
