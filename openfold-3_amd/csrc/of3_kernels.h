@@ -197,9 +197,16 @@ struct TrimulF32Args {
   const float *w_ap, *w_ag, *w_bp, *w_bg, *w_g, *w_z;
   float *a, *b, *x;                  // workspace, [B][CH][N][N] each
   void* wsplit;                      // workspace, trimul_wsplit_bytes(C, CH) bytes, 16-byte aligned; may be null
+  void* ab_split;                    // workspace, trimul_ab_split_bytes(B, N, CH) bytes, 16-byte aligned, may
+                                     // overlap a and b; may be null
   float* out;
   int B, N, C, CH, add_residual;
 };
+// a and b in three bf16 terms each, rows and k padded to whole 32-wide panels
+inline size_t trimul_ab_split_bytes(long B, long N, long CH) {
+  const long Np = (N + 31) / 32 * 32;
+  return (size_t)12 * B * CH * Np * Np;
+}
 hipError_t trimul_fwd_f32(const TrimulF32Args& args, hipStream_t stream);
 // room for the six weight matrices split into three bf16 terms each, rows padded to multiples of 32
 inline long wsplit_elems(long rows, long K) { return (rows + 31) / 32 * 32 * K; }

@@ -85,6 +85,10 @@ inline int64_t f32_triattn_qkv_bytes(int64_t B, int64_t N, int64_t H, int64_t D)
   const int64_t fp32 = 3 * align256(B * N * N * H * D * 4), split = align256((int64_t)of3::triattn_qkv_split_bytes(B, N, H, D));
   return fp32 > split ? fp32 : split;
 }
+inline int64_t f32_trimul_ab_bytes(int64_t B, int64_t N, int64_t CH) {
+  const int64_t fp32 = 2 * align256(B * CH * N * N * 4), split = align256((int64_t)of3::trimul_ab_split_bytes(B, N, CH));
+  return fp32 > split ? fp32 : split;
+}
 // the triangle bias, rows padded to whole 32-key tiles
 inline int64_t f32_triattn_tb_bytes(int64_t B, int64_t N, int64_t H) { return align256(B * H * N * ((N + 31) / 32 * 32) * 4); }
 inline bool f32_strides_ok(const int64_t s[3]) { return s && s[0] >= 0 && s[1] > 0 && s[2] > 0; }
@@ -169,8 +173,8 @@ int64_t of3_trimul_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t CH) 
 int64_t of3_trimul_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t CH) {
   if (dtype == OF3_DTYPE_BF16) return of3_trimul_workspace_bytes(B, N, C, CH);
   if (dtype != OF3_DTYPE_F32 || !f32_trimul_dims_ok(B, N, C, CH)) return OF3_EINVAL;
-  // a, b, x and the weights split into three bf16 terms
-  return 3 * align256(B * CH * N * N * 4) + align256((int64_t)of3::trimul_wsplit_bytes(C, CH));
+  // a, b (fp32, or split into three bf16 terms in whole 32-wide panels), x and the weights split into three bf16 terms
+  return f32_trimul_ab_bytes(B, N, CH) + align256(B * CH * N * N * 4) + align256((int64_t)of3::trimul_wsplit_bytes(C, CH));
 }
 
 int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
@@ -269,10 +273,12 @@ int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask,
     a.w_bg = f(w_b_g);
     a.w_g = f(w_g);
     a.w_z = f(w_z);
+    const int64_t ab = f32_trimul_ab_bytes(B, N, CH);
     a.a = reinterpret_cast<float*>(ws);
     a.b = reinterpret_cast<float*>(ws + part);
-    a.x = reinterpret_cast<float*>(ws + 2 * part);
-    a.wsplit = ws + 3 * part;
+    a.ab_split = ws;  // in place of a and b
+    a.x = reinterpret_cast<float*>(ws + ab);
+    a.wsplit = ws + ab + part;
     a.out = static_cast<float*>(out);
     a.B = (int)B;
     a.N = (int)N;

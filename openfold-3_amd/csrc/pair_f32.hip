@@ -388,6 +388,12 @@ struct TrimulF32 {
   const float *w_ap, *w_ag, *w_bp, *w_bg, *w_g, *w_z;
   WeightX3 s_ap, s_ag, s_bp, s_bg, s_g, s_z;  // split copies (the *_x3 kernels only)
   float *a, *b, *x, *out;
+  // a and b split into three bf16 terms in the k-panel layout (the split-operand contraction only):
+  // element (b, c, r, k) of a term sits at ((((b CH + c) Np / 32 + k / 32) Np + r) 32 + k % 32, the
+  // three terms ab_plane elements apart; Np = N rounded up to whole 32-wide panels
+  bf16_t *as, *bs;
+  long ab_plane;
+  int Np;
   int B, N, C, CH, add_residual;
 };
 
@@ -656,7 +662,8 @@ __global__ __launch_bounds__(kThreads) void trimul_out_mm_f32(TrimulF32 p, int g
 // per work-group.  WIDE: more than 128 channels on either side (two output tiles per wave).  FAST:
 // channel counts in multiples of 64 and 8-byte aligned rows; a work-group whose positions all lie
 // below N then stores without lane conditions, from one address per lane plus wave-uniform offsets.
-template <int XT, bool FAST>
+// SPLIT: a and b leave as bf16 terms in the k-panel layout of the split-operand contraction.
+template <int XT, bool FAST, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int groups) {
   extern __shared__ float smem[];
   constexpr int TPX = 32 * XT;
@@ -685,6 +692,42 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
     const int pair = t / n_ot, o0 = 32 * (t - pair * n_ot);
     const WeightX3 W[2] = {pair ? p.s_bg : p.s_ag, pair ? p.s_bp : p.s_ap};
     f32x16_t acc[2][XT];
+    if (SPLIT) {
+      // Channels in the lanes, positions in the registers: registers 8 t .. 8 t + 7 of a lane are the k
+      // 16 t + 8 (e >> 2) + 4 lh + (e & 3) of its channel, stored as the 8 consecutive columns
+      // 16 t + 8 lh .. + 7 of the panel row (16 bytes per term).  a and b use the same order inside
+      // every 16 columns, which is all a sum over k needs.  Positions past N were normalised to zero
+      // rows: they store zeros, the k padding of the panel.
+      linear_tiles_x3<2, XT, false>(xn, W, o0, C, acc);
+      const int c = o0 + l32;
+      const size_t chan = (size_t)p.Np * p.Np;  // elements per channel
+#pragma unroll
+      for (int xt = 0; xt < XT; ++xt) {
+        if (k0 + 32 * xt >= p.Np || !(FAST || c < CH)) continue;
+        bf16_t* lp = (pair ? p.bs : p.as) + ((size_t)b * CH + c) * chan +
+                     ((size_t)((k0 + 32 * xt) >> 5) * p.Np + r) * 32 + 8 * lh;
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          float x[8];
+#pragma unroll
+          for (int a = 0; a < 2; ++a) {
+            const float4 m4 = *reinterpret_cast<const float4*>(msk + 32 * xt + 16 * st + 8 * a + 4 * lh);
+            const float m[4] = {m4.x, m4.y, m4.z, m4.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int v = 8 * st + 4 * a + e;
+              x[4 * a + e] = m[e] * sigmoid_hw_f32(acc[0][xt][v]) * acc[1][xt][v];
+            }
+          }
+          u32x4_t h, mid, lo;
+          split8(x, h, mid, lo);
+          *reinterpret_cast<u32x4_t*>(lp + 16 * st) = h;
+          *reinterpret_cast<u32x4_t*>(lp + p.ab_plane + 16 * st) = mid;
+          *reinterpret_cast<u32x4_t*>(lp + 2 * p.ab_plane + 16 * st) = lo;
+        }
+      }
+      continue;
+    }
     linear_tiles_x3<2, XT, true>(xn, W, o0, C, acc);
     float* dst = pair ? p.b : p.a;
 #pragma unroll
@@ -706,6 +749,131 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
       }
     }
   }
+}
+
+// Contraction on split operands: x[b][c][i][j] = sum_k a[b][c][i][k] b[b][c][j][k] in fp32, six bf16
+// products per k-step.  Work-group = 8 waves (4 x 2) = a 256 x 128 tile of one channel, a wave owns
+// 64 x 64 (2 x 2 MFMA tiles).  Per 32-wide k-panel the three terms of the tile's a rows and b rows
+// travel global -> LDS with direct-to-LDS buffer loads, one panel ahead, into double buffers; one
+// vmcnt(0) + barrier per panel.  A row of a panel is 64 bytes = 4 chunks of 16 bytes; chunk c of row
+// r is stored at position c ^ ((r >> 2) & 3), so that the 8 lanes of an operand read (8 rows, same
+// chunk) fall into different banks; the swizzle is applied on the global side.
+constexpr int kCtM = 256, kCtN = 128;
+constexpr int kCtASlots = kCtM * 4, kCtBSlots = kCtN * 4;      // per term and stage, in 16-byte slots
+constexpr int kCtStage = 3 * (kCtASlots + kCtBSlots);
+constexpr size_t kContractX3Lds = (size_t)2 * kCtStage * 16;
+
+__global__ __launch_bounds__(512) void trimul_contract_x3_f32(TrimulF32 p, int tiles_m, int tiles_n, int total,
+                                                               int per_xcd) {
+  extern __shared__ u32x4_t lds4[];
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int N = p.N, Np = p.Np, panels = Np / 32;
+  const int logical = xcd_logical_block(blockIdx.x, per_xcd);
+  if (logical >= total) return;  // the whole work-group leaves together
+  const int tn = logical % tiles_n, tm = (logical / tiles_n) % tiles_m, bc = logical / (tiles_n * tiles_m);
+  const int i0 = tm * kCtM, j0 = tn * kCtN;
+  const size_t chan = (size_t)Np * Np;
+  // one descriptor per term and side over the channel's plane
+  __amdgpu_buffer_rsrc_t a_rsrc[3], b_rsrc[3];
+#pragma unroll
+  for (int pl = 0; pl < 3; ++pl) {
+    a_rsrc[pl] = buffer_rsrc(p.as + pl * p.ab_plane + bc * chan, chan * sizeof(bf16_t));
+    b_rsrc[pl] = buffer_rsrc(p.bs + pl * p.ab_plane + bc * chan, chan * sizeof(bf16_t));
+  }
+  // slot t of a stage's a (b) part holds chunk (t & 3) ^ ((row >> 2) & 3) of tile row t >> 2; wave w
+  // fills a slots 128 w .. + 127 (two instructions) and b slots 64 w .. + 63 of each term
+  uint32_t a_off[2], b_off;
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    const int t = 128 * wave + 64 * n + lane, row = t >> 2, c = (t & 3) ^ ((row >> 2) & 3);
+    a_off[n] = (uint32_t)(((i0 + row) * 32 + 8 * c) * sizeof(bf16_t));
+  }
+  {
+    const int t = 64 * wave + lane, row = t >> 2, c = (t & 3) ^ ((row >> 2) & 3);
+    b_off = (uint32_t)(((j0 + row) * 32 + 8 * c) * sizeof(bf16_t));
+  }
+  auto issue_loads = [&](int panel, int buf) {  // buf is a constant at every call site
+    u32x4_t* st = lds4 + buf * kCtStage;
+    const int soff = panel * Np * 32 * (int)sizeof(bf16_t);
+#pragma unroll
+    for (int pl = 0; pl < 3; ++pl) {
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc[pl], (void OF3_LDS_AS*)(st + pl * kCtASlots + 128 * wave + 64 * n), 16,
+                                                 a_off[n], soff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc[pl], (void OF3_LDS_AS*)(st + 3 * kCtASlots + pl * kCtBSlots + 64 * wave),
+                                               16, b_off, soff, 0, 0);
+    }
+  };
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni) acc[mi][ni] = zero16();
+  const int key = (l32 >> 2) & 3;
+  auto panel_products = [&](int buf) {
+    const u32x4_t* sa = lds4 + buf * kCtStage + (64 * wm + l32) * 4;
+    const u32x4_t* sb = lds4 + buf * kCtStage + 3 * kCtASlots + (64 * wn + l32) * 4;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int c = (2 * st + lh) ^ key;
+      u32x4_t ao[2][3], bo[2][3];
+#pragma unroll
+      for (int pl = 0; pl < 3; ++pl) {
+#pragma unroll
+        for (int mi = 0; mi < 2; ++mi) ao[mi][pl] = sa[pl * kCtASlots + mi * 128 + c];
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) bo[ni][pl] = sb[pl * kCtBSlots + ni * 128 + c];
+      }
+#pragma unroll
+      for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) {  // smallest terms first
+          acc[mi][ni] = mfma_32x32x16(ao[mi][2], bo[ni][0], acc[mi][ni]);
+          acc[mi][ni] = mfma_32x32x16(ao[mi][0], bo[ni][2], acc[mi][ni]);
+          acc[mi][ni] = mfma_32x32x16(ao[mi][1], bo[ni][1], acc[mi][ni]);
+          acc[mi][ni] = mfma_32x32x16(ao[mi][1], bo[ni][0], acc[mi][ni]);
+          acc[mi][ni] = mfma_32x32x16(ao[mi][0], bo[ni][1], acc[mi][ni]);
+          acc[mi][ni] = mfma_32x32x16(ao[mi][0], bo[ni][0], acc[mi][ni]);
+        }
+    }
+  };
+  issue_loads(0, 0);
+  auto step = [&](int panel, int buf) {
+    wait_vmcnt<0>();               // this wave's loads of the panel have landed ...
+    __builtin_amdgcn_s_barrier();  // ... and everybody's; nobody reads the previous panel's buffers any more
+    compiler_fence();
+    issue_loads(panel + 1 < panels ? panel + 1 : panels - 1, buf ^ 1);
+    panel_products(buf);
+    compiler_fence();
+  };
+  for (int panel = 0; panel < panels; panel += 2) {
+    step(panel, 0);
+    if (panel + 1 < panels) step(panel + 1, 1);
+  }
+  wait_vmcnt<0>();  // the loads issued past the end must not outlive the work-group's LDS
+
+  float* xc = p.x + (size_t)bc * N * N;
+#pragma unroll
+  for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+    for (int ni = 0; ni < 2; ++ni) {
+      const int ib = i0 + 64 * wm + 32 * mi, j = j0 + 64 * wn + 32 * ni + l32;
+      if (ib + 32 <= N && j0 + 64 * wn + 32 * ni + 32 <= N) {
+        float* lp = xc + (size_t)(ib + 4 * lh) * N + j;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) lp[(size_t)(8 * (v >> 2) + (v & 3)) * N] = acc[mi][ni][v];
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int i = ib + acc_row(v, lh);
+          if (i < N && j < N) xc[(size_t)i * N + j] = acc[mi][ni][v];
+        }
+      }
+    }
 }
 
 // Output pass.  The gate is computed first and kept in registers, so that LayerNorm(x) can take the
@@ -1860,6 +2028,12 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   // channel counts in multiples of 64 and rows of z on 8-byte boundaries in both frames
   const bool fast = a.C % 64 == 0 && a.CH % 64 == 0 && (reinterpret_cast<uintptr_t>(a.z) & 7u) == 0 &&
                     even_strides(a.z_view) && even_strides(a.z_canonical);
+  // a and b as bf16 terms for the split-operand contraction (a channel's plane within 32-bit byte offsets)
+  p.Np = (a.N + 31) / 32 * 32;
+  p.ab_plane = (long)a.B * a.CH * p.Np * p.Np;
+  p.as = static_cast<bf16_t*>(a.ab_split);
+  p.bs = p.as + 3 * p.ab_plane;
+  const bool split_ab = x3 && a.ab_split && aligned16({a.ab_split}) && (long)p.Np * p.Np * 2 <= 0x7fffffffL;
   const int xgroups = (a.N + 32 * kXT - 1) / (32 * kXT);
   const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
   if (x3) {
@@ -1878,18 +2052,20 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
     split(a.w_bg, a.CH, a.C, p.s_bg);
     split(a.w_g, a.C, a.C, p.s_g);
     split(a.w_z, a.C, a.CH, p.s_z);
-    hipError_t e = allow_lds(trimul_proj_x3_f32<kXT, false>, 4, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, true>, 11, kLdsLimit);
+    auto proj = split_ab ? (fast ? trimul_proj_x3_f32<kXT, true, true> : trimul_proj_x3_f32<kXT, false, true>)
+                         : (fast ? trimul_proj_x3_f32<kXT, true, false> : trimul_proj_x3_f32<kXT, false, false>);
+    hipError_t e = allow_lds(trimul_proj_x3_f32<kXT, false, false>, 4, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, true, false>, 11, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, false, true>, 14, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, true, true>, 15, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, false, false>, 5, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, true, false>, 6, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, false, true>, 12, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, true, true>, 13, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_contract_x3_f32, 0, kLdsLimit);
     if (e != hipSuccess) return e;
     const size_t lds = tile_bytes_x3(a.C, 32 * kXT) + 32 * kXT * sizeof(float);
-    if (fast)
-      hipLaunchKernelGGL((trimul_proj_x3_f32<kXT, true>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
-    else
-      hipLaunchKernelGGL((trimul_proj_x3_f32<kXT, false>), dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    hipLaunchKernelGGL(proj, dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
   } else if (mm) {
     hipError_t e = allow_lds(trimul_proj_mm_f32, 0);
     if (e == hipSuccess) e = allow_lds(trimul_out_mm_f32, 1);
@@ -1901,7 +2077,14 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   }
   // the contraction has no shape or alignment condition of its own; the FMA kernel stays with the
   // FMA passes so that odd shapes run one family of kernels
-  if (mm || x3) {
+  if (split_ab) {
+    const int tiles_m = (a.N + kCtM - 1) / kCtM, tiles_n = (a.N + kCtN - 1) / kCtN;
+    const long total = (long)a.B * a.CH * tiles_m * tiles_n;
+    if (total > 0x7fffffffL - 8) return hipErrorInvalidValue;
+    const int per_xcd = (int)((total + 7) / 8);
+    hipLaunchKernelGGL(trimul_contract_x3_f32, dim3(per_xcd * 8), dim3(512), kContractX3Lds, stream, p, tiles_m, tiles_n,
+                       (int)total, per_xcd);
+  } else if (mm || x3) {
     const unsigned t = (unsigned)((a.N + 127) / 128);
     hipLaunchKernelGGL(trimul_contract_mm_f32, dim3(t, t, (unsigned)(a.B * a.CH)), dim3(kThreads), 0, stream, p.a, p.b,
                        p.x, a.N);

@@ -102,7 +102,8 @@ def test_trimul_fwd_rejects_bad_arguments(lib):
     assert call(dtype=7) == _lib.OF3_EINVAL                        # unknown dtype code
     # fp32 has its own (larger) workspace and looser shape rules; never call it with a workable argument set here
     need32 = lib.of3_trimul_workspace_bytes_for(_lib.OF3_DTYPE_F32, 1, 64, 128, 128)
-    assert need32 == 3 * 128 * 64 * 64 * 4 + 6 * (5 * 128 * 128 + 128 * 128)  # a, b, x + the weights split in three
+    # a and b in three bf16 terms (12 bytes per element pair, more than 2 fp32 arrays), x, the weights split in three
+    assert need32 == 12 * 128 * 64 * 64 + 128 * 64 * 64 * 4 + 6 * 6 * 128 * 128
     assert call(dtype=_lib.OF3_DTYPE_F32, ws_bytes=need32 - 1) == _lib.OF3_ENOSPC
     assert call(dtype=_lib.OF3_DTYPE_F32, C=300, CH=300) == _lib.OF3_EINVAL
     assert call(dtype=_lib.OF3_DTYPE_F32, z=FAKE + 2, ws_bytes=need32) == _lib.OF3_EINVAL
