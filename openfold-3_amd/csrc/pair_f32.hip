@@ -196,6 +196,12 @@ struct TileX3 {
     h[plane + pos * ld + c] = s.m;
     h[2 * plane + pos * ld + c] = s.l;
   }
+  // the same tile from position `rows` on
+  __device__ __forceinline__ TileX3 at(int rows) const {
+    TileX3 t = *this;
+    t.h += rows * ld;
+    return t;
+  }
   // two adjacent channels c (even) and c + 1 in one 4-byte write per plane
   __device__ __forceinline__ void store2(int pos, int c, float v0, float v1) const {
     const uint32_t ph = pack_bf16(v0, v1);
@@ -246,16 +252,16 @@ __global__ __launch_bounds__(kThreads) void split_weights_f32(const float* __res
   }
 }
 
-// LayerNorm of 32 * XT positions into a split tile, a row per 32 lanes, at most 256 channels (a
+// LayerNorm of 32 * TILES positions by NT threads into a split tile, a row per 32 lanes, at most 256 channels (a
 // multiple of 16).  Lane l holds channels 2 l + 64 e and 2 l + 64 e + 1, e < 4.  A row is read once
 // and kept in registers (the reads of four rows are in flight together).  extra(pos, y) sees the
 // normalised row: y[2 e + i] is channel 2 l + 64 e + i.
 // FAST: the channel count is a multiple of 64 (whole wave-uniform steps instead of lane masks) and
 // the rows are 8-byte aligned (one read per pair).
-template <int XT, bool FAST, typename Src, typename Extra>
+template <int TILES, bool FAST, int NT, typename Src, typename Extra>
 __device__ __forceinline__ void layer_norm_tile_x3(Src src, const float* __restrict__ w, const float* __restrict__ bsh,
                                                    int C, const TileX3& t, Extra extra) {
-  constexpr int kGroups = kThreads / 32, ITERS = 32 * XT / kGroups;
+  constexpr int kGroups = NT / 32, ITERS = 32 * TILES / kGroups;
   static_assert(ITERS % 4 == 0, "rows in batches of four");
   const int l = threadIdx.x & 31, grp = threadIdx.x >> 5;
   const int nE = C / 64;
@@ -663,32 +669,40 @@ __global__ __launch_bounds__(kThreads) void trimul_out_mm_f32(TrimulF32 p, int g
 // channel counts in multiples of 64 and 8-byte aligned rows; a work-group whose positions all lie
 // below N then stores without lane conditions, from one address per lane plus wave-uniform offsets.
 // SPLIT: a and b leave as bf16 terms in the k-panel layout of the split-operand contraction.
-template <int XT, bool FAST, bool SPLIT>
-__global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int groups) {
+template <int XT, int PT, bool FAST, bool SPLIT>
+__global__ __launch_bounds__(kThreads * PT) void trimul_proj_x3_f32(TrimulF32 p, int groups) {
   extern __shared__ float smem[];
-  constexpr int TPX = 32 * XT;
+  constexpr int TPX = 32 * XT * PT, NT = kThreads * PT;
   const int N = p.N, C = p.C, CH = p.CH;
   const TileX3 xn = make_tile_x3(smem, C, TPX);
   float* msk = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + tile_bytes_x3(C, TPX));  // [TPX]
-  const int g = blockIdx.x % groups, r = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
-  const int k0 = g * TPX;
-  const bool whole = k0 + TPX <= N;
-  layer_norm_tile_x3<XT, FAST>(
+  // the PT groups of four waves take PT consecutive rows r of the same 32 XT columns k: in the
+  // k-panel layout of a and b these are contiguous, PT x 64 bytes per channel and term
+  constexpr int KT = 32 * XT;
+  const int row_groups = (N + PT - 1) / PT;
+  const int g = blockIdx.x % groups, r0 = ((blockIdx.x / groups) % row_groups) * PT, b = blockIdx.x / (groups * row_groups);
+  const int k0 = g * KT;
+  layer_norm_tile_x3<XT * PT, FAST, NT>(
       [&](int pos) -> const float* {
-        const int k = k0 + pos;
-        return k < N ? p.z + b * p.zv.stride_b + r * p.zv.stride_r + k * p.zv.stride_k : nullptr;
+        const int r = r0 + pos / KT, k = k0 + pos % KT;
+        return (r < N && k < N) ? p.z + b * p.zv.stride_b + r * p.zv.stride_r + k * p.zv.stride_k : nullptr;
       },
       p.ln_in_w, p.ln_in_b, C, xn, NoExtra{});
   if (threadIdx.x < TPX) {
-    const int k = k0 + threadIdx.x;
-    msk[threadIdx.x] = (k < N && p.mask) ? p.mask[b * p.mv.stride_b + r * p.mv.stride_r + k * p.mv.stride_k] : 1.f;
+    const int r = r0 + threadIdx.x / KT, k = k0 + threadIdx.x % KT;
+    msk[threadIdx.x] =
+        (r < N && k < N && p.mask) ? p.mask[b * p.mv.stride_b + r * p.mv.stride_r + k * p.mv.stride_k] : 1.f;
   }
   __syncthreads();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
             lh = lane >> 5;
+  const int jw = wave & 3, pb = KT * (wave >> 2);  // this wave's share of the output tiles and its positions
+  const int r = r0 + (wave >> 2);                  // (its row)
+  if (r >= N) return;                              // no barrier follows
+  const bool whole = k0 + KT <= N;
   const int n_ot = (CH + 31) / 32;
   const size_t NN = (size_t)N * N;
-  for (int t = wave; t < 2 * n_ot; t += kThreads / 64) {
+  for (int t = jw; t < 2 * n_ot; t += 4) {
     const int pair = t / n_ot, o0 = 32 * (t - pair * n_ot);
     const WeightX3 W[2] = {pair ? p.s_bg : p.s_ag, pair ? p.s_bp : p.s_ap};
     f32x16_t acc[2][XT];
@@ -698,7 +712,7 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
       // 16 t + 8 lh .. + 7 of the panel row (16 bytes per term).  a and b use the same order inside
       // every 16 columns, which is all a sum over k needs.  Positions past N were normalised to zero
       // rows: they store zeros, the k padding of the panel.
-      linear_tiles_x3<2, XT, false>(xn, W, o0, C, acc);
+      linear_tiles_x3<2, XT, false>(xn.at(pb), W, o0, C, acc);
       const int c = o0 + l32;
       const size_t chan = (size_t)p.Np * p.Np;  // elements per channel
 #pragma unroll
@@ -711,7 +725,7 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
           float x[8];
 #pragma unroll
           for (int a = 0; a < 2; ++a) {
-            const float4 m4 = *reinterpret_cast<const float4*>(msk + 32 * xt + 16 * st + 8 * a + 4 * lh);
+            const float4 m4 = *reinterpret_cast<const float4*>(msk + pb + 32 * xt + 16 * st + 8 * a + 4 * lh);
             const float m[4] = {m4.x, m4.y, m4.z, m4.w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -728,12 +742,12 @@ __global__ __launch_bounds__(kThreads) void trimul_proj_x3_f32(TrimulF32 p, int 
       }
       continue;
     }
-    linear_tiles_x3<2, XT, true>(xn, W, o0, C, acc);
+    linear_tiles_x3<2, XT, true>(xn.at(pb), W, o0, C, acc);
     float* dst = pair ? p.b : p.a;
 #pragma unroll
     for (int xt = 0; xt < XT; ++xt) {
       const int k = k0 + 32 * xt + l32;
-      const float m = msk[32 * xt + l32];
+      const float m = msk[pb + 32 * xt + l32];
       if (FAST && whole) {
         float* lp = dst + (((size_t)b * CH + o0) * N + r) * N + (size_t)(4 * lh) * NN + k;
 #pragma unroll
@@ -880,17 +894,17 @@ __global__ __launch_bounds__(512) void trimul_contract_x3_f32(TrimulF32 p, int t
 // place of LayerNorm(z) in LDS.  x is read channel-major straight into registers: thread (position
 // pos = tid % TPX, channel group cg = tid / TPX) holds the channel pairs 2 cg + 2 CG e, + 1; the
 // statistics of a position are summed over the channel groups through LDS.
-template <int XT, bool WIDE, bool FAST>
-__global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int groups) {
+template <int XT, int PT, bool WIDE, bool FAST>
+__global__ __launch_bounds__(kThreads * PT) void trimul_out_x3_f32(TrimulF32 p, int groups) {
   extern __shared__ float smem[];
-  constexpr int TPX = 32 * XT, CG = kThreads / TPX, XP = (WIDE ? 128 : 64) / CG, MAXT = WIDE ? 2 : 1;
+  constexpr int TPX = 32 * XT * PT, NT = kThreads * PT, CG = NT / TPX, XP = (WIDE ? 128 : 64) / CG, MAXT = WIDE ? 2 : 1;
   const int N = p.N, C = p.C, CH = p.CH;
   char* base = reinterpret_cast<char*>(smem);
   const TileX3 zn = make_tile_x3(base, C, TPX);   // LayerNorm(z), then
   const TileX3 xo = make_tile_x3(base, CH, TPX);  // LayerNorm(x) in the same memory
   const size_t tile_max = tile_bytes_x3(C > CH ? C : CH, TPX);
   float* red_s = reinterpret_cast<float*>(base + tile_max);  // [CG][TPX]
-  float* red_q = red_s + kThreads;                           // [CG][TPX]
+  float* red_q = red_s + NT;                                 // [CG][TPX]
   const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
   const int j0 = g * TPX;
   const bool whole = j0 + TPX <= N;
@@ -907,7 +921,7 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
       xv[2 * e + 1] = in ? xp[(size_t)(2 * CG * e + 1) * NN] : 0.f;
     }
   }
-  layer_norm_tile_x3<XT, FAST>(
+  layer_norm_tile_x3<XT * PT, FAST, NT>(
       [&](int pos) -> const float* {
         const int j = j0 + pos;
         return j < N ? p.z + b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k : nullptr;
@@ -916,14 +930,15 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
   __syncthreads();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
             lh = lane >> 5;
+  const int jw = wave & 3, pb = 32 * XT * (wave >> 2);  // this wave's share of the output tiles and its positions
   const int n_ot = (C + 31) / 32;
   f32x16_t gate[MAXT][1][XT];
 #pragma unroll
   for (int u = 0; u < MAXT; ++u) {
-    const int t = wave + u * (kThreads / 64);
+    const int t = jw + 4 * u;
     if (t < n_ot) {
       const WeightX3 Wg[1] = {p.s_g};
-      linear_tiles_x3<1, XT, false>(zn, Wg, 32 * t, C, gate[u]);
+      linear_tiles_x3<1, XT, false>(zn.at(pb), Wg, 32 * t, C, gate[u]);
     }
   }
   // LayerNorm over the channels of x
@@ -964,16 +979,16 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
   __syncthreads();
 #pragma unroll
   for (int u = 0; u < MAXT; ++u) {
-    const int t = wave + u * (kThreads / 64);
+    const int t = jw + 4 * u;
     if (t < n_ot) {
       const int o0 = 32 * t, co = o0 + l32;
       const WeightX3 Wz[1] = {p.s_z};
       f32x16_t lin[1][XT];
-      linear_tiles_x3<1, XT, false>(xo, Wz, o0, CH, lin);
+      linear_tiles_x3<1, XT, false>(xo.at(pb), Wz, o0, CH, lin);
 #pragma unroll
       for (int xt = 0; xt < XT; ++xt) {
         if (FAST && whole) {
-          const size_t lo = b * p.zc.stride_b + i * p.zc.stride_r + (size_t)(j0 + 32 * xt + 4 * lh) * p.zc.stride_k + co;
+          const size_t lo = b * p.zc.stride_b + i * p.zc.stride_r + (size_t)(j0 + pb + 32 * xt + 4 * lh) * p.zc.stride_k + co;
           const float* zp = p.z + lo;
           float* op = p.out + lo;
 #pragma unroll
@@ -986,7 +1001,7 @@ __global__ __launch_bounds__(kThreads) void trimul_out_x3_f32(TrimulF32 p, int g
         } else {
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
-            const int j = j0 + 32 * xt + acc_row(v, lh);
+            const int j = j0 + pb + 32 * xt + acc_row(v, lh);
             if (co < C && j < N) {
               float res = lin[0][xt][v] * sigmoid_hw_f32(gate[u][0][xt][v]);
               const size_t o = b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k + co;
@@ -1150,17 +1165,17 @@ __global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int
 // 8 s .. 8 s + 7 of a lane are its operand for step s (q, k: head channels 16 s + 4 lh + r and
 // 16 s + 8 + 4 lh + r, the same for both, so the order inside the dot product does not matter;
 // v: the keys the core's S^T accumulator holds in the same registers).
-template <int XT, bool SPLIT, bool FAST>
-__global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, int groups) {
+template <int XT, int PT, bool SPLIT, bool FAST>
+__global__ __launch_bounds__(kThreads * PT) void triattn_proj_x3_f32(TriattnF32 p, int groups) {
   extern __shared__ float smem[];
-  constexpr int TPX = 32 * XT;
+  constexpr int TPX = 32 * XT * PT, NT = kThreads * PT;
   const int N = p.N, C = p.C, H = p.H, D = p.D, HD = H * D;
   const TileX3 xn = make_tile_x3(smem, C, TPX);
   float* tbs = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + tile_bytes_x3(C, TPX));  // [H][TPX]
   const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
   const int j0 = g * TPX;
   const int l = threadIdx.x & 31;
-  layer_norm_tile_x3<XT, FAST>(
+  layer_norm_tile_x3<XT * PT, FAST, NT>(
       [&](int pos) -> const float* {
         const int j = j0 + pos;
         return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
@@ -1181,7 +1196,7 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
         }
       });
   __syncthreads();
-  for (int idx = threadIdx.x; idx < H * TPX; idx += kThreads) {
+  for (int idx = threadIdx.x; idx < H * TPX; idx += NT) {
     const int h = idx / TPX, j = j0 + idx % TPX;
     if (SPLIT) {
       // rows padded to whole 32-position tiles; positions past N were normalised to zero rows and store 0
@@ -1193,14 +1208,15 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
   const float scale = 1.0f / sqrtf((float)D);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
             lh = lane >> 5;
-  for (int t = wave; t < (HD + 31) / 32; t += kThreads / 64) {
+  const int jw = wave & 3, pb = 32 * XT * (wave >> 2);  // this wave's share of the output tiles and its positions
+  for (int t = jw; t < (HD + 31) / 32; t += 4) {
     const int o0 = 32 * t;
     if (SPLIT) {
       // positions past N were normalised to zero rows: their q, k and v are zeros, and are stored
-      const size_t slot0 = ((((size_t)b * N + i) * H + t) * (p.Jp / 32) + j0 / 32) * 128 + lane;
+      const size_t slot0 = ((((size_t)b * N + i) * H + t) * (p.Jp / 32) + (j0 + pb) / 32) * 128 + lane;
       const long plane = p.qkv_plane / 8;
       auto store = [&](bf16_t* dst, const f32x16_t& acc, int xt, float mul) {
-        if (j0 + 32 * xt >= p.Jp) return;  // a tile past the padded row (XT > 1 only)
+        if (j0 + pb + 32 * xt >= p.Jp) return;  // a tile past the padded row (XT > 1 only)
         u32x4_t* d4 = reinterpret_cast<u32x4_t*>(dst) + slot0 + xt * 128;
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
@@ -1217,7 +1233,7 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
       {
         const WeightX3 W[2] = {p.s_q, p.s_k};
         f32x16_t acc[2][XT];
-        linear_tiles_x3<2, XT, true>(xn, W, o0, C, acc);
+        linear_tiles_x3<2, XT, true>(xn.at(pb), W, o0, C, acc);
 #pragma unroll
         for (int xt = 0; xt < XT; ++xt) {
           store(p.qs, acc[0][xt], xt, scale);  // q / sqrt(c) after the projection (attention.py:283-284)
@@ -1227,7 +1243,7 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
       {
         const WeightX3 W[1] = {p.s_v};
         f32x16_t acc[1][XT];
-        linear_tiles_x3<1, XT, false>(xn, W, o0, C, acc);
+        linear_tiles_x3<1, XT, false>(xn.at(pb), W, o0, C, acc);
 #pragma unroll
         for (int xt = 0; xt < XT; ++xt) store(p.vs, acc[0][xt], xt, 1.f);
       }
@@ -1235,12 +1251,12 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
       const int hd = o0 + l32, h = hd / D, d = hd - h * D;
       const WeightX3 W[3] = {p.s_q, p.s_k, p.s_v};
       f32x16_t acc[3][XT];
-      linear_tiles_x3<3, XT, false>(xn, W, o0, C, acc);
+      linear_tiles_x3<3, XT, false>(xn.at(pb), W, o0, C, acc);
 #pragma unroll
       for (int xt = 0; xt < XT; ++xt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int j = j0 + 32 * xt + acc_row(v, lh);
+          const int j = j0 + pb + 32 * xt + acc_row(v, lh);
           if (hd < HD && j < N) {
             const size_t o = ((((size_t)b * N + i) * H + h) * N + j) * D + d;
             p.q[o] = acc[0][xt][v] * scale;  // q / sqrt(c) after the projection (attention.py:283-284)
@@ -1254,16 +1270,16 @@ __global__ __launch_bounds__(kThreads) void triattn_proj_x3_f32(TriattnF32 p, in
 
 // Output pass: the gate stays in registers until every wave has finished with LayerNorm(x), then the
 // gated attention output takes its place in LDS.
-template <int XT, bool WIDE, bool FAST>
-__global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int groups) {
+template <int XT, int PT, bool WIDE, bool FAST>
+__global__ __launch_bounds__(kThreads * PT) void triattn_out_x3_f32(TriattnF32 p, int groups) {
   extern __shared__ float smem[];
-  constexpr int TPX = 32 * XT, MAXT = WIDE ? 2 : 1;
+  constexpr int TPX = 32 * XT * PT, NT = kThreads * PT, MAXT = WIDE ? 2 : 1;
   const int N = p.N, C = p.C, HD = p.H * p.D;
   const TileX3 xn = make_tile_x3(smem, C, TPX);
   const TileX3 og = make_tile_x3(smem, HD, TPX);  // gated attention output, in the same memory
   const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
   const int j0 = g * TPX;
-  layer_norm_tile_x3<XT, FAST>(
+  layer_norm_tile_x3<XT * PT, FAST, NT>(
       [&](int pos) -> const float* {
         const int j = j0 + pos;
         return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
@@ -1272,33 +1288,34 @@ __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int
   __syncthreads();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
             lh = lane >> 5;
+  const int jw = wave & 3, pb = 32 * XT * (wave >> 2);  // this wave's share of the output tiles and its positions
   const bool whole = j0 + TPX <= N;
   const int n_gt = (HD + 31) / 32;
   f32x16_t gate[MAXT][1][XT];
 #pragma unroll
   for (int u = 0; u < MAXT; ++u) {
-    const int t = wave + u * (kThreads / 64);
+    const int t = jw + 4 * u;
     if (t < n_gt) {
       const WeightX3 W[1] = {p.s_g};
-      linear_tiles_x3<1, XT, false>(xn, W, 32 * t, C, gate[u]);
+      linear_tiles_x3<1, XT, false>(xn.at(pb), W, 32 * t, C, gate[u]);
     }
   }
   __syncthreads();
 #pragma unroll
   for (int u = 0; u < MAXT; ++u) {
-    const int t = wave + u * (kThreads / 64), hd = 32 * t + l32;
+    const int t = jw + 4 * u, hd = 32 * t + l32;
     if (t < n_gt && hd < HD) {
 #pragma unroll
       for (int xt = 0; xt < XT; ++xt) {
         if (whole) {
-          const float* op = p.o + (((size_t)b * N + i) * N + j0 + 32 * xt + 4 * lh) * HD + hd;
+          const float* op = p.o + (((size_t)b * N + i) * N + j0 + pb + 32 * xt + 4 * lh) * HD + hd;
 #pragma unroll
           for (int v = 0; v < 16; ++v)
-            og.store(32 * xt + acc_row(v, lh), hd, op[(8 * (v >> 2) + (v & 3)) * HD] * sigmoid_hw_f32(gate[u][0][xt][v]));
+            og.store(pb + 32 * xt + acc_row(v, lh), hd, op[(8 * (v >> 2) + (v & 3)) * HD] * sigmoid_hw_f32(gate[u][0][xt][v]));
         } else {
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
-            const int pos = 32 * xt + acc_row(v, lh), j = j0 + pos;
+            const int pos = pb + 32 * xt + acc_row(v, lh), j = j0 + pos;
             og.store(pos, hd,
                      j < N ? p.o[(((size_t)b * N + i) * N + j) * HD + hd] * sigmoid_hw_f32(gate[u][0][xt][v]) : 0.f);
           }
@@ -1307,15 +1324,15 @@ __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int
     }
   }
   __syncthreads();
-  for (int t = wave; t < (C + 31) / 32; t += kThreads / 64) {
+  for (int t = jw; t < (C + 31) / 32; t += 4) {
     const int o0 = 32 * t, co = o0 + l32;
     const WeightX3 W[1] = {p.s_o};
     f32x16_t acc[1][XT];
-    linear_tiles_x3<1, XT, false>(og, W, o0, HD, acc);
+    linear_tiles_x3<1, XT, false>(og.at(pb), W, o0, HD, acc);
 #pragma unroll
     for (int xt = 0; xt < XT; ++xt) {
       if (FAST && whole) {
-        const size_t lo = b * p.xv.stride_b + i * p.xv.stride_r + (size_t)(j0 + 32 * xt + 4 * lh) * p.xv.stride_k + co;
+        const size_t lo = b * p.xv.stride_b + i * p.xv.stride_r + (size_t)(j0 + pb + 32 * xt + 4 * lh) * p.xv.stride_k + co;
         const float* xp = p.x + lo;
         float* op = p.out + lo;
 #pragma unroll
@@ -1328,7 +1345,7 @@ __global__ __launch_bounds__(kThreads) void triattn_out_x3_f32(TriattnF32 p, int
       } else {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int j = j0 + 32 * xt + acc_row(v, lh);
+          const int j = j0 + pb + 32 * xt + acc_row(v, lh);
           if (co < C && j < N) {
             float res = acc[0][xt][v];
             const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
@@ -1942,7 +1959,12 @@ constexpr size_t kLdsLimit = 160 * 1024;
 #ifndef OF3_X3_XT
 #define OF3_X3_XT 1
 #endif
-constexpr int kXT = OF3_X3_XT;  // 32-position tiles per work-group of the split-operand passes
+constexpr int kXT = OF3_X3_XT;  // 32-position tiles per wave of the split-operand passes
+#ifndef OF3_X3_PT
+#define OF3_X3_PT 2
+#endif
+constexpr int kPT = OF3_X3_PT;  // groups of four waves per work-group, each with its own positions: waves of different
+                                // groups read the same weights at about the same time, once from L2
 template <typename Kern>
 hipError_t allow_lds(Kern kern, int slot, size_t max_bytes = 3 * (size_t)kTP * (kMaxC + 4) * sizeof(float)) {
   static int cache[16][kMaxDevices];
@@ -2034,7 +2056,7 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   p.as = static_cast<bf16_t*>(a.ab_split);
   p.bs = p.as + 3 * p.ab_plane;
   const bool split_ab = x3 && a.ab_split && aligned16({a.ab_split}) && (long)p.Np * p.Np * 2 <= 0x7fffffffL;
-  const int xgroups = (a.N + 32 * kXT - 1) / (32 * kXT);
+  const int xgroups = (a.N + 32 * kXT * kPT - 1) / (32 * kXT * kPT);
   const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
   if (x3) {
     bf16_t* w = static_cast<bf16_t*>(a.wsplit);
@@ -2052,20 +2074,21 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
     split(a.w_bg, a.CH, a.C, p.s_bg);
     split(a.w_g, a.C, a.C, p.s_g);
     split(a.w_z, a.C, a.CH, p.s_z);
-    auto proj = split_ab ? (fast ? trimul_proj_x3_f32<kXT, true, true> : trimul_proj_x3_f32<kXT, false, true>)
-                         : (fast ? trimul_proj_x3_f32<kXT, true, false> : trimul_proj_x3_f32<kXT, false, false>);
-    hipError_t e = allow_lds(trimul_proj_x3_f32<kXT, false, false>, 4, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, true, false>, 11, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, false, true>, 14, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, true, true>, 15, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, false, false>, 5, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, true, false>, 6, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, false, true>, 12, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, true, true>, 13, kLdsLimit);
+    auto proj = split_ab ? (fast ? trimul_proj_x3_f32<kXT, kPT, true, true> : trimul_proj_x3_f32<kXT, kPT, false, true>)
+                         : (fast ? trimul_proj_x3_f32<kXT, kPT, true, false> : trimul_proj_x3_f32<kXT, kPT, false, false>);
+    hipError_t e = allow_lds(trimul_proj_x3_f32<kXT, kPT, false, false>, 4, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, kPT, true, false>, 11, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, kPT, false, true>, 14, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, kPT, true, true>, 15, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, kPT, false, false>, 5, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, kPT, true, false>, 6, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, kPT, false, true>, 12, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, kPT, true, true>, 13, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(trimul_contract_x3_f32, 0, kLdsLimit);
     if (e != hipSuccess) return e;
-    const size_t lds = tile_bytes_x3(a.C, 32 * kXT) + 32 * kXT * sizeof(float);
-    hipLaunchKernelGGL(proj, dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    const size_t lds = tile_bytes_x3(a.C, 32 * kXT * kPT) + 32 * kXT * kPT * sizeof(float);
+    const int kgroups = (a.N + 32 * kXT - 1) / (32 * kXT), row_groups = (a.N + kPT - 1) / kPT;
+    hipLaunchKernelGGL(proj, dim3((unsigned)((long)a.B * row_groups * kgroups)), dim3(kThreads * kPT), lds, stream, p, kgroups);
   } else if (mm) {
     hipError_t e = allow_lds(trimul_proj_mm_f32, 0);
     if (e == hipSuccess) e = allow_lds(trimul_out_mm_f32, 1);
@@ -2094,11 +2117,11 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
                        p.x, a.N);
   }
   if (x3) {
-    const size_t lds = tile_bytes_x3(a.C > a.CH ? a.C : a.CH, 32 * kXT) + 2 * kThreads * sizeof(float);
+    const size_t lds = tile_bytes_x3(a.C > a.CH ? a.C : a.CH, 32 * kXT * kPT) + 2 * kThreads * kPT * sizeof(float);
     const bool wide = a.C > 128 || a.CH > 128;
-    auto kern = wide ? (fast ? trimul_out_x3_f32<kXT, true, true> : trimul_out_x3_f32<kXT, true, false>)
-                     : (fast ? trimul_out_x3_f32<kXT, false, true> : trimul_out_x3_f32<kXT, false, false>);
-    hipLaunchKernelGGL(kern, dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    auto kern = wide ? (fast ? trimul_out_x3_f32<kXT, kPT, true, true> : trimul_out_x3_f32<kXT, kPT, true, false>)
+                     : (fast ? trimul_out_x3_f32<kXT, kPT, false, true> : trimul_out_x3_f32<kXT, kPT, false, false>);
+    hipLaunchKernelGGL(kern, dim3(xblocks), dim3(kThreads * kPT), lds, stream, p, xgroups);
   }
   else if (mm)
     hipLaunchKernelGGL(trimul_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + 2 * tile_bytes(a.CH), stream,
@@ -2154,7 +2177,7 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   p.qs = static_cast<bf16_t*>(a.qkv_split);
   p.ks = p.qs + 3 * p.qkv_plane;
   p.vs = p.qs + 6 * p.qkv_plane;
-  const int xgroups = (a.N + 32 * kXT - 1) / (32 * kXT);
+  const int xgroups = (a.N + 32 * kXT * kPT - 1) / (32 * kXT * kPT);
   const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
   if (x3) {
     bf16_t* w = static_cast<bf16_t*>(a.wsplit);
@@ -2172,20 +2195,20 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     split(a.w_v, HD, a.C, p.s_v);
     split(a.w_g, HD, a.C, p.s_g);
     split(a.w_o, a.C, HD, p.s_o);
-    auto proj = core_x3 ? (fast ? triattn_proj_x3_f32<kXT, true, true> : triattn_proj_x3_f32<kXT, true, false>)
-                        : (fast ? triattn_proj_x3_f32<kXT, false, true> : triattn_proj_x3_f32<kXT, false, false>);
-    hipError_t e = allow_lds(triattn_proj_x3_f32<kXT, false, false>, 7, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, true, false>, 10, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, false, true>, 11, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, true, true>, 12, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, false, false>, 8, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, true, false>, 9, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, false, true>, 13, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, true, true>, 14, kLdsLimit);
+    auto proj = core_x3 ? (fast ? triattn_proj_x3_f32<kXT, kPT, true, true> : triattn_proj_x3_f32<kXT, kPT, true, false>)
+                        : (fast ? triattn_proj_x3_f32<kXT, kPT, false, true> : triattn_proj_x3_f32<kXT, kPT, false, false>);
+    hipError_t e = allow_lds(triattn_proj_x3_f32<kXT, kPT, false, false>, 7, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, kPT, true, false>, 10, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, kPT, false, true>, 11, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, kPT, true, true>, 12, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, kPT, false, false>, 8, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, kPT, true, false>, 9, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, kPT, false, true>, 13, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, kPT, true, true>, 14, kLdsLimit);
     if (e == hipSuccess) e = allow_lds(triattn_core_x3_f32, 0, kLdsLimit);
     if (e != hipSuccess) return e;
-    const size_t lds = tile_bytes_x3(a.C, 32 * kXT) + (size_t)a.H * 32 * kXT * sizeof(float);
-    hipLaunchKernelGGL(proj, dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    const size_t lds = tile_bytes_x3(a.C, 32 * kXT * kPT) + (size_t)a.H * 32 * kXT * kPT * sizeof(float);
+    hipLaunchKernelGGL(proj, dim3(xblocks), dim3(kThreads * kPT), lds, stream, p, xgroups);
   } else if (mm) {
     hipError_t e = allow_lds(triattn_proj_mm_f32, 2);
     if (e == hipSuccess) e = allow_lds(triattn_out_mm_f32, 3);
@@ -2211,11 +2234,11 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     return hipErrorInvalidValue;
   if (x3) {
     const int HD = a.H * a.D;
-    const size_t lds = tile_bytes_x3(a.C > HD ? a.C : HD, 32 * kXT);
+    const size_t lds = tile_bytes_x3(a.C > HD ? a.C : HD, 32 * kXT * kPT);
     const bool wide = a.C > 128 || HD > 128;
-    auto kern = wide ? (fast ? triattn_out_x3_f32<kXT, true, true> : triattn_out_x3_f32<kXT, true, false>)
-                     : (fast ? triattn_out_x3_f32<kXT, false, true> : triattn_out_x3_f32<kXT, false, false>);
-    hipLaunchKernelGGL(kern, dim3(xblocks), dim3(kThreads), lds, stream, p, xgroups);
+    auto kern = wide ? (fast ? triattn_out_x3_f32<kXT, kPT, true, true> : triattn_out_x3_f32<kXT, kPT, true, false>)
+                     : (fast ? triattn_out_x3_f32<kXT, kPT, false, true> : triattn_out_x3_f32<kXT, kPT, false, false>);
+    hipLaunchKernelGGL(kern, dim3(xblocks), dim3(kThreads * kPT), lds, stream, p, xgroups);
   }
   else if (mm)
     hipLaunchKernelGGL(triattn_out_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + tile_bytes(a.H * a.D), stream,
