@@ -3,6 +3,8 @@
 Tolerance (north star, fp32): max-abs error <= 1e-4.  Inputs are N(0,1), weights N(0, 1/fan_in)
 and LayerNorm affine near identity, so outputs are O(1) and an absolute bound is meaningful;
 benchmark configuration 1 (N=64, c_z=128, 4 heads x 32, all-ones mask) is the first case."""
+import random
+
 import pytest
 import torch
 
@@ -92,3 +94,44 @@ def test_block_fp32_padded():
     mask = orc.tail_padding_mask((2,), n, torch.tensor([9, 0]))
     got = m(z.to(DEV), mask.to(DEV))
     _maxerr("block fp32 padded", got, orc.pair_stack_block(z, mask, p, heads))
+
+
+def test_block_fp32_n768():
+    """the headline shape in fp32 (N=768, c_z=128, 4 heads x 32) against the oracle: the split-operand
+    kernels at the size the bench times them at, every key tile and k-panel of the full loops."""
+    lib()
+    n, c, d, heads = 768, 128, 32, 4
+    p = orc.make_block_params(0, c, c, d, heads)
+    m = _load(of3pair.PairStack(c, c, d, heads), p)
+    z = orc.make_pair_input(1, (1,), n, c)
+    mask = orc.tail_padding_mask((1,), n, torch.tensor([40]))
+    print("fp32 block n=768", flush=True)
+    got = m(z.to(DEV), mask.to(DEV))
+    _maxerr("block fp32 n=768", got, orc.pair_stack_block(z, mask, p, heads, row_chunk=32))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_fp32_random_shapes(seed):
+    """seeded random shapes through both fp32 modules: ragged N around the tile sizes (32-key tiles,
+    128-query ranges, 256 x 128 contraction tiles), channel counts on and off the multiples of 64, masks
+    from empty to dense, batch 1-2."""
+    lib()
+    rnd = random.Random(900 + seed)
+    n = rnd.choice([1, 2, 3, 5, 31, 32, 33, 63, 65, 96, 127, 129, 130, 160, 200, 257, 260])
+    c = rnd.choice([64, 128, 48, 80])
+    ch = rnd.choice([64, 128, 32, 48])
+    heads = rnd.choice([1, 2, 4])
+    batch = rnd.choice([(), (1,), (2,)])
+    keep = rnd.choice([0.0, 0.3, 0.8, 1.0])
+    gen = torch.Generator().manual_seed(1000 + seed)
+    z = torch.randn(*batch, n, n, c, generator=gen) * rnd.choice([0.5, 1.0, 3.0])
+    mask = (torch.rand(*batch, n, n, generator=gen) < keep).float() if keep < 1.0 else None
+    print("fp32 random shape seed=%d n=%d c=%d ch=%d heads=%d batch=%s keep=%.1f" % (seed, n, c, ch, heads, batch, keep), flush=True)
+    outgoing, starting = bool(seed & 1), bool(seed & 2)
+    pm = orc.make_trimul_params(gen, c, ch)
+    cls = of3pair.TriangleMultiplicationOutgoing if outgoing else of3pair.TriangleMultiplicationIncoming
+    got = _load(cls(c, ch), pm)(z.to(DEV), mask=None if mask is None else mask.to(DEV))
+    _maxerr("trimul fp32 random", got, orc.trimul_update(z, mask, pm, outgoing))
+    pa = orc.make_triattn_params(gen, c, 32, heads)
+    got = _load(of3pair.TriangleAttention(c, 32, heads, starting=starting), pa)(z.to(DEV), mask=None if mask is None else mask.to(DEV))
+    _maxerr("triattn fp32 random", got, orc.triattn_update(z, mask, pa, heads, starting=starting))
