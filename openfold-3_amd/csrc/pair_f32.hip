@@ -1361,7 +1361,9 @@ __global__ __launch_bounds__(kThreads * PT) void triattn_out_x3_f32(TriattnF32 p
 // Attention core on split operands, head width 32.  Work-group = 8 waves = 4 consecutive rows i x 2
 // halves of one (head, 128-query range); a wave owns 64 queries (two 32-query tiles) of one row.
 //   S^T = K Q^T  (rows = keys, columns = queries), six bf16 products per k-step, started from the
-//                triangle bias (the accumulator is loaded with it); the mask bias of a key tile rides
+//                triangle bias (the accumulator is loaded with it; logits stay in natural units, not
+//                pre-multiplied by log2(e): a row of masked keys has to lose its logits against -1e9 at
+//                the reference's granularity, or it averages other keys than the reference does); the mask bias of a key tile rides
 //                on one more k-step, A = [hi, mid, lo, 0 ...] of the key's bias split exactly into
 //                three bf16 terms, B = [1, 1, 1, 0 ...], taken only by tiles with a masked or padded key
 //   O^T = V^T P^T, the weights split in registers straight from the S^T accumulator into B operands
