@@ -258,11 +258,51 @@ __global__ __launch_bounds__(kThreads) void split_weights_f32(const float* __res
 // normalised row: y[2 e + i] is channel 2 l + 64 e + i.
 // FAST: the channel count is a multiple of 64 (whole wave-uniform steps instead of lane masks) and
 // the rows are 8-byte aligned (one read per pair).
-template <int TILES, bool FAST, int NT, typename Src, typename Extra>
-__device__ __forceinline__ void layer_norm_tile_x3(Src src, const float* __restrict__ w, const float* __restrict__ bsh,
-                                                   int C, const TileX3& t, Extra extra) {
-  constexpr int kGroups = NT / 32, ITERS = 32 * TILES / kGroups;
-  static_assert(ITERS % 4 == 0, "rows in batches of four");
+//
+// The work comes in two halves, so that a persistent work-group can have the rows of its next tile
+// in flight while it multiplies the current one: ln_rows_load issues the reads (src(pos, valid)
+// returns an address that can always be read, of a real row, and says whether the position exists:
+// no read is under a lane condition, which would make the compiler wait for every read in flight),
+// ln_rows_store normalises, splits and writes the tile.
+template <int TILES, int NT>
+struct LnRows {
+  static constexpr int kGroups = NT / 32, ITERS = 32 * TILES / kGroups;
+  float val[ITERS][8];
+  bool has[ITERS];
+};
+
+template <int TILES, bool FAST, int NT, typename Src>
+__device__ __forceinline__ void ln_rows_load(Src src, int C, LnRows<TILES, NT>& r) {
+  constexpr int kGroups = NT / 32, ITERS = LnRows<TILES, NT>::ITERS;
+  const int l = threadIdx.x & 31, grp = threadIdx.x >> 5;
+  const int nE = C / 64;
+#pragma unroll
+  for (int u = 0; u < ITERS; ++u) {
+    bool valid;
+    const float* row = src(grp + u * kGroups, valid);
+    r.has[u] = valid;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (FAST) {
+        if (e < nE) {
+          const float2 v = *reinterpret_cast<const float2*>(row + 2 * l + 64 * e);
+          r.val[u][2 * e] = v.x, r.val[u][2 * e + 1] = v.y;
+        } else {
+          r.val[u][2 * e] = r.val[u][2 * e + 1] = 0.f;
+        }
+      } else {
+        const bool in = 2 * l + 64 * e < C;
+        r.val[u][2 * e] = in ? row[2 * l + 64 * e] : 0.f;
+        r.val[u][2 * e + 1] = in ? row[2 * l + 64 * e + 1] : 0.f;
+      }
+    }
+  }
+}
+
+template <int TILES, bool FAST, int NT, typename Extra>
+__device__ __forceinline__ void ln_rows_store(const LnRows<TILES, NT>& r, const float* __restrict__ w,
+                                              const float* __restrict__ bsh, int C, const TileX3& t, Extra extra) {
+  constexpr int kGroups = NT / 32, ITERS = LnRows<TILES, NT>::ITERS;
   const int l = threadIdx.x & 31, grp = threadIdx.x >> 5;
   const int nE = C / 64;
   auto ok = [&](int e) { return FAST ? e < nE : 2 * l + 64 * e < C; };
@@ -276,56 +316,43 @@ __device__ __forceinline__ void layer_norm_tile_x3(Src src, const float* __restr
       bv[2 * e] = bsh[c], bv[2 * e + 1] = bsh[c + 1];
     }
   }
-  for (int it0 = 0; it0 < ITERS; it0 += 4) {
-    float val[4][8];
-    bool has[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const float* row = src(grp + (it0 + u) * kGroups);
-      has[u] = row != nullptr;
+  for (int u = 0; u < ITERS; ++u) {
+    const int pos = grp + u * kGroups;
+    float s = 0.f;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        val[u][2 * e] = val[u][2 * e + 1] = 0.f;
-        if (row && ok(e)) {
-          if (FAST) {
-            const float2 v = *reinterpret_cast<const float2*>(row + 2 * l + 64 * e);
-            val[u][2 * e] = v.x, val[u][2 * e + 1] = v.y;
-          } else {
-            val[u][2 * e] = row[2 * l + 64 * e], val[u][2 * e + 1] = row[2 * l + 64 * e + 1];
-          }
-        }
+    for (int e = 0; e < 8; ++e) s += r.val[u][e];  // channels past C hold 0
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, 32);
+    const float mean = s / (float)C;
+    float q = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (ok(e)) {
+        const float d0 = r.val[u][2 * e] - mean, d1 = r.val[u][2 * e + 1] - mean;
+        q += d0 * d0;
+        q += d1 * d1;
       }
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 32);
+    const float rstd = 1.0f / sqrtf(q / (float)C + kEps);
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      y[2 * e] = r.has[u] ? (r.val[u][2 * e] - mean) * rstd * wv[2 * e] + bv[2 * e] : 0.f;
+      y[2 * e + 1] = r.has[u] ? (r.val[u][2 * e + 1] - mean) * rstd * wv[2 * e + 1] + bv[2 * e + 1] : 0.f;
+      if (ok(e)) t.store2(pos, 2 * l + 64 * e, y[2 * e], y[2 * e + 1]);
     }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int pos = grp + (it0 + u) * kGroups;
-      float s = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) s += val[u][e];  // channels past C hold 0
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) s += __shfl_xor(s, o, 32);
-      const float mean = s / (float)C;
-      float q = 0.f;
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (ok(e)) {
-          const float d0 = val[u][2 * e] - mean, d1 = val[u][2 * e + 1] - mean;
-          q += d0 * d0;
-          q += d1 * d1;
-        }
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) q += __shfl_xor(q, o, 32);
-      const float rstd = 1.0f / sqrtf(q / (float)C + kEps);
-      float y[8];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        y[2 * e] = has[u] ? (val[u][2 * e] - mean) * rstd * wv[2 * e] + bv[2 * e] : 0.f;
-        y[2 * e + 1] = has[u] ? (val[u][2 * e + 1] - mean) * rstd * wv[2 * e + 1] + bv[2 * e + 1] : 0.f;
-        if (ok(e)) t.store2(pos, 2 * l + 64 * e, y[2 * e], y[2 * e + 1]);
-      }
-      extra(pos, y);
-    }
+    extra(pos, y);
   }
+}
+
+template <int TILES, bool FAST, int NT, typename Src, typename Extra>
+__device__ __forceinline__ void layer_norm_tile_x3(Src src, const float* __restrict__ w, const float* __restrict__ bsh,
+                                                   int C, const TileX3& t, Extra extra) {
+  LnRows<TILES, NT> r;
+  ln_rows_load<TILES, FAST, NT>(src, C, r);
+  ln_rows_store<TILES, FAST, NT>(r, w, bsh, C, t, extra);
 }
 struct NoExtra {
   __device__ __forceinline__ void operator()(int, const float (&)[8]) const {}
@@ -683,9 +710,10 @@ __global__ __launch_bounds__(kThreads * PT) void trimul_proj_x3_f32(TrimulF32 p,
   const int g = blockIdx.x % groups, r0 = ((blockIdx.x / groups) % row_groups) * PT, b = blockIdx.x / (groups * row_groups);
   const int k0 = g * KT;
   layer_norm_tile_x3<XT * PT, FAST, NT>(
-      [&](int pos) -> const float* {
+      [&](int pos, bool& valid) -> const float* {
         const int r = r0 + pos / KT, k = k0 + pos % KT;
-        return (r < N && k < N) ? p.z + b * p.zv.stride_b + r * p.zv.stride_r + k * p.zv.stride_k : nullptr;
+        valid = r < N && k < N;
+        return p.z + b * p.zv.stride_b + (r < N ? r : N - 1) * p.zv.stride_r + (k < N ? k : N - 1) * p.zv.stride_k;
       },
       p.ln_in_w, p.ln_in_b, C, xn, NoExtra{});
   if (threadIdx.x < TPX) {
@@ -922,9 +950,10 @@ __global__ __launch_bounds__(kThreads * PT) void trimul_out_x3_f32(TrimulF32 p, 
     }
   }
   layer_norm_tile_x3<XT * PT, FAST, NT>(
-      [&](int pos) -> const float* {
+      [&](int pos, bool& valid) -> const float* {
         const int j = j0 + pos;
-        return j < N ? p.z + b * p.zc.stride_b + i * p.zc.stride_r + j * p.zc.stride_k : nullptr;
+        valid = j < N;
+        return p.z + b * p.zc.stride_b + i * p.zc.stride_r + (j < N ? j : N - 1) * p.zc.stride_k;
       },
       p.ln_in_w, p.ln_in_b, C, zn, NoExtra{});
   __syncthreads();
@@ -1176,9 +1205,10 @@ __global__ __launch_bounds__(kThreads * PT) void triattn_proj_x3_f32(TriattnF32 
   const int j0 = g * TPX;
   const int l = threadIdx.x & 31;
   layer_norm_tile_x3<XT * PT, FAST, NT>(
-      [&](int pos) -> const float* {
+      [&](int pos, bool& valid) -> const float* {
         const int j = j0 + pos;
-        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+        valid = j < N;
+        return p.x + b * p.xv.stride_b + i * p.xv.stride_r + (j < N ? j : N - 1) * p.xv.stride_k;
       },
       p.ln_w, p.ln_b, C, xn, [&](int pos, const float(&y)[8]) {
         for (int h = 0; h < H; ++h) {
@@ -1280,9 +1310,10 @@ __global__ __launch_bounds__(kThreads * PT) void triattn_out_x3_f32(TriattnF32 p
   const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
   const int j0 = g * TPX;
   layer_norm_tile_x3<XT * PT, FAST, NT>(
-      [&](int pos) -> const float* {
+      [&](int pos, bool& valid) -> const float* {
         const int j = j0 + pos;
-        return j < N ? p.x + b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k : nullptr;
+        valid = j < N;
+        return p.x + b * p.xv.stride_b + i * p.xv.stride_r + (j < N ? j : N - 1) * p.xv.stride_k;
       },
       p.ln_w, p.ln_b, C, xn, NoExtra{});
   __syncthreads();
