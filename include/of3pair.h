@@ -191,6 +191,17 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
                        void* out, int64_t B, int64_t N, int64_t C, int64_t HID, int add_residual, int dtype,
                        void* stream);
 
+/* The same with a workspace (same reference lines): in fp32, with
+ * of3_transition_workspace_bytes_for(dtype, B, N, C, HID) bytes (256-byte aligned) for the weights
+ * split into three bf16 terms, C a multiple of 16 and HID a multiple of 128 run on the bf16 matrix
+ * instructions with fp32-grade products, as the triangle modules do; other shapes, a null workspace
+ * and bf16 (which needs none: 0 bytes) behave exactly like of3_transition_fwd. */
+int64_t of3_transition_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t HID);
+int of3_transition_fwd_ws(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
+                          const void* ln_w, const void* ln_b, const void* w_a, const void* w_b, const void* w_out,
+                          void* out, int64_t B, int64_t N, int64_t C, int64_t HID, int add_residual, void* workspace,
+                          int64_t workspace_bytes, int dtype, void* stream);
+
 /* ---- pair-bias projection ------------------------------------------------------------- */
 
 /* out[b][h][i][j] = sum_c LN(z[b,i,j,:])[c] * w[h][c]: the pair bias the single-representation

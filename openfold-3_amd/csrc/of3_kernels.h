@@ -243,9 +243,14 @@ struct TransitionF32Args {
   const float* mask;  // may be null
   PairView x_view, mask_view;
   const float *ln_w, *ln_b, *w_a, *w_b, *w_out;  // [C], [C], [HID][C], [HID][C], [C][HID]
+  void* wsplit;  // workspace, transition_wsplit_bytes(C, HID) bytes, 16-byte aligned; may be null (fp32 MFMA kernel)
   float* out;
   int B, N, C, HID, add_residual;
 };
+// the three weight matrices split into three bf16 terms each, rows padded to multiples of 32
+inline size_t transition_wsplit_bytes(long C, long HID) {
+  return (size_t)6 * (2 * wsplit_elems(HID, C) + wsplit_elems(C, HID));
+}
 hipError_t transition_fwd_f32(const TransitionF32Args& args, hipStream_t stream);
 
 struct PairBiasF32Args {

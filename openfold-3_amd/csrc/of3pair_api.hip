@@ -487,10 +487,24 @@ int of3_triattn_fwd(const void* x, const int64_t x_strides[3], const float* mask
   return of3_triattn_out(o, x, x_strides, out, ln_w, ln_b, w_g, w_o, B, N, C, H, D, add_residual, stream);
 }
 
+int64_t of3_transition_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t HID) {
+  if (dtype == OF3_DTYPE_BF16) return (B >= 1 && N >= 1) ? 0 : (int64_t)OF3_EINVAL;
+  if (dtype != OF3_DTYPE_F32 || B < 1 || N < 1 || C < 1 || C > 256 || HID < 1 || HID > 1024) return OF3_EINVAL;
+  return align256((int64_t)of3::transition_wsplit_bytes(C, HID));  // the weights split into three bf16 terms
+}
+
 int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
                        const void* ln_w, const void* ln_b, const void* w_a, const void* w_b, const void* w_out,
                        void* out, int64_t B, int64_t N, int64_t C, int64_t HID, int add_residual, int dtype,
                        void* stream) {
+  return of3_transition_fwd_ws(x, x_strides, mask, mask_strides, ln_w, ln_b, w_a, w_b, w_out, out, B, N, C, HID,
+                               add_residual, nullptr, 0, dtype, stream);
+}
+
+int of3_transition_fwd_ws(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
+                          const void* ln_w, const void* ln_b, const void* w_a, const void* w_b, const void* w_out,
+                          void* out, int64_t B, int64_t N, int64_t C, int64_t HID, int add_residual, void* workspace,
+                          int64_t workspace_bytes, int dtype, void* stream) {
   const void* ptrs[] = {x, ln_w, ln_b, w_a, w_b, w_out, out};
   if (!positions_ok(B, N) || !mask_ok(mask, mask_strides)) return OF3_EINVAL;
   if (dtype == OF3_DTYPE_F32) {
@@ -508,6 +522,13 @@ int of3_transition_fwd(const void* x, const int64_t x_strides[3], const float* m
     a.w_a = f(w_a);
     a.w_b = f(w_b);
     a.w_out = f(w_out);
+    // with room for the split weights the split-operand kernel runs (where the shape allows)
+    a.wsplit = nullptr;
+    if (workspace) {
+      if (reinterpret_cast<uintptr_t>(workspace) & 255u) return OF3_EINVAL;
+      if (workspace_bytes < of3_transition_workspace_bytes_for(dtype, B, N, C, HID)) return OF3_ENOSPC;
+      a.wsplit = workspace;
+    }
     a.out = static_cast<float*>(out);
     a.B = (int)B;
     a.N = (int)N;

@@ -362,21 +362,26 @@ struct NoExtra {
 // for all of them): K % 16 == 0, o0 a multiple of 32; lane (row or column l32, half lh) supplies the 8
 // consecutive k-values 16 s + 8 lh .. + 7 of step s, one 16-byte read per term and operand.  The
 // result layout of acc[n][xt] is that of linear_tiles for positions 32 xt .. 32 xt + 31.
-template <int NW, int XT, bool OUT_ROWS>
+// ACCUMULATE: acc is added to.  A slice of a wider weight matrix: w_step0 = its first k-step,
+// w_steps = the matrix's k-steps per row tile (0: K / 16, the whole width).
+template <int NW, int XT, bool OUT_ROWS, bool ACCUMULATE = false>
 __device__ __forceinline__ void linear_tiles_x3(const TileX3& xs, const WeightX3 (&W)[NW], int o0, int K,
-                                                f32x16_t (&acc)[NW][XT]) {
+                                                f32x16_t (&acc)[NW][XT], int w_step0 = 0, int w_steps = 0) {
   const int lane = threadIdx.x & 63, l32 = lane & 31, lh = lane >> 5;
   const int steps = K / 16;
+  if (w_steps == 0) w_steps = steps;
   const u32x4_t* xh = reinterpret_cast<const u32x4_t*>(xs.h + l32 * xs.ld + 8 * lh);
   const int xplane = xs.plane / 8, xtile = 32 * xs.ld / 8;  // in 16-byte units
   const u32x4_t* wh[NW];
   long wplane[NW];
 #pragma unroll
   for (int n = 0; n < NW; ++n) {
-    wh[n] = reinterpret_cast<const u32x4_t*>(W[n].h) + (size_t)(o0 >> 5) * steps * 64 + lane;
+    wh[n] = reinterpret_cast<const u32x4_t*>(W[n].h) + ((size_t)(o0 >> 5) * w_steps + w_step0) * 64 + lane;
     wplane[n] = W[n].plane / 8;
+    if (!ACCUMULATE) {
 #pragma unroll
-    for (int xt = 0; xt < XT; ++xt) acc[n][xt] = zero16();
+      for (int xt = 0; xt < XT; ++xt) acc[n][xt] = zero16();
+    }
   }
   for (int s = 0; s < steps; ++s) {
     u32x4_t x_h[XT], x_m[XT], x_l[XT];
@@ -1778,6 +1783,7 @@ struct TransitionF32 {
   const float *x, *mask;
   PairView xv, mv;
   const float *ln_w, *ln_b, *w_a, *w_b, *w_out;
+  WeightX3 s_a, s_b, s_out;  // split copies (transition_x3_f32 only)
   float* out;
   int B, N, C, HID, add_residual;
 };
@@ -1876,6 +1882,88 @@ __global__ __launch_bounds__(kThreads) void transition_mm_f32(TransitionF32 p, i
         const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
         if (p.add_residual) res = p.x[o] + res;
         p.out[o] = res;
+      }
+    }
+  }
+}
+
+// the same on split operands (C a multiple of 16, HID a multiple of 128), 32 positions per
+// work-group, the hidden dimension in slices of 128: a wave computes one 32-column tile of the slice
+// (both projections), writes silu(a) * b split into LDS, and adds the slice's share to its output tile
+constexpr int kTrHC = 128;
+template <bool WIDE, bool FAST>
+__global__ __launch_bounds__(kThreads) void transition_x3_f32(TransitionF32 p, int groups) {
+  extern __shared__ float smem[];
+  constexpr int MAXT = WIDE ? 2 : 1;
+  const int N = p.N, C = p.C, HID = p.HID;
+  const TileX3 xn = make_tile_x3(smem, C, kTP);
+  const TileX3 hid = make_tile_x3(reinterpret_cast<char*>(smem) + tile_bytes_x3(C, kTP), kTrHC, kTP);
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kTP;
+  const bool whole = j0 + kTP <= N;
+  layer_norm_tile_x3<1, FAST, kThreads>(
+      [&](int pos, bool& valid) -> const float* {
+        const int j = j0 + pos;
+        valid = j < N;
+        return p.x + b * p.xv.stride_b + i * p.xv.stride_r + (j < N ? j : N - 1) * p.xv.stride_k;
+      },
+      p.ln_w, p.ln_b, C, xn, NoExtra{});
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, l32 = lane & 31,
+            lh = lane >> 5;
+  f32x16_t out_acc[MAXT][1][1];
+#pragma unroll
+  for (int u = 0; u < MAXT; ++u) out_acc[u][0][0] = zero16();
+  const int n_ot = (C + 31) / 32;
+  for (int h0 = 0; h0 < HID; h0 += kTrHC) {
+    __syncthreads();  // xn is complete (first slice); nobody reads the previous slice any more
+    {
+      const WeightX3 W[2] = {p.s_a, p.s_b};
+      f32x16_t acc[2][1];
+      linear_tiles_x3<2, 1, false>(xn, W, h0 + 32 * wave, C, acc);
+      const int hd = 32 * wave + l32;
+#pragma unroll
+      for (int v = 0; v < 16; v += 2) {  // positions acc_row(v) and acc_row(v) + 1 of this lane's hidden channel
+        const float a0 = acc[0][0][v], a1 = acc[0][0][v + 1];
+        hid.store(acc_row(v, lh), hd, (a0 * sigmoid_hw_f32(a0)) * acc[1][0][v]);
+        hid.store(acc_row(v + 1, lh), hd, (a1 * sigmoid_hw_f32(a1)) * acc[1][0][v + 1]);
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < MAXT; ++u) {
+      const int t = wave + 4 * u;
+      if (t < n_ot) {
+        const WeightX3 W[1] = {p.s_out};
+        linear_tiles_x3<1, 1, false, true>(hid, W, 32 * t, kTrHC, out_acc[u], h0 / 16, HID / 16);
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < MAXT; ++u) {
+    const int t = wave + 4 * u, co = 32 * t + l32;
+    if (t >= n_ot) continue;
+    if (FAST && whole) {
+      const size_t lo = b * p.xv.stride_b + i * p.xv.stride_r + (size_t)(j0 + 4 * lh) * p.xv.stride_k + co;
+      const float* mp = p.mask ? p.mask + b * p.mv.stride_b + i * p.mv.stride_r + (j0 + 4 * lh) * p.mv.stride_k : nullptr;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int dj = 8 * (v >> 2) + (v & 3);
+        float res = out_acc[u][0][0][v];
+        if (mp) res *= mp[dj * p.mv.stride_k];
+        if (p.add_residual) res = p.x[lo + (size_t)dj * p.xv.stride_k] + res;
+        p.out[lo + (size_t)dj * p.xv.stride_k] = res;
+      }
+    } else {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int j = j0 + acc_row(v, lh);
+        if (co < C && j < N) {
+          float res = out_acc[u][0][0][v];
+          if (p.mask) res *= p.mask[b * p.mv.stride_b + i * p.mv.stride_r + j * p.mv.stride_k];
+          const size_t o = b * p.xv.stride_b + i * p.xv.stride_r + j * p.xv.stride_k + co;
+          if (p.add_residual) res = p.x[o] + res;
+          p.out[o] = res;
+        }
       }
     }
   }
@@ -2299,6 +2387,35 @@ hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
   p.C = a.C;
   p.HID = a.HID;
   p.add_residual = a.add_residual;
+  if (a.C % 16 == 0 && a.HID % kTrHC == 0 && a.wsplit && aligned16({a.wsplit})) {
+    bf16_t* w = static_cast<bf16_t*>(a.wsplit);
+    auto split = [&](const float* src, int rows, int K, WeightX3& dst) {
+      dst.h = w;
+      dst.plane = packed_elems(rows, K);
+      const long items = dst.plane / 8;
+      hipLaunchKernelGGL(split_weights_f32, dim3((unsigned)((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream,
+                         src, w, rows, K);
+      w += 3 * dst.plane;
+    };
+    split(a.w_a, a.HID, a.C, p.s_a);
+    split(a.w_b, a.HID, a.C, p.s_b);
+    split(a.w_out, a.C, a.HID, p.s_out);
+    const bool fast = a.C % 64 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 7u) == 0 && even_strides(a.x_view);
+    const bool wide = a.C > 128;
+    auto kern = wide ? (fast ? transition_x3_f32<true, true> : transition_x3_f32<true, false>)
+                     : (fast ? transition_x3_f32<false, true> : transition_x3_f32<false, false>);
+    hipError_t e = allow_lds(transition_x3_f32<false, false>, 0, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(transition_x3_f32<false, true>, 1, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(transition_x3_f32<true, false>, 2, kLdsLimit);
+    if (e == hipSuccess) e = allow_lds(transition_x3_f32<true, true>, 3, kLdsLimit);
+    if (e != hipSuccess) return e;
+    const int mgroups = (a.N + kTP - 1) / kTP;
+    const long mblocks = (long)a.B * a.N * mgroups;
+    if (mblocks > 0x7fffffffL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kern, dim3((unsigned)mblocks), dim3(kThreads), tile_bytes_x3(a.C, kTP) + tile_bytes_x3(kTrHC, kTP),
+                       stream, p, mgroups);
+    return hipGetLastError();
+  }
   if (a.C % 8 == 0 && a.HID % 8 == 0 && aligned16({a.w_a, a.w_b, a.w_out})) {
     // hidden slice: as wide as keeps three work-groups on a CU (about 52 KB of LDS each)
     int hchunk = (int)((52 * 1024 - tile_bytes(a.C)) / (kTP * sizeof(float))) - 4;

@@ -210,10 +210,13 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
     keep = [_w(t, x.dtype) for t in (norm_weight, norm_bias, a_weight, b_weight, out_weight)]
     m3, mptr, mstr = _mask_arg(mask, lead, B, N, x.device)
     out4 = x4 if inplace else _out_like(x4)
+    need = lib.of3_transition_workspace_bytes_for(code, B, N, C, HID)  # fp32: room for the split weights
+    ws = _workspace(x.device, need) if need > 0 else None
     with torch.cuda.device(x.device):
-        st = lib.of3_transition_fwd(x4.data_ptr(), _lib.strides3(x4.stride()[:3]), mptr, mstr,
-                                    *[k.data_ptr() for k in keep], out4.data_ptr(), B, N, C, HID,
-                                    int(bool(add_residual)), code, _stream(x))
+        st = lib.of3_transition_fwd_ws(x4.data_ptr(), _lib.strides3(x4.stride()[:3]), mptr, mstr,
+                                       *[k.data_ptr() for k in keep], out4.data_ptr(), B, N, C, HID,
+                                       int(bool(add_residual)), ws.data_ptr() if ws is not None else None,
+                                       need if ws is not None else 0, code, _stream(x))
     if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and C <= 256 and HID <= 1024:
         return _through_fp32(swiglu_transition, x, inplace, mask, norm_weight, norm_bias, a_weight, b_weight, out_weight,
                              add_residual=add_residual)

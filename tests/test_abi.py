@@ -242,3 +242,17 @@ def test_transition_rows_entry_point_validates(lib):
     nul = list(args)
     nul[4] = None
     assert lib.of3_transition_rows_fwd(*nul, L.OF3_DTYPE_BF16, None) == L.OF3_EINVAL
+
+def test_transition_workspace_variant_validates_on_the_host(lib):
+    """of3_transition_fwd_ws: the fp32 workspace holds the weights split into three bf16 terms; bf16 needs none."""
+    from of3pair import _lib as L
+
+    assert lib.of3_transition_workspace_bytes_for(L.OF3_DTYPE_BF16, 1, 64, 128, 512) == 0
+    need = lib.of3_transition_workspace_bytes_for(L.OF3_DTYPE_F32, 1, 64, 128, 512)
+    assert need == 6 * 3 * 512 * 128
+    assert lib.of3_transition_workspace_bytes_for(L.OF3_DTYPE_F32, 1, 64, 300, 512) == L.OF3_EINVAL
+    assert lib.of3_transition_workspace_bytes_for(7, 1, 64, 128, 512) == L.OF3_EINVAL
+    xs = _s3(64 * 64 * 128, 64 * 128, 128)
+    args = (FAKE, xs, None, None, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 1, 64, 128, 512, 1)
+    assert lib.of3_transition_fwd_ws(*args, FAKE, need - 1, L.OF3_DTYPE_F32, None) == L.OF3_ENOSPC
+    assert lib.of3_transition_fwd_ws(*args, FAKE + 4, need, L.OF3_DTYPE_F32, None) == L.OF3_EINVAL  # workspace alignment

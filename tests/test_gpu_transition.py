@@ -104,7 +104,8 @@ def test_transition_deterministic_and_side_stream():
     assert torch.equal(a, b) and torch.equal(a, c)
 
 
-@pytest.mark.parametrize("c,n_mult,n,batch", [(128, 4, 33, ()), (96, 2, 20, (2,)), (64, 4, 50, ())])
+@pytest.mark.parametrize("c,n_mult,n,batch", [(128, 4, 33, ()), (96, 2, 20, (2,)), (64, 4, 50, ()), (48, 8, 40, (2,)), (256, 2, 37, ()),
+                                              (128, 4, 160, ())])
 def test_transition_fp32(c, n_mult, n, batch):
     lib()
     gen = torch.Generator().manual_seed(400 + n)
