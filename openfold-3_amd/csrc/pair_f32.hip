@@ -2075,7 +2075,7 @@ bool aligned16(std::initializer_list<const void*> ptrs) {
 inline bool even_strides(const PairView& v) { return ((v.stride_b | v.stride_r | v.stride_k) & 1) == 0; }
 
 // the largest tiles exceed the default dynamic LDS limit: raised to max_bytes once per device and
-// kernel (slot = index of the kernel's cache)
+// kernel
 constexpr size_t kLdsLimit = 160 * 1024;
 #ifndef OF3_X3_XT
 #define OF3_X3_XT 1
@@ -2086,15 +2086,15 @@ constexpr int kXT = OF3_X3_XT;  // 32-position tiles per wave of the split-opera
 #endif
 constexpr int kPT = OF3_X3_PT;  // groups of four waves per work-group, each with its own positions: waves of different
                                 // groups read the same weights at about the same time, once from L2
-template <typename Kern>
-hipError_t allow_lds(Kern kern, int slot, size_t max_bytes = 3 * (size_t)kTP * (kMaxC + 4) * sizeof(float)) {
-  static int cache[16][kMaxDevices];
+template <auto Kern>
+hipError_t allow_lds(size_t max_bytes = 3 * (size_t)kTP * (kMaxC + 4) * sizeof(float)) {
+  static int cache[kMaxDevices];  // one per kernel: Kern is part of the function's identity
   int done = 0;
   return per_device(
-      cache[slot],
+      cache,
       [&](int, int* v) {
         *v = 1;
-        return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)max_bytes);
       },
       &done);
@@ -2197,22 +2197,22 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
     split(a.w_z, a.C, a.CH, p.s_z);
     auto proj = split_ab ? (fast ? trimul_proj_x3_f32<kXT, kPT, true, true> : trimul_proj_x3_f32<kXT, kPT, false, true>)
                          : (fast ? trimul_proj_x3_f32<kXT, kPT, true, false> : trimul_proj_x3_f32<kXT, kPT, false, false>);
-    hipError_t e = allow_lds(trimul_proj_x3_f32<kXT, kPT, false, false>, 4, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, kPT, true, false>, 11, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, kPT, false, true>, 14, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_proj_x3_f32<kXT, kPT, true, true>, 15, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, kPT, false, false>, 5, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, kPT, true, false>, 6, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, kPT, false, true>, 12, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_out_x3_f32<kXT, kPT, true, true>, 13, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(trimul_contract_x3_f32, 0, kLdsLimit);
+    hipError_t e = allow_lds<trimul_proj_x3_f32<kXT, kPT, false, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<trimul_proj_x3_f32<kXT, kPT, true, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<trimul_proj_x3_f32<kXT, kPT, false, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<trimul_proj_x3_f32<kXT, kPT, true, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<trimul_out_x3_f32<kXT, kPT, false, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<trimul_out_x3_f32<kXT, kPT, true, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<trimul_out_x3_f32<kXT, kPT, false, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<trimul_out_x3_f32<kXT, kPT, true, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<trimul_contract_x3_f32>(kLdsLimit);
     if (e != hipSuccess) return e;
     const size_t lds = tile_bytes_x3(a.C, 32 * kXT * kPT) + 32 * kXT * kPT * sizeof(float);
     const int kgroups = (a.N + 32 * kXT - 1) / (32 * kXT), row_groups = (a.N + kPT - 1) / kPT;
     hipLaunchKernelGGL(proj, dim3((unsigned)((long)a.B * row_groups * kgroups)), dim3(kThreads * kPT), lds, stream, p, kgroups);
   } else if (mm) {
-    hipError_t e = allow_lds(trimul_proj_mm_f32, 0);
-    if (e == hipSuccess) e = allow_lds(trimul_out_mm_f32, 1);
+    hipError_t e = allow_lds<trimul_proj_mm_f32>();
+    if (e == hipSuccess) e = allow_lds<trimul_out_mm_f32>();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(trimul_proj_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C) + kTP * sizeof(float), stream,
                        p, mgroups);
@@ -2318,21 +2318,21 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     split(a.w_o, a.C, HD, p.s_o);
     auto proj = core_x3 ? (fast ? triattn_proj_x3_f32<kXT, kPT, true, true> : triattn_proj_x3_f32<kXT, kPT, true, false>)
                         : (fast ? triattn_proj_x3_f32<kXT, kPT, false, true> : triattn_proj_x3_f32<kXT, kPT, false, false>);
-    hipError_t e = allow_lds(triattn_proj_x3_f32<kXT, kPT, false, false>, 7, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, kPT, true, false>, 10, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, kPT, false, true>, 11, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_proj_x3_f32<kXT, kPT, true, true>, 12, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, kPT, false, false>, 8, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, kPT, true, false>, 9, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, kPT, false, true>, 13, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_out_x3_f32<kXT, kPT, true, true>, 14, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(triattn_core_x3_f32, 0, kLdsLimit);
+    hipError_t e = allow_lds<triattn_proj_x3_f32<kXT, kPT, false, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_proj_x3_f32<kXT, kPT, true, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_proj_x3_f32<kXT, kPT, false, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_proj_x3_f32<kXT, kPT, true, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, false, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, true, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, false, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, true, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_core_x3_f32>(kLdsLimit);
     if (e != hipSuccess) return e;
     const size_t lds = tile_bytes_x3(a.C, 32 * kXT * kPT) + (size_t)a.H * 32 * kXT * kPT * sizeof(float);
     hipLaunchKernelGGL(proj, dim3(xblocks), dim3(kThreads * kPT), lds, stream, p, xgroups);
   } else if (mm) {
-    hipError_t e = allow_lds(triattn_proj_mm_f32, 2);
-    if (e == hipSuccess) e = allow_lds(triattn_out_mm_f32, 3);
+    hipError_t e = allow_lds<triattn_proj_mm_f32>();
+    if (e == hipSuccess) e = allow_lds<triattn_out_mm_f32>();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(triattn_proj_mm_f32, dim3(mblocks), dim3(kThreads), tile_bytes(a.C), stream, p, mgroups);
   } else {
@@ -2404,10 +2404,10 @@ hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
     const bool wide = a.C > 128;
     auto kern = wide ? (fast ? transition_x3_f32<true, true> : transition_x3_f32<true, false>)
                      : (fast ? transition_x3_f32<false, true> : transition_x3_f32<false, false>);
-    hipError_t e = allow_lds(transition_x3_f32<false, false>, 0, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(transition_x3_f32<false, true>, 1, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(transition_x3_f32<true, false>, 2, kLdsLimit);
-    if (e == hipSuccess) e = allow_lds(transition_x3_f32<true, true>, 3, kLdsLimit);
+    hipError_t e = allow_lds<transition_x3_f32<false, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<transition_x3_f32<false, true>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<transition_x3_f32<true, false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<transition_x3_f32<true, true>>(kLdsLimit);
     if (e != hipSuccess) return e;
     const int mgroups = (a.N + kTP - 1) / kTP;
     const long mblocks = (long)a.B * a.N * mgroups;
@@ -2423,7 +2423,7 @@ hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
     if (hchunk < 32) hchunk = 32;
     if (hchunk > a.HID) hchunk = (a.HID + 31) / 32 * 32;
     const size_t mm_bytes = tile_bytes(a.C) + tile_bytes(hchunk);
-    hipError_t e = allow_lds(transition_mm_f32, 0, kLdsLimit);
+    hipError_t e = allow_lds<transition_mm_f32>(kLdsLimit);
     if (e != hipSuccess) return e;
     const int mgroups = (a.N + kTP - 1) / kTP;
     const long mblocks = (long)a.B * a.N * mgroups;
