@@ -135,3 +135,33 @@ def test_fp32_random_shapes(seed):
     pa = orc.make_triattn_params(gen, c, 32, heads)
     got = _load(of3pair.TriangleAttention(c, 32, heads, starting=starting), pa)(z.to(DEV), mask=None if mask is None else mask.to(DEV))
     _maxerr("triattn fp32 random", got, orc.triattn_update(z, mask, pa, heads, starting=starting))
+
+
+@pytest.mark.parametrize("kind", ["offset", "odd_stride", "transposed"])
+def test_fp32_views(kind):
+    """fp32 inputs that are views: a pair tensor that starts 4 bytes into its storage, one whose position
+    stride is odd (both leave the 8-byte row alignment the fast kernels ask for), and a transposed one."""
+    lib()
+    n, c, d, heads = 70, 128, 32, 4
+    gen = torch.Generator().manual_seed(77)
+    z = torch.randn(n, n, c, generator=gen)
+    mask = (torch.rand(n, n, generator=gen) > 0.15).float()
+    if kind == "offset":
+        buf = torch.zeros(n * n * c + 1, device=DEV)
+        zg = buf[1:].view(n, n, c)
+        zg.copy_(z)
+    elif kind == "odd_stride":
+        buf = torch.zeros(n, n, c + 1, device=DEV)
+        zg = buf[:, :, :c]
+        zg.copy_(z)
+    else:
+        zg = z.transpose(0, 1).contiguous().to(DEV).transpose(0, 1)
+    assert not zg.is_contiguous() or kind == "offset"
+    print("fp32 view %s strides %s offset %d" % (kind, zg.stride(), zg.storage_offset()), flush=True)
+    pm = orc.make_trimul_params(gen, c, c)
+    got = _load(of3pair.TriangleMultiplicationIncoming(c, c), pm)(zg, mask=mask.to(DEV))
+    _maxerr("trimul fp32 view", got, orc.trimul_update(z, mask, pm, False))
+    pa = orc.make_triattn_params(gen, c, d, heads)
+    got = _load(of3pair.TriangleAttention(c, d, heads, starting=False), pa)(zg, mask=mask.to(DEV))
+    _maxerr("triattn fp32 view", got, orc.triattn_update(z, mask, pa, heads, starting=False))
+    assert torch.equal(zg.cpu(), z), "the input view is left as it was"
