@@ -33,7 +33,8 @@ def _load(module, params):
 @pytest.mark.parametrize("outgoing", [True, False])
 @pytest.mark.parametrize("c,ch,n,batch,masked", [(128, 128, 64, (1,), False), (64, 64, 45, (2,), True), (96, 40, 33, (), True),
                                                   (36, 20, 19, (), True),  # channel counts off the multiples of 8: the plain FMA kernels
-                                                  (48, 80, 29, (2,), True), (256, 64, 40, (), False)])  # multiples of 16, not of 64; more than 128 channels
+                                                  (48, 80, 29, (2,), True), (256, 64, 40, (), False),  # multiples of 16, not of 64; more than 128 channels
+                                                  (16, 16, 9, (), True), (64, 256, 35, (), True)])  # the narrowest and the widest hidden width
 def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
     lib()
     gen = torch.Generator().manual_seed(300 + n)
@@ -51,7 +52,8 @@ def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
 @pytest.mark.parametrize("c,d,heads,n,batch,masked", [(128, 32, 4, 64, (1,), False), (64, 16, 4, 45, (2,), True),
                                                      (48, 64, 2, 37, (), True), (36, 16, 3, 21, (), True),
                                                      (64, 32, 2, 150, (), True),  # more than one 128-query group
-                                                     (128, 32, 4, 44, (2,), True), (32, 32, 1, 129, (), False)])
+                                                     (128, 32, 4, 44, (2,), True), (32, 32, 1, 129, (), False),
+                                                     (16, 32, 1, 9, (), True), (256, 32, 8, 40, (), True)])  # narrowest and widest
 def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
     lib()
     gen = torch.Generator().manual_seed(400 + n)
