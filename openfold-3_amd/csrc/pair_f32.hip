@@ -230,13 +230,29 @@ struct WeightX3 {
 };
 __host__ __device__ constexpr long packed_elems(long rows, long K) { return (rows + 31) / 32 * 32 * K; }
 
-__global__ __launch_bounds__(kThreads) void split_weights_f32(const float* __restrict__ src, bf16_t* __restrict__ dst,
-                                                              int rows, int K) {
-  // one thread per (row tile, step, lane): its 8 consecutive k-values
+// up to six matrices in one launch
+struct SplitJobs {
+  static constexpr int kMax = 6;
+  const float* src[kMax];
+  bf16_t* dst[kMax];
+  int rows[kMax], K[kMax];
+  long first[kMax + 1];  // first item of each matrix; first[n] = all items
+  int n;
+};
+
+__global__ __launch_bounds__(kThreads) void split_weights_f32(SplitJobs j) {
+  // one thread per (matrix, row tile, step, lane): its 8 consecutive k-values
+  const long gitem = (long)blockIdx.x * kThreads + threadIdx.x;
+  if (gitem >= j.first[j.n]) return;
+  int q = 0;
+#pragma unroll
+  for (int i = 1; i < SplitJobs::kMax; ++i)
+    if (i < j.n && gitem >= j.first[i]) q = i;
+  const float* __restrict__ src = j.src[q];
+  bf16_t* __restrict__ dst = j.dst[q];
+  const int rows = j.rows[q], K = j.K[q];
+  const long item = gitem - j.first[q];
   const int steps = K / 16;
-  const long item = (long)blockIdx.x * kThreads + threadIdx.x;
-  const long n_items = (long)((rows + 31) / 32) * steps * 64;
-  if (item >= n_items) return;
   const int lane = (int)(item & 63), l32 = lane & 31, lh = lane >> 5;
   const long ts = item >> 6;
   const int s = (int)(ts % steps), t = (int)(ts / steps);
@@ -251,6 +267,28 @@ __global__ __launch_bounds__(kThreads) void split_weights_f32(const float* __res
     dst[2 * plane + item * 8 + e] = v.l;
   }
 }
+
+// host side: matrices are added one after the other into the workspace, then split by one launch
+struct WeightSplitter {
+  SplitJobs j;
+  bf16_t* w;
+  explicit WeightSplitter(void* workspace) : j(), w(static_cast<bf16_t*>(workspace)) {}
+  void add(const float* src, int rows, int K, WeightX3& dst) {
+    dst.h = w;
+    dst.plane = packed_elems(rows, K);
+    j.src[j.n] = src;
+    j.dst[j.n] = w;
+    j.rows[j.n] = rows;
+    j.K[j.n] = K;
+    j.first[j.n + 1] = j.first[j.n] + dst.plane / 8;
+    ++j.n;
+    w += 3 * dst.plane;
+  }
+  void launch(hipStream_t stream) const {
+    const long items = j.first[j.n];
+    hipLaunchKernelGGL(split_weights_f32, dim3((unsigned)((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, j);
+  }
+};
 
 // LayerNorm of 32 * TILES positions by NT threads into a split tile, a row per 32 lanes, at most 256 channels (a
 // multiple of 16).  Lane l holds channels 2 l + 64 e and 2 l + 64 e + 1, e < 4.  A row is read once
@@ -2180,21 +2218,14 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
   const int xgroups = (a.N + 32 * kXT * kPT - 1) / (32 * kXT * kPT);
   const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
   if (x3) {
-    bf16_t* w = static_cast<bf16_t*>(a.wsplit);
-    auto split = [&](const float* src, int rows, int K, WeightX3& dst) {
-      dst.h = w;
-      dst.plane = packed_elems(rows, K);
-      const long items = dst.plane / 8;
-      hipLaunchKernelGGL(split_weights_f32, dim3((unsigned)((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream,
-                         src, w, rows, K);
-      w += 3 * dst.plane;
-    };
-    split(a.w_ap, a.CH, a.C, p.s_ap);
-    split(a.w_ag, a.CH, a.C, p.s_ag);
-    split(a.w_bp, a.CH, a.C, p.s_bp);
-    split(a.w_bg, a.CH, a.C, p.s_bg);
-    split(a.w_g, a.C, a.C, p.s_g);
-    split(a.w_z, a.C, a.CH, p.s_z);
+    WeightSplitter splitter(a.wsplit);
+    splitter.add(a.w_ap, a.CH, a.C, p.s_ap);
+    splitter.add(a.w_ag, a.CH, a.C, p.s_ag);
+    splitter.add(a.w_bp, a.CH, a.C, p.s_bp);
+    splitter.add(a.w_bg, a.CH, a.C, p.s_bg);
+    splitter.add(a.w_g, a.C, a.C, p.s_g);
+    splitter.add(a.w_z, a.C, a.CH, p.s_z);
+    splitter.launch(stream);
     auto proj = split_ab ? (fast ? trimul_proj_x3_f32<kXT, kPT, true, true> : trimul_proj_x3_f32<kXT, kPT, false, true>)
                          : (fast ? trimul_proj_x3_f32<kXT, kPT, true, false> : trimul_proj_x3_f32<kXT, kPT, false, false>);
     hipError_t e = allow_lds<trimul_proj_x3_f32<kXT, kPT, false, false>>(kLdsLimit);
@@ -2301,21 +2332,14 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   const int xgroups = (a.N + 32 * kXT * kPT - 1) / (32 * kXT * kPT);
   const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
   if (x3) {
-    bf16_t* w = static_cast<bf16_t*>(a.wsplit);
-    auto split = [&](const float* src, int rows, int K, WeightX3& dst) {
-      dst.h = w;
-      dst.plane = packed_elems(rows, K);
-      const long items = dst.plane / 8;
-      hipLaunchKernelGGL(split_weights_f32, dim3((unsigned)((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream,
-                         src, w, rows, K);
-      w += 3 * dst.plane;
-    };
+    WeightSplitter splitter(a.wsplit);
     const int HD = a.H * a.D;
-    split(a.w_q, HD, a.C, p.s_q);
-    split(a.w_k, HD, a.C, p.s_k);
-    split(a.w_v, HD, a.C, p.s_v);
-    split(a.w_g, HD, a.C, p.s_g);
-    split(a.w_o, a.C, HD, p.s_o);
+    splitter.add(a.w_q, HD, a.C, p.s_q);
+    splitter.add(a.w_k, HD, a.C, p.s_k);
+    splitter.add(a.w_v, HD, a.C, p.s_v);
+    splitter.add(a.w_g, HD, a.C, p.s_g);
+    splitter.add(a.w_o, a.C, HD, p.s_o);
+    splitter.launch(stream);
     auto proj = core_x3 ? (fast ? triattn_proj_x3_f32<kXT, kPT, true, true> : triattn_proj_x3_f32<kXT, kPT, true, false>)
                         : (fast ? triattn_proj_x3_f32<kXT, kPT, false, true> : triattn_proj_x3_f32<kXT, kPT, false, false>);
     hipError_t e = allow_lds<triattn_proj_x3_f32<kXT, kPT, false, false>>(kLdsLimit);
@@ -2388,18 +2412,11 @@ hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
   p.HID = a.HID;
   p.add_residual = a.add_residual;
   if (a.C % 16 == 0 && a.HID % kTrHC == 0 && a.wsplit && aligned16({a.wsplit})) {
-    bf16_t* w = static_cast<bf16_t*>(a.wsplit);
-    auto split = [&](const float* src, int rows, int K, WeightX3& dst) {
-      dst.h = w;
-      dst.plane = packed_elems(rows, K);
-      const long items = dst.plane / 8;
-      hipLaunchKernelGGL(split_weights_f32, dim3((unsigned)((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream,
-                         src, w, rows, K);
-      w += 3 * dst.plane;
-    };
-    split(a.w_a, a.HID, a.C, p.s_a);
-    split(a.w_b, a.HID, a.C, p.s_b);
-    split(a.w_out, a.C, a.HID, p.s_out);
+    WeightSplitter splitter(a.wsplit);
+    splitter.add(a.w_a, a.HID, a.C, p.s_a);
+    splitter.add(a.w_b, a.HID, a.C, p.s_b);
+    splitter.add(a.w_out, a.C, a.HID, p.s_out);
+    splitter.launch(stream);
     const bool fast = a.C % 64 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 7u) == 0 && even_strides(a.x_view);
     const bool wide = a.C > 128;
     auto kern = wide ? (fast ? transition_x3_f32<true, true> : transition_x3_f32<true, false>)
