@@ -167,3 +167,22 @@ def test_fp32_views(kind):
     got = _load(of3pair.TriangleAttention(c, d, heads, starting=False), pa)(zg, mask=mask.to(DEV))
     _maxerr("triattn fp32 view", got, orc.triattn_update(z, mask, pa, heads, starting=False))
     assert torch.equal(zg.cpu(), z), "the input view is left as it was"
+
+
+def test_block_fp32_is_deterministic():
+    """no atomics, no run-to-run ordering: two calls (one on another stream) give the same bits."""
+    lib()
+    n, c, d, heads = 200, 128, 32, 4
+    p = orc.make_block_params(5, c, c, d, heads)
+    m = _load(of3pair.PairStack(c, c, d, heads), p)
+    z = orc.make_pair_input(9, (1,), n, c).to(DEV)
+    mask = orc.tail_padding_mask((1,), n, torch.tensor([17])).to(DEV)
+    a = m(z, mask)
+    b = m(z, mask)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        c2 = m(z, mask)
+    s.synchronize()
+    torch.cuda.synchronize()
+    assert torch.equal(a, b) and torch.equal(a, c2)
