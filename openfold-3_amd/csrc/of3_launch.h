@@ -46,4 +46,20 @@ inline hipError_t resident_blocks(Kernel kern, int threads, int dev, int* out) {
   return hipSuccess;
 }
 
+// lets work-groups of Kern ask for up to max_bytes of dynamic LDS (beyond the 64 KB a kernel may use
+// without asking); once per kernel and device
+template <auto Kern>
+inline hipError_t allow_dynamic_lds(size_t max_bytes) {
+  static int cache[kMaxDevices];  // one per kernel: Kern is part of the function's identity
+  int done = 0;
+  return per_device(
+      cache,
+      [&](int, int* v) {
+        *v = 1;
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)max_bytes);
+      },
+      &done);
+}
+
 }  // namespace of3

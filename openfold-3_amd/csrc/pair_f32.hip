@@ -2126,16 +2126,7 @@ constexpr int kPT = OF3_X3_PT;  // groups of four waves per work-group, each wit
                                 // groups read the same weights at about the same time, once from L2
 template <auto Kern>
 hipError_t allow_lds(size_t max_bytes = 3 * (size_t)kTP * (kMaxC + 4) * sizeof(float)) {
-  static int cache[kMaxDevices];  // one per kernel: Kern is part of the function's identity
-  int done = 0;
-  return per_device(
-      cache,
-      [&](int, int* v) {
-        *v = 1;
-        return hipFuncSetAttribute(reinterpret_cast<const void*>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   (int)max_bytes);
-      },
-      &done);
+  return allow_dynamic_lds<Kern>(max_bytes);
 }
 
 }  // namespace

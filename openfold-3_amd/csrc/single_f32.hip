@@ -1,9 +1,11 @@
 // fp32 versions of the single-representation kernels (AttentionPairBias of the trunk,
 // attention_pair_bias.py:189-244, and the SwiGLU transition over s, transition.py:225-271): plain
 // fp32 FMA arithmetic in the reference's order of operations, any N, C_s <= 512, head width
-// <= 64, hidden width <= 2048.  The precision path, not a fast one.
+// <= 64, hidden width <= 2048.  The precision path, not a fast one: the linear layers give a thread
+// one output channel and stage the weights through LDS, the attention gives a thread one query.
 #include "of3_device.h"
 #include "of3_kernels.h"
+#include "of3_launch.h"
 
 namespace of3 {
 
@@ -21,14 +23,95 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
   return v;
 }
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
-__device__ __forceinline__ float dot_f32(const float* __restrict__ x, const float* __restrict__ w, int n) {
-  float acc = 0.f;
-  for (int k = 0; k < n; ++k) acc = fmaf(x[k], w[k], acc);
-  return acc;
+
+// ---- linear layers over kRows rows held in LDS -----------------------------------------------------
+// y[r][o] = sum_k xs[r][k] W[o][k], k ascending, one fused multiply-add per term.  Thread t owns output
+// o0 + t of a tile of kThreads outputs.  The weights of a tile come through LDS in pieces of kWK inputs:
+// 16 lanes read 256 contiguous bytes of a weight row (a thread walking its own row would touch 64
+// cache lines per wave instruction), the piece is stored with a row stride of kWK + 1 words, so that
+// both the staging stores and the per-thread row reads are free of bank conflicts, and the next piece
+// is already on its way in registers while the current one is multiplied.  xs must be readable and
+// zero up to the next multiple of kWK past K: whole pieces are multiplied, the padding adds zeros.
+constexpr int kWK = 64;
+constexpr int kWLd = kWK + 1;
+constexpr int kWLoads = kWK / 4;  // 16-byte pieces per thread and tile piece (kThreads rows of kWK / 4 pieces)
+constexpr size_t kWTileBytes = (size_t)kThreads * kWLd * sizeof(float);
+
+__device__ __forceinline__ int round_up_wk(int n) { return (n + kWK - 1) / kWK * kWK; }
+
+template <bool VEC, int LD, class Epilogue>
+__device__ __forceinline__ void rows_linear_impl(const float (*xs)[LD], const float* __restrict__ W, int n_out, int K,
+                                                 float* wt, Epilogue&& epilogue) {
+  const int t = threadIdx.x;
+  for (int o0 = 0; o0 < n_out; o0 += kThreads) {
+    float4 nxt[kWLoads];
+    // every load is issued whatever the lane's position: addresses are clamped into the matrix, and
+    // what lies outside is masked to zero bit-wise when the piece goes to LDS, after the products of
+    // the piece before (a load or a replacement under a lane condition makes the compiler wait for all
+    // loads in flight where the lanes join, and a mask applied here would wait for them at once)
+    auto fetch = [&](int k0) {
+#pragma unroll
+      for (int i = 0; i < kWLoads; ++i) {
+        const int idx = t + i * kThreads, row = idx >> 4, k = k0 + 4 * (idx & 15), o = o0 + row;
+        const float* src = W + (size_t)(o < n_out ? o : n_out - 1) * K;
+        if (VEC) {  // K is a multiple of 4: a piece lies inside the row or outside
+          nxt[i] = *reinterpret_cast<const float4*>(src + (k < K ? k : K - 4));
+        } else {
+          nxt[i].x = src[k < K ? k : K - 1];
+          nxt[i].y = src[k + 1 < K ? k + 1 : K - 1];
+          nxt[i].z = src[k + 2 < K ? k + 2 : K - 1];
+          nxt[i].w = src[k + 3 < K ? k + 3 : K - 1];
+        }
+      }
+    };
+    auto to_lds = [&](int k0) {
+#pragma unroll
+      for (int i = 0; i < kWLoads; ++i) {
+        const int idx = t + i * kThreads, row = idx >> 4, k = k0 + 4 * (idx & 15), o = o0 + row;
+        float* dst = wt + row * kWLd + 4 * (idx & 15);
+        const float v[4] = {nxt[i].x, nxt[i].y, nxt[i].z, nxt[i].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned keep = o < n_out && k + (VEC ? 0 : j) < K ? ~0u : 0u;
+          dst[j] = __uint_as_float(__float_as_uint(v[j]) & keep);
+        }
+      }
+    };
+    float acc[kRows];
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) acc[r] = 0.f;
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += kWK) {
+      __syncthreads();  // the previous piece has been multiplied by everybody
+      to_lds(k0);
+      __syncthreads();
+      if (k0 + kWK < K) fetch(k0 + kWK);
+      const float* wrow = wt + t * kWLd;
+#pragma unroll 4
+      for (int kk = 0; kk < kWK; kk += 4) {
+        const float w0 = wrow[kk], w1 = wrow[kk + 1], w2 = wrow[kk + 2], w3 = wrow[kk + 3];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r) {
+          const float4 x = *reinterpret_cast<const float4*>(&xs[r][k0 + kk]);  // one address per wave: a broadcast
+          acc[r] = fmaf(x.x, w0, acc[r]);
+          acc[r] = fmaf(x.y, w1, acc[r]);
+          acc[r] = fmaf(x.z, w2, acc[r]);
+          acc[r] = fmaf(x.w, w3, acc[r]);
+        }
+      }
+    }
+    if (o0 + t < n_out) epilogue(o0 + t, acc);
+  }
+}
+template <int LD, class Epilogue>
+__device__ __forceinline__ void rows_linear(const float (*xs)[LD], const float* __restrict__ W, int n_out, int K,
+                                            float* wt, Epilogue&& epilogue) {
+  if ((K & 3) == 0 && (reinterpret_cast<uintptr_t>(W) & 15u) == 0) rows_linear_impl<true>(xs, W, n_out, K, wt, epilogue);
+  else rows_linear_impl<false>(xs, W, n_out, K, wt, epilogue);
 }
 
 // LayerNorm of rows pos0 .. pos0+kRows-1 of src [rows][C] into xn (two-pass statistics); rows
-// past n_rows give zeros
+// past n_rows give zeros, and so do the channels from C to the next multiple of kWK
 __device__ __forceinline__ void norm_rows(const float* __restrict__ src, long pos0, long n_rows, int C,
                                           const float* __restrict__ w, const float* __restrict__ b,
                                           float (*xn)[kMaxCs]) {
@@ -46,26 +129,30 @@ __device__ __forceinline__ void norm_rows(const float* __restrict__ src, long po
       q += d * d;
     }
   const float rstd = 1.0f / sqrtf(wave_sum_f32(q) / (float)C + kEps);
-  for (int c = l; c < C; c += 64) xn[r][c] = x ? (x[c] - mean) * rstd * w[c] + b[c] : 0.f;
+  for (int c = l; c < round_up_wk(C); c += 64) xn[r][c] = x && c < C ? (x[c] - mean) * rstd * w[c] + b[c] : 0.f;
 }
 
 // q (bias added, then / sqrt(D)), k, v and the gate after the sigmoid, all [B*N][H*D]
 __global__ __launch_bounds__(kThreads) void single_proj_f32(SingleAttnF32Args p) {
-  __shared__ float xn[kRows][kMaxCs];
+  __shared__ __align__(16) float xn[kRows][kMaxCs];
+  extern __shared__ float wt[];
   const long rows = (long)p.B * p.N, pos0 = (long)blockIdx.x * kRows;
   const int C = p.C, HD = p.H * p.D;
   norm_rows(p.a, pos0, rows, C, p.ln_w, p.ln_b, xn);
-  __syncthreads();
   const float scale = 1.0f / sqrtf((float)p.D);
-  for (int idx = threadIdx.x; idx < kRows * 4 * HD; idx += kThreads) {
-    const int r = idx / (4 * HD), o = idx % (4 * HD), kind = o / HD, ch = o % HD;
-    if (pos0 + r >= rows) continue;
+  for (int kind = 0; kind < 4; ++kind) {
     const float* W = kind == 0 ? p.wq : kind == 1 ? p.wk : kind == 2 ? p.wv : p.wg;
-    float v = dot_f32(xn[r], W + (size_t)ch * C, C);
-    if (kind == 0) v = (v + p.bq[ch]) * scale;
-    if (kind == 3) v = sigmoid_f32(v);
     float* dst = kind == 0 ? p.q : kind == 1 ? p.k : kind == 2 ? p.v : p.g;
-    dst[(pos0 + r) * HD + ch] = v;
+    rows_linear(xn, W, HD, C, wt, [&](int ch, const float (&acc)[kRows]) {
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        if (pos0 + r >= rows) continue;
+        float v = acc[r];
+        if (kind == 0) v = (v + p.bq[ch]) * scale;
+        if (kind == 3) v = sigmoid_f32(v);
+        dst[(pos0 + r) * HD + ch] = v;
+      }
+    });
   }
 }
 
@@ -145,47 +232,59 @@ __global__ __launch_bounds__(128) void single_attn_f32(SingleAttnF32Args p) {
 }
 
 __global__ __launch_bounds__(kThreads) void single_out_f32(SingleAttnF32Args p) {
-  __shared__ float og[kRows][kMaxCs];
+  __shared__ __align__(16) float og[kRows][kMaxCs];
+  extern __shared__ float wt[];
   const long rows = (long)p.B * p.N, pos0 = (long)blockIdx.x * kRows;
-  const int C = p.C, HD = p.H * p.D;
-  for (int idx = threadIdx.x; idx < kRows * HD; idx += kThreads) {
-    const int r = idx / HD, c = idx % HD;
-    og[r][c] = pos0 + r < rows ? p.og[(pos0 + r) * HD + c] : 0.f;
+  const int C = p.C, HD = p.H * p.D, hd_pad = round_up_wk(HD);
+  for (int idx = threadIdx.x; idx < kRows * hd_pad; idx += kThreads) {
+    const int r = idx / hd_pad, c = idx % hd_pad;
+    og[r][c] = pos0 + r < rows && c < HD ? p.og[(pos0 + r) * HD + c] : 0.f;
   }
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < kRows * C; idx += kThreads) {
-    const int r = idx / C, o = idx % C;
-    if (pos0 + r >= rows) continue;
-    float v = dot_f32(og[r], p.wo + (size_t)o * HD, HD);
-    if (p.add_residual) v = p.a[(pos0 + r) * C + o] + v;
-    p.out[(pos0 + r) * C + o] = v;
-  }
+  rows_linear(og, p.wo, C, HD, wt, [&](int o, const float (&acc)[kRows]) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      if (pos0 + r >= rows) continue;
+      float v = acc[r];
+      if (p.add_residual) v = p.a[(pos0 + r) * C + o] + v;
+      p.out[(pos0 + r) * C + o] = v;
+    }
+  });
 }
 
 // out = [x +] ((silu(LN(x) Wa^T) * (LN(x) Wb^T)) Wout^T) * mask for kRows rows per work-group; the
 // hidden activations stay in LDS
 __global__ __launch_bounds__(kThreads) void row_transition_f32(RowTransitionF32Args p) {
-  __shared__ float xn[kRows][kMaxCs];
-  __shared__ float hid[kRows][kMaxHidden];
+  __shared__ __align__(16) float xn[kRows][kMaxCs];
+  __shared__ __align__(16) float hid[kRows][kMaxHidden];
+  extern __shared__ float wt[];
   const long pos0 = (long)blockIdx.x * kRows;
   const int C = p.C, HID = p.HID;
   norm_rows(p.x, pos0, p.rows, C, p.ln_w, p.ln_b, xn);
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < kRows * HID; idx += kThreads) {
-    const int r = idx / HID, o = idx % HID;
-    const float a = dot_f32(xn[r], p.wa + (size_t)o * C, C);
-    const float b = dot_f32(xn[r], p.wb + (size_t)o * C, C);
-    hid[r][o] = (a * sigmoid_f32(a)) * b;  // silu(a) * b (activations.py:60-61)
-  }
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < kRows * C; idx += kThreads) {
-    const int r = idx / C, o = idx % C;
-    if (pos0 + r >= p.rows) continue;
-    float v = dot_f32(hid[r], p.wout + (size_t)o * HID, HID);
-    if (p.mask) v = v * p.mask[pos0 + r];
-    if (p.add_residual) v = p.x[(pos0 + r) * C + o] + v;
-    p.out[(pos0 + r) * C + o] = v;
-  }
+  for (int idx = HID + threadIdx.x; idx < round_up_wk(HID); idx += kThreads)
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) hid[r][idx] = 0.f;
+  // a thread writes a and then silu(a) * b into the same words of hid: no barrier between the two
+  rows_linear(xn, p.wa, HID, C, wt, [&](int o, const float (&acc)[kRows]) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) hid[r][o] = acc[r];
+  });
+  rows_linear(xn, p.wb, HID, C, wt, [&](int o, const float (&acc)[kRows]) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const float a = hid[r][o];
+      hid[r][o] = (a * sigmoid_f32(a)) * acc[r];  // silu(a) * b (activations.py:60-61)
+    }
+  });
+  rows_linear(hid, p.wout, C, HID, wt, [&](int o, const float (&acc)[kRows]) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      if (pos0 + r >= p.rows) continue;
+      float v = acc[r];
+      if (p.mask) v = v * p.mask[pos0 + r];
+      if (p.add_residual) v = p.x[(pos0 + r) * C + o] + v;
+      p.out[(pos0 + r) * C + o] = v;
+    }
+  });
 }
 
 }  // namespace
@@ -197,15 +296,18 @@ hipError_t single_attn_fwd_f32(const SingleAttnF32Args& a, hipStream_t stream) {
   const long rows = (long)a.B * a.N;
   const long blocks = (rows + kRows - 1) / kRows;
   if (blocks > 0x7fffffffl) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(single_proj_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
-  hipError_t e = hipGetLastError();
+  hipError_t e = allow_dynamic_lds<single_proj_f32>(kWTileBytes);
+  if (e == hipSuccess) e = allow_dynamic_lds<single_out_f32>(kWTileBytes);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(single_proj_f32, dim3((unsigned)blocks), dim3(kThreads), kWTileBytes, stream, a);
+  e = hipGetLastError();
   if (e != hipSuccess) return e;
   const dim3 grid((a.N + 127) / 128, a.H, a.B);
   if (a.D <= 32) hipLaunchKernelGGL(single_attn_f32<32>, grid, dim3(128), 0, stream, a);
   else hipLaunchKernelGGL(single_attn_f32<64>, grid, dim3(128), 0, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(single_out_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+  hipLaunchKernelGGL(single_out_f32, dim3((unsigned)blocks), dim3(kThreads), kWTileBytes, stream, a);
   return hipGetLastError();
 }
 
@@ -213,7 +315,9 @@ hipError_t row_transition_fwd_f32(const RowTransitionF32Args& a, hipStream_t str
   if (a.rows < 1 || a.C < 1 || a.C > kMaxCs || a.HID < 1 || a.HID > kMaxHidden) return hipErrorInvalidValue;
   const long blocks = (a.rows + kRows - 1) / kRows;
   if (blocks > 0x7fffffffl) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(row_transition_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, a);
+  const hipError_t e = allow_dynamic_lds<row_transition_f32>(kWTileBytes);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(row_transition_f32, dim3((unsigned)blocks), dim3(kThreads), kWTileBytes, stream, a);
   return hipGetLastError();
 }
 
