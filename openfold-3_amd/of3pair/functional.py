@@ -196,10 +196,11 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
     add_residual.  x [*, N, N, C], mask [*, N, N] or None; a_weight / b_weight [n*C, C] are
     SwiGLU's linear_a (through SiLU) and linear_b, out_weight [C, n*C].  With C = 384 (the single
     representation) x is [*, 384] and mask [*]: any leading dimensions (the transition is
-    position-wise, so a pair tensor of 384 channels takes that route too and gets the same result)."""
+    position-wise, so a pair tensor of 384 channels takes that route too and gets the same result).
+    A tensor of fewer than three dimensions cannot be a pair tensor and is taken as rows [*, C] too."""
     code = _require_gpu(x, "x")
     lib = _lib.load()
-    if x.shape[-1] == 384:  # the single representation: position-wise over [*, 384] rows
+    if x.shape[-1] == 384 or x.dim() < 3:  # the single representation: position-wise over [*, C] rows
         return _swiglu_transition_rows(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_weight,
                                        add_residual, inplace, code)
     x4, lead = _flatten_pair(x)

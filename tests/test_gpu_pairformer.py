@@ -83,14 +83,16 @@ def test_single_transition_in_place_on_a_strided_view():
     assert torch.equal(wg[:, 0].float().cpu(), wide[:, 0]), "the other rows of the storage are untouched"
 
 
-@pytest.mark.parametrize("shape,n_mult", [((50,), 4), ((2, 19), 2)])
-def test_single_transition_fp32(shape, n_mult):
+@pytest.mark.parametrize("shape,n_mult,c", [((50,), 4, 384), ((2, 19), 2, 384), ((23,), 3, 90), ((9,), 5, 62)])
+def test_single_transition_fp32(shape, n_mult, c):
+    """Widths that are no multiples of 4 take the kernels' scalar weight reads, hidden widths that are
+    no multiples of 64 their zero padding."""
     lib()
     gen = torch.Generator().manual_seed(940 + shape[-1])
-    p = orc.make_transition_params(gen, 384, n_mult)
-    x = 1.5 * torch.randn(*shape, 384, generator=gen) + 0.1
+    p = orc.make_transition_params(gen, c, n_mult)
+    x = 1.5 * torch.randn(*shape, c, generator=gen) + 0.1
     mask = (torch.rand(*shape, generator=gen) > 0.25).float()
-    m = of3pair.SwiGLUTransition(384, n_mult)
+    m = of3pair.SwiGLUTransition(c, n_mult)
     m.load_state_dict(p, strict=True)
     m = m.to(DEV).eval()
     got = m(x.to(DEV), mask=mask.to(DEV))

@@ -111,7 +111,8 @@ def test_attention_pair_bias_rejects_unsupported():
 
 
 @pytest.mark.parametrize("n,batch,c_s,c_head,heads,masked", [(37, (), 384, 24, 16, True), (130, (2,), 96, 12, 8, True),
-                                                             (16, (), 256, 64, 4, False)])
+                                                             (16, (), 256, 64, 4, False), (21, (), 90, 10, 9, True),
+                                                             (11, (3,), 70, 7, 10, False)])
 def test_attention_pair_bias_fp32(n, batch, c_s, c_head, heads, masked):
     """fp32 (the reference's default inference precision): max-abs 1e-4 against the oracle."""
     lib()
