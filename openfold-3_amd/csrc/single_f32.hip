@@ -156,16 +156,21 @@ __global__ __launch_bounds__(kThreads) void single_proj_f32(SingleAttnF32Args p)
   }
 }
 
-// one thread per query of one (batch, head); keys in chunks of 32 through LDS together with the
-// [128 queries][32 keys] slice of the pair bias; online softmax; output times gate
+// 32 queries of one (batch, head) per work-group, four threads per query: keys in chunks of 32 through
+// LDS together with the [32 queries][32 keys] slice of the pair bias, thread (query, part) takes keys
+// 8 part .. 8 part + 7 of every chunk with a running softmax of its own; the four partial results of a
+// query are merged at the end; output times gate
+constexpr int kAttnQ = 32, kAttnParts = 4;
 template <int DMAX>
-__global__ __launch_bounds__(128) void single_attn_f32(SingleAttnF32Args p) {
-  constexpr int KC = 32;
+__global__ __launch_bounds__(kAttnQ * kAttnParts) void single_attn_f32(SingleAttnF32Args p) {
+  constexpr int KC = 32, KP = KC / kAttnParts, NT = kAttnQ * kAttnParts;
   __shared__ float ks[KC][DMAX], vs[KC][DMAX], mbs[KC];
-  __shared__ float pbs[128][KC + 1];
+  __shared__ float pbs[kAttnQ][KC + 1];
+  __shared__ float part_o[kAttnParts][kAttnQ][DMAX + 1], part_m[kAttnParts][kAttnQ], part_l[kAttnParts][kAttnQ];
   const int N = p.N, H = p.H, D = p.D, HD = H * D;
   const int qg = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int qi = qg * 128 + threadIdx.x;
+  const int ql = threadIdx.x % kAttnQ, part = threadIdx.x / kAttnQ;
+  const int qi = qg * kAttnQ + ql;
   const bool active = qi < N;
   float qv[DMAX], ov[DMAX];
 #pragma unroll
@@ -173,19 +178,20 @@ __global__ __launch_bounds__(128) void single_attn_f32(SingleAttnF32Args p) {
     qv[d] = (active && d < D) ? p.q[((size_t)b * N + qi) * HD + h * D + d] : 0.f;
     ov[d] = 0.f;
   }
-  const float* pb = p.pair_bias + (((size_t)b * H + h) * N + (size_t)qg * 128) * N;
-  float m = -__builtin_inff(), l = 0.f;
+  const float* pb = p.pair_bias + (((size_t)b * H + h) * N + (size_t)qg * kAttnQ) * N;
+  const float ninf = -__builtin_inff();
+  float m = ninf, l = 0.f;
   for (int k0 = 0; k0 < N; k0 += KC) {
     __syncthreads();
-    for (int e = threadIdx.x; e < KC * DMAX; e += 128) {
+    for (int e = threadIdx.x; e < KC * DMAX; e += NT) {
       const int kk = e / DMAX, d = e % DMAX;
       const bool in = k0 + kk < N && d < D;
       ks[kk][d] = in ? p.k[((size_t)b * N + k0 + kk) * HD + h * D + d] : 0.f;
       vs[kk][d] = in ? p.v[((size_t)b * N + k0 + kk) * HD + h * D + d] : 0.f;
     }
-    for (int e = threadIdx.x; e < 128 * KC; e += 128) {
+    for (int e = threadIdx.x; e < kAttnQ * KC; e += NT) {
       const int r = e / KC, c = e % KC;
-      pbs[r][c] = (qg * 128 + r < N && k0 + c < N) ? pb[(size_t)r * N + k0 + c] : 0.f;
+      pbs[r][c] = (qg * kAttnQ + r < N && k0 + c < N) ? pb[(size_t)r * N + k0 + c] : 0.f;
     }
     if (threadIdx.x < KC) {
       const int kx = k0 + threadIdx.x;
@@ -195,35 +201,56 @@ __global__ __launch_bounds__(128) void single_attn_f32(SingleAttnF32Args p) {
     }
     __syncthreads();
     const int kn = N - k0 < KC ? N - k0 : KC;
-    float s[KC];
-    float cmax = -__builtin_inff();
+    float s[KP];
+    float cmax = ninf;
 #pragma unroll
-    for (int kk = 0; kk < KC; ++kk) {
+    for (int j = 0; j < KP; ++j) {
+      const int kk = part * KP + j;
       float acc = 0.f;
 #pragma unroll
       for (int d = 0; d < DMAX; ++d) acc = fmaf(qv[d], ks[kk][d], acc);
       // logits in the reference's order: q.k, then the mask bias, then the pair bias
       acc = acc + mbs[kk];
-      acc = acc + pbs[threadIdx.x][kk];
-      s[kk] = kk < kn ? acc : -__builtin_inff();
-      cmax = fmaxf(cmax, s[kk]);
+      acc = acc + pbs[ql][kk];
+      s[j] = kk < kn ? acc : ninf;
+      cmax = fmaxf(cmax, s[j]);
     }
+    if (cmax == ninf) continue;  // none of this thread's keys of the chunk exists (the barriers are above)
     const float m_new = fmaxf(m, cmax);
-    const float alpha = expf(m - m_new);
+    const float alpha = expf(m - m_new);  // 0 the first time (m = -inf, m_new finite)
     l *= alpha;
 #pragma unroll
     for (int d = 0; d < DMAX; ++d) ov[d] *= alpha;
 #pragma unroll
-    for (int kk = 0; kk < KC; ++kk) {
-      const float pw = expf(s[kk] - m_new);
+    for (int j = 0; j < KP; ++j) {
+      const float pw = expf(s[j] - m_new);  // 0 for a key that does not exist
       l += pw;
 #pragma unroll
-      for (int d = 0; d < DMAX; ++d) ov[d] = fmaf(pw, vs[kk][d], ov[d]);
+      for (int d = 0; d < DMAX; ++d) ov[d] = fmaf(pw, vs[part * KP + j][d], ov[d]);
     }
     m = m_new;
   }
-  if (active) {
-    const float inv = 1.0f / l;
+  // merge the parts of a query: a part that saw no key has m = -inf, l = 0 and weighs nothing
+  part_m[part][ql] = m;
+  part_l[part][ql] = l;
+#pragma unroll
+  for (int d = 0; d < DMAX; ++d) part_o[part][ql][d] = ov[d];
+  __syncthreads();
+  if (part == 0 && active) {
+    float mm = ninf;
+#pragma unroll
+    for (int q = 0; q < kAttnParts; ++q) mm = fmaxf(mm, part_m[q][ql]);
+    float lsum = 0.f;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d) ov[d] = 0.f;
+#pragma unroll
+    for (int q = 0; q < kAttnParts; ++q) {
+      const float w = part_m[q][ql] == ninf ? 0.f : expf(part_m[q][ql] - mm);
+      lsum = fmaf(part_l[q][ql], w, lsum);
+#pragma unroll
+      for (int d = 0; d < DMAX; ++d) ov[d] = fmaf(part_o[q][ql][d], w, ov[d]);
+    }
+    const float inv = 1.0f / lsum;
     const size_t off = ((size_t)b * N + qi) * HD + h * D;
 #pragma unroll
     for (int d = 0; d < DMAX; ++d)
@@ -302,9 +329,9 @@ hipError_t single_attn_fwd_f32(const SingleAttnF32Args& a, hipStream_t stream) {
   hipLaunchKernelGGL(single_proj_f32, dim3((unsigned)blocks), dim3(kThreads), kWTileBytes, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
-  const dim3 grid((a.N + 127) / 128, a.H, a.B);
-  if (a.D <= 32) hipLaunchKernelGGL(single_attn_f32<32>, grid, dim3(128), 0, stream, a);
-  else hipLaunchKernelGGL(single_attn_f32<64>, grid, dim3(128), 0, stream, a);
+  const dim3 grid((a.N + kAttnQ - 1) / kAttnQ, a.H, a.B);
+  if (a.D <= 32) hipLaunchKernelGGL(single_attn_f32<32>, grid, dim3(kAttnQ * kAttnParts), 0, stream, a);
+  else hipLaunchKernelGGL(single_attn_f32<64>, grid, dim3(kAttnQ * kAttnParts), 0, stream, a);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(single_out_f32, dim3((unsigned)blocks), dim3(kThreads), kWTileBytes, stream, a);
