@@ -2042,6 +2042,78 @@ __global__ __launch_bounds__(kThreads) void pair_bias_f32(PairBiasF32 p, int gro
   }
 }
 
+// the same on split operands (C a multiple of 16, H <= 32): one wave per 32 positions of a row and no
+// other wave in the work-group, so that a CU holds as many independent tiles as its LDS has room for.
+// The weights are few (H rows): a lane splits the eight values of its operand for a step on the way,
+// the values of the next step being read while the current one is multiplied; head h is row h of
+// the accumulator tile, the position its column: a head's 32 positions are one 128-byte store.
+template <bool FAST>
+__global__ __launch_bounds__(64) void pair_bias_x3_f32(PairBiasF32 p, int groups) {
+  extern __shared__ float smem[];
+  const int N = p.N, C = p.C, H = p.H;
+  const TileX3 xn = make_tile_x3(smem, C, kTP);
+  float* zero_bias = reinterpret_cast<float*>(reinterpret_cast<char*>(smem) + tile_bytes_x3(C, kTP));  // [C]
+  const int g = blockIdx.x % groups, i = (blockIdx.x / groups) % N, b = blockIdx.x / (groups * N);
+  const int j0 = g * kTP;
+  const int lane = threadIdx.x, l32 = lane & 31, lh = lane >> 5;
+  const float* lb = p.ln_b;
+  if (!lb) {
+    for (int c = lane; c < C; c += 64) zero_bias[c] = 0.f;
+    __syncthreads();
+    lb = zero_bias;
+  }
+  // this lane's weight operand: row min(l32, H - 1) (the rows from H on are dropped), k = 16 s + 8 lh ..
+  const float* wrow = p.w + (size_t)(l32 < H ? l32 : H - 1) * C + 8 * lh;
+  const bool wvec = (reinterpret_cast<uintptr_t>(p.w) & 15u) == 0;  // C % 16 == 0: every operand is then 16-byte aligned
+  float wn[8];
+  auto read_w = [&](int s) {
+    if (wvec) {
+      const float4 u = *reinterpret_cast<const float4*>(wrow + 16 * s), v = *reinterpret_cast<const float4*>(wrow + 16 * s + 4);
+      wn[0] = u.x, wn[1] = u.y, wn[2] = u.z, wn[3] = u.w, wn[4] = v.x, wn[5] = v.y, wn[6] = v.z, wn[7] = v.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) wn[e] = wrow[16 * s + e];
+    }
+  };
+  read_w(0);
+  layer_norm_tile_x3<1, FAST, 64>(
+      [&](int pos, bool& valid) -> const float* {
+        const int j = j0 + pos;
+        valid = j < N;
+        return p.z + b * p.zv.stride_b + i * p.zv.stride_r + (j < N ? j : N - 1) * p.zv.stride_k;
+      },
+      p.ln_w, lb, C, xn, NoExtra{});
+  __syncthreads();
+  const u32x4_t* xh = reinterpret_cast<const u32x4_t*>(xn.h + l32 * xn.ld + 8 * lh);
+  const int xplane = xn.plane / 8;
+  // the small terms and the large ones in accumulators of their own: two chains of dependent MFMAs
+  // instead of one, and the small terms are summed among themselves before they meet the large ones
+  f32x16_t acc = zero16(), acc_small = zero16();
+  const int steps = C / 16;
+  for (int s = 0; s < steps; ++s) {
+    u32x4_t w_h, w_m, w_l;
+    split8(wn, w_h, w_m, w_l);
+    if (s + 1 < steps) read_w(s + 1);
+    const u32x4_t x_h = xh[2 * s], x_m = xh[xplane + 2 * s], x_l = xh[2 * xplane + 2 * s];
+    acc_small = mfma_32x32x16(w_l, x_h, acc_small);
+    acc = mfma_32x32x16(w_m, x_h, acc);
+    acc_small = mfma_32x32x16(w_h, x_l, acc_small);
+    acc = mfma_32x32x16(w_h, x_m, acc);
+    acc_small = mfma_32x32x16(w_m, x_m, acc_small);
+    acc = mfma_32x32x16(w_h, x_h, acc);
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] += acc_small[v];
+  const int j = j0 + l32;
+  if (j < N) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int h = acc_row(v, lh);
+      if (h < H) p.out[(((size_t)b * H + h) * N + i) * N + j] = acc[v];
+    }
+  }
+}
+
 // ---- template branch: closing LayerNorm of the stack and the mean / ReLU / linear_t tail -------
 struct TemplateTailF32 {
   const float *t, *ln_w, *ln_b, *w;
@@ -2458,6 +2530,18 @@ hipError_t pair_bias_fwd_f32(const PairBiasF32Args& a, hipStream_t stream) {
   p.N = a.N;
   p.C = a.C;
   p.H = a.H;
+  if (a.C % 16 == 0 && a.H <= 32) {
+    const bool fast = a.C % 64 == 0 && (reinterpret_cast<uintptr_t>(a.z) & 7u) == 0 && even_strides(a.z_view);
+    hipError_t e = allow_lds<pair_bias_x3_f32<false>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<pair_bias_x3_f32<true>>(kLdsLimit);
+    if (e != hipSuccess) return e;
+    const int mgroups = (a.N + kTP - 1) / kTP;
+    const long mblocks = (long)a.B * a.N * mgroups;
+    if (mblocks > 0x7fffffffL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fast ? pair_bias_x3_f32<true> : pair_bias_x3_f32<false>, dim3((unsigned)mblocks), dim3(64),
+                       tile_bytes_x3(a.C, kTP) + a.C * sizeof(float), stream, p, mgroups);
+    return hipGetLastError();
+  }
   const int groups = (a.N + kP - 1) / kP;
   const long blocks = (long)a.B * a.N * groups;
   hipLaunchKernelGGL(pair_bias_f32, dim3((unsigned)blocks), dim3(kThreads), 0, stream, p, groups);
