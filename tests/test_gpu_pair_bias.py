@@ -72,7 +72,8 @@ def test_pair_bias_full_size_sampled():
     _check("pair bias rows at N=768", got[0][:, rows].permute(1, 0, 2), want[:, :, 0])
 
 
-@pytest.mark.parametrize("c,h,n,batch,offset", [(128, 16, 33, (), True), (96, 5, 20, (2,), False), (256, 64, 9, (), True)])
+@pytest.mark.parametrize("c,h,n,batch,offset", [(128, 16, 33, (), True), (96, 5, 20, (2,), False), (256, 64, 9, (), True),
+                                                     (40, 3, 17, (), False), (64, 32, 70, (2,), True)])
 def test_pair_bias_fp32(c, h, n, batch, offset):
     lib()
     gen = torch.Generator().manual_seed(900 + n)
