@@ -233,9 +233,10 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& args, hipStream_t stream);
 inline size_t triattn_wsplit_bytes(long C, long H, long D) {
   return (size_t)6 * (4 * wsplit_elems(H * D, C) + wsplit_elems(C, H * D));
 }
-// q, k and v^T in three bf16 terms each, rows padded to whole 32-position tiles
+// q, k and v^T in three bf16 terms each, rows padded to whole 32-position tiles; v^T operands always
+// have 32 rows (head widths below 32 leave the rest zero)
 inline size_t triattn_qkv_split_bytes(long B, long N, long H, long D) {
-  return (size_t)18 * B * N * H * ((N + 31) / 32 * 32) * D;
+  return (size_t)6 * B * N * H * ((N + 31) / 32 * 32) * (2 * D + (D > 32 ? D : 32));
 }
 
 struct TransitionF32Args {

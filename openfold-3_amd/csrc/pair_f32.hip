@@ -1096,9 +1096,11 @@ struct TriattnF32 {
   float *q, *k, *v, *tb, *o, *out;
   // q, k and v^T split into three bf16 terms and stored as MFMA operands (the split-operand core only):
   // the 16 bytes of lane l for step s of 32-position tile t of (b, i, h) are slot
-  // (((b N + i) H + h) * Jp / 32 + t) * 2 + s) * 64 + l of a plane, planes qkv_plane elements apart
+  // (((b N + i) H + h) * Jp / 32 + t) * steps + s) * 64 + l of a plane.  q and k have D / 16 steps (16
+  // head channels each) and planes of qk_plane elements; v^T always has two steps (16 keys each) of 32
+  // rows, the rows from D on being zero, and planes of v_plane elements
   bf16_t *qs, *ks, *vs;
-  long qkv_plane;
+  long qk_plane, v_plane;
   int Jp;  // N rounded up to whole 32-position tiles
   int B, N, C, H, D, add_residual;
   float inf;
@@ -1231,8 +1233,8 @@ __global__ __launch_bounds__(kThreads) void triattn_out_mm_f32(TriattnF32 p, int
 // The two position-wise passes of the attention on split operands (channel counts that are multiples
 // of 16), 32 * XT positions per work-group.  The H rows of the triangle bias are too few for a matrix
 // tile: they are fp32 dot products taken on the normalised row while it is in registers.
-// SPLIT (head width 32): q, k and v leave as operands of the split-operand core instead of fp32 arrays.
-// A 32-column tile of the projections is one head.  q and k are computed with the head channels in
+// SPLIT (head width 32 or 16): q, k and v leave as operands of the split-operand core instead of fp32 arrays.
+// A 32-column tile of the projections is one head, or two of width 16.  q and k are computed with the head channels in
 // the accumulator rows and the positions in the lanes, v the other way round: in both cases registers
 // 8 s .. 8 s + 7 of a lane are its operand for step s (q, k: head channels 16 s + 4 lh + r and
 // 16 s + 8 + 4 lh + r, the same for both, so the order inside the dot product does not matter;
@@ -1285,22 +1287,52 @@ __global__ __launch_bounds__(kThreads * PT) void triattn_proj_x3_f32(TriattnF32 
   for (int t = jw; t < (HD + 31) / 32; t += 4) {
     const int o0 = 32 * t;
     if (SPLIT) {
-      // positions past N were normalised to zero rows: their q, k and v are zeros, and are stored
-      const size_t slot0 = ((((size_t)b * N + i) * H + t) * (p.Jp / 32) + (j0 + pb) / 32) * 128 + lane;
-      const long plane = p.qkv_plane / 8;
-      auto store = [&](bf16_t* dst, const f32x16_t& acc, int xt, float mul) {
+      // positions past N were normalised to zero rows: their q, k and v are zeros, and are stored.
+      // Head width 32: tile t is head t.  Head width 16: tile t is heads 2 t and 2 t + 1; step st of the
+      // q / k tile is the one step of head 2 t + st, and lane l32 of the v tile is row l32 % 16 of head
+      // 2 t + l32 / 16, whose rows 16 .. 31 are written as zeros.
+      const bool narrow = D == 16;
+      const int nt = p.Jp / 32, jt0 = (j0 + pb) / 32;
+      const size_t bi = (size_t)b * N + i;
+      auto split_regs = [&](const f32x16_t& acc, int st, float mul, u32x4_t& h, u32x4_t& m, u32x4_t& lo) {
+        float x[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = acc[8 * st + e] * mul;
+        split8(x, h, m, lo);
+      };
+      auto store_qk = [&](bf16_t* dst, const f32x16_t& acc, int xt, float mul) {
         if (j0 + pb + 32 * xt >= p.Jp) return;  // a tile past the padded row (XT > 1 only)
-        u32x4_t* d4 = reinterpret_cast<u32x4_t*>(dst) + slot0 + xt * 128;
+        const long plane = p.qk_plane / 8;
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
-          float x[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) x[e] = acc[8 * st + e] * mul;
+          const size_t slot = narrow ? ((bi * H + 2 * t + st) * nt + jt0 + xt) * 64 + lane
+                                     : (((bi * H + t) * nt + jt0 + xt) * 2 + st) * 64 + lane;
+          u32x4_t* d4 = reinterpret_cast<u32x4_t*>(dst) + slot;
           u32x4_t h, m, lo;
-          split8(x, h, m, lo);
-          d4[st * 64] = h;
-          d4[plane + st * 64] = m;
-          d4[2 * plane + st * 64] = lo;
+          split_regs(acc, st, mul, h, m, lo);
+          d4[0] = h;
+          d4[plane] = m;
+          d4[2 * plane] = lo;
+        }
+      };
+      auto store_v = [&](const f32x16_t& acc, int xt) {
+        if (j0 + pb + 32 * xt >= p.Jp) return;
+        const long plane = p.v_plane / 8;
+        const int head = narrow ? 2 * t + (l32 >> 4) : t, vrow = narrow ? (l32 & 15) : l32;
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          u32x4_t* d4 = reinterpret_cast<u32x4_t*>(p.vs) + (((bi * H + head) * nt + jt0 + xt) * 2 + st) * 64 + vrow + 32 * lh;
+          u32x4_t h, m, lo;
+          split_regs(acc, st, 1.f, h, m, lo);
+          d4[0] = h;
+          d4[plane] = m;
+          d4[2 * plane] = lo;
+          if (narrow) {
+            const u32x4_t zero = {0u, 0u, 0u, 0u};
+            d4[16] = zero;
+            d4[plane + 16] = zero;
+            d4[2 * plane + 16] = zero;
+          }
         }
       };
       {
@@ -1309,8 +1341,8 @@ __global__ __launch_bounds__(kThreads * PT) void triattn_proj_x3_f32(TriattnF32 
         linear_tiles_x3<2, XT, true>(xn.at(pb), W, o0, C, acc);
 #pragma unroll
         for (int xt = 0; xt < XT; ++xt) {
-          store(p.qs, acc[0][xt], xt, scale);  // q / sqrt(c) after the projection (attention.py:283-284)
-          store(p.ks, acc[1][xt], xt, 1.f);
+          store_qk(p.qs, acc[0][xt], xt, scale);  // q / sqrt(c) after the projection (attention.py:283-284)
+          store_qk(p.ks, acc[1][xt], xt, 1.f);
         }
       }
       {
@@ -1318,7 +1350,7 @@ __global__ __launch_bounds__(kThreads * PT) void triattn_proj_x3_f32(TriattnF32 
         f32x16_t acc[1][XT];
         linear_tiles_x3<1, XT, false>(xn.at(pb), W, o0, C, acc);
 #pragma unroll
-        for (int xt = 0; xt < XT; ++xt) store(p.vs, acc[0][xt], xt, 1.f);
+        for (int xt = 0; xt < XT; ++xt) store_v(acc[0][xt], xt);
       }
     } else {
       const int hd = o0 + l32, h = hd / D, d = hd - h * D;
@@ -1432,7 +1464,8 @@ __global__ __launch_bounds__(kThreads * PT) void triattn_out_x3_f32(TriattnF32 p
   }
 }
 
-// Attention core on split operands, head width 32.  Work-group = 8 waves = 4 consecutive rows i x 2
+// Attention core on split operands, head width 16 * STEPS (32 or 16; the narrow head leaves half of the
+// O^T tile's rows unused).  Work-group = 8 waves = 4 consecutive rows i x 2
 // halves of one (head, 128-query range); a wave owns 64 queries (two 32-query tiles) of one row.
 //   S^T = K Q^T  (rows = keys, columns = queries), six bf16 products per k-step, started from the
 //                triangle bias (the accumulator is loaded with it; logits stay in natural units, not
@@ -1453,8 +1486,9 @@ constexpr int kXTbSlots = 128 * 8;                     // bias slice [128 querie
 constexpr int kXKvSlots = 12 * 64;                     // K step 0, 1 (h m l each), then V^T step 0, 1
 constexpr size_t kCoreX3Lds = (size_t)(2 * kXTbSlots + 2 * kXRows * kXKvSlots) * 16;
 
+template <int STEPS>
 __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_qc, int n_rg, int total, int per_xcd) {
-  constexpr int QT = 2;
+  constexpr int QT = 2, D = 16 * STEPS;
   extern __shared__ u32x4_t lds4[];
   u32x4_t* tb_lds = lds4;                   // [2][kXTbSlots]
   u32x4_t* kv_lds = lds4 + 2 * kXTbSlots;   // [kXRows][2][kXKvSlots]
@@ -1472,19 +1506,19 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
   const int b = bh / H, h = bh % H;
   const int q0 = qc * 128 + 64 * qh;
   const size_t bih = ((size_t)b * N + i) * H + h;
-  const long plane = p.qkv_plane / 8;  // in 16-byte slots
-  const u32x4_t* Q = reinterpret_cast<const u32x4_t*>(p.qs) + bih * nt * 128 + lane;
+  const long plane = p.qk_plane / 8;  // in 16-byte slots
+  const u32x4_t* Q = reinterpret_cast<const u32x4_t*>(p.qs) + bih * nt * (64 * STEPS) + lane;
   const float* tbp = p.tb + ((size_t)b * H + h) * N * Jp;  // rows padded to Jp, zeros past N
   const int nkt = nt;
 
-  u32x4_t qop[QT][2][3];
+  u32x4_t qop[QT][STEPS][3];
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const int jt = q0 / 32 + qt < nt ? q0 / 32 + qt : nt - 1;  // tiles past the end: computed, not stored
 #pragma unroll
-    for (int st = 0; st < 2; ++st)
+    for (int st = 0; st < STEPS; ++st)
 #pragma unroll
-      for (int pl = 0; pl < 3; ++pl) qop[qt][st][pl] = Q[pl * plane + (jt * 2 + st) * 64];
+      for (int pl = 0; pl < 3; ++pl) qop[qt][st][pl] = Q[pl * plane + (jt * STEPS + st) * 64];
   }
 
   // bias slice: instruction n of wave w fills slots 64 (2 w + n) .. + 63; slot t holds chunk
@@ -1500,10 +1534,12 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
   }
   // this wave's share of its row's tile: the K operands (first wave of the row) or the V^T operands,
   // one descriptor per term (a plane can be larger than a descriptor's range)
-  const bf16_t* kvp = (qh ? p.vs : p.ks) + bih * Jp * 32;
-  const __amdgpu_buffer_rsrc_t kv_rsrc[3] = {buffer_rsrc(kvp, (size_t)Jp * 64),
-                                             buffer_rsrc(kvp + p.qkv_plane, (size_t)Jp * 64),
-                                             buffer_rsrc(kvp + 2 * p.qkv_plane, (size_t)Jp * 64)};
+  const int kv_steps = qh ? 2 : STEPS;  // 1-KB operands per key tile and term
+  const long kv_plane = qh ? p.v_plane : p.qk_plane;
+  const bf16_t* kvp = (qh ? p.vs : p.ks) + bih * Jp * (16 * kv_steps);
+  const size_t kv_bytes = (size_t)Jp * (32 * kv_steps);
+  const __amdgpu_buffer_rsrc_t kv_rsrc[3] = {buffer_rsrc(kvp, kv_bytes), buffer_rsrc(kvp + kv_plane, kv_bytes),
+                                             buffer_rsrc(kvp + 2 * kv_plane, kv_bytes)};
   const __amdgpu_buffer_rsrc_t tb_rsrc = buffer_rsrc(tbp, (size_t)N * Jp * sizeof(float));
   const uint32_t lane_off = lane * 16;
   u32x4_t* kv_row = kv_lds + row * (2 * kXKvSlots);
@@ -1516,10 +1552,12 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
                                                kt * (32 * (int)sizeof(float)), 0, 0);
 #pragma unroll
     for (int st = 0; st < 2; ++st)
+      if (st < kv_steps) {  // wave-uniform
 #pragma unroll
-      for (int pl = 0; pl < 3; ++pl)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(kv_rsrc[pl], (void OF3_LDS_AS*)(kdst + (st * 3 + pl) * 64), 16, lane_off,
-                                                 (kt * 2 + st) * 1024, 0, 0);
+        for (int pl = 0; pl < 3; ++pl)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(kv_rsrc[pl], (void OF3_LDS_AS*)(kdst + (st * 3 + pl) * 64), 16, lane_off,
+                                                   (kt * kv_steps + st) * 1024, 0, 0);
+      }
   };
   // mask value of key 32 kt + l32 (clamped to a real key; some bias value when there is no mask: not used)
   const float* mrow = p.mask ? p.mask + b * p.mv.stride_b + i * p.mv.stride_r : tbp;
@@ -1557,9 +1595,9 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
     const bool has_mb = __builtin_amdgcn_ballot_w64(mb != 0.f) != 0;
     const u32x4_t* kvb = kv_row + buf * kXKvSlots + lane;
     const u32x4_t* tbuf = tb_lds + buf * kXTbSlots + (64 * qh + l32) * 8;
-    u32x4_t kop[2][3];
+    u32x4_t kop[STEPS][3];
 #pragma unroll
-    for (int st = 0; st < 2; ++st)
+    for (int st = 0; st < STEPS; ++st)
 #pragma unroll
       for (int pl = 0; pl < 3; ++pl) kop[st][pl] = kvb[(st * 3 + pl) * 64];
 #pragma unroll
@@ -1573,7 +1611,7 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
       }
       if (has_mb) s = mask_step(mb, s);
 #pragma unroll
-      for (int st = 0; st < 2; ++st) {  // smallest terms first
+      for (int st = 0; st < STEPS; ++st) {  // smallest terms first
         s = mfma_32x32x16(kop[st][2], qop[qt][st][0], s);
         s = mfma_32x32x16(kop[st][0], qop[qt][st][2], s);
         s = mfma_32x32x16(kop[st][1], qop[qt][st][1], s);
@@ -1641,9 +1679,9 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
       const float l_tot = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
       if (q >= N) continue;
       const float inv = 1.0f / l_tot;
-      float* dst = p.o + ((((size_t)b * N + i) * N + q) * H + h) * 32 + 4 * lh;
+      float* dst = p.o + ((((size_t)b * N + i) * N + q) * H + h) * D + 4 * lh;
 #pragma unroll
-      for (int a = 0; a < 4; ++a)
+      for (int a = 0; a < D / 8; ++a)  // registers 4 a .. 4 a + 3 are head channels 8 a + 4 lh .. + 3
         *reinterpret_cast<float4*>(dst + 8 * a) = make_float4(oacc[qt][4 * a] * inv, oacc[qt][4 * a + 1] * inv,
                                                               oacc[qt][4 * a + 2] * inv, oacc[qt][4 * a + 3] * inv);
     }
@@ -2384,14 +2422,17 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
   const bool x3 = a.C % 16 == 0 && (a.H * a.D) % 16 == 0 && a.wsplit && aligned16({a.wsplit});
   const bool fast = a.C % 64 == 0 && (a.H * a.D) % 64 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 7u) == 0 &&
                     even_strides(a.x_view);
-  // head width 32: q, k and v leave the projection pass as split operands of the split-operand core
+  // head width 32 or 16 (then an even number of heads: a 32-channel tile of the projections is two of
+  // them): q, k and v leave the projection pass as split operands of the split-operand core
   p.Jp = (a.N + 31) / 32 * 32;
   // (the core addresses the bias of one (batch, head) with 32-bit byte offsets)
-  const bool core_x3 = x3 && a.D == 32 && a.qkv_split && aligned16({a.qkv_split}) && (long)a.N * p.Jp * 4 <= 0x7fffffffL;
-  p.qkv_plane = (long)a.B * a.N * a.H * p.Jp * 32;
+  const bool core_x3 = x3 && (a.D == 32 || (a.D == 16 && a.H % 2 == 0)) && a.qkv_split && aligned16({a.qkv_split}) &&
+                       (long)a.N * p.Jp * 4 <= 0x7fffffffL;
+  p.qk_plane = (long)a.B * a.N * a.H * p.Jp * a.D;
+  p.v_plane = (long)a.B * a.N * a.H * p.Jp * 32;
   p.qs = static_cast<bf16_t*>(a.qkv_split);
-  p.ks = p.qs + 3 * p.qkv_plane;
-  p.vs = p.qs + 6 * p.qkv_plane;
+  p.ks = p.qs + 3 * p.qk_plane;
+  p.vs = p.qs + 6 * p.qk_plane;
   const int xgroups = (a.N + 32 * kXT * kPT - 1) / (32 * kXT * kPT);
   const unsigned xblocks = (unsigned)((long)a.B * a.N * xgroups);
   if (x3) {
@@ -2413,7 +2454,8 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, true, false>>(kLdsLimit);
     if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, false, true>>(kLdsLimit);
     if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, true, true>>(kLdsLimit);
-    if (e == hipSuccess) e = allow_lds<triattn_core_x3_f32>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_core_x3_f32<1>>(kLdsLimit);
+    if (e == hipSuccess) e = allow_lds<triattn_core_x3_f32<2>>(kLdsLimit);
     if (e != hipSuccess) return e;
     const size_t lds = tile_bytes_x3(a.C, 32 * kXT * kPT) + (size_t)a.H * 32 * kXT * kPT * sizeof(float);
     hipLaunchKernelGGL(proj, dim3(xblocks), dim3(kThreads * kPT), lds, stream, p, xgroups);
@@ -2430,8 +2472,8 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     const long total = (long)n_qc * n_rg * a.B * a.H;
     if (total > 0x7fffffffL - 8) return hipErrorInvalidValue;
     const int per_xcd = (int)((total + 7) / 8);
-    hipLaunchKernelGGL(triattn_core_x3_f32, dim3(per_xcd * 8), dim3(512), kCoreX3Lds, stream, p, n_qc, n_rg, (int)total,
-                       per_xcd);
+    hipLaunchKernelGGL(a.D == 32 ? triattn_core_x3_f32<2> : triattn_core_x3_f32<1>, dim3(per_xcd * 8), dim3(512), kCoreX3Lds,
+                       stream, p, n_qc, n_rg, (int)total, per_xcd);
   } else if (a.D == 32)
     hipLaunchKernelGGL(triattn_core_f32<32>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
   else if (a.D == 16)

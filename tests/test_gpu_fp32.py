@@ -53,7 +53,11 @@ def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
                                                      (48, 64, 2, 37, (), True), (36, 16, 3, 21, (), True),
                                                      (64, 32, 2, 150, (), True),  # more than one 128-query group
                                                      (128, 32, 4, 44, (2,), True), (32, 32, 1, 129, (), False),
-                                                     (16, 32, 1, 9, (), True), (256, 32, 8, 40, (), True)])  # narrowest and widest
+                                                     (16, 32, 1, 9, (), True), (256, 32, 8, 40, (), True),  # narrowest and widest
+                                                     # head width 16: the template stack's; several query groups; an odd
+                                                     # number of heads (no pair of heads per 32-channel tile)
+                                                     (64, 16, 4, 150, (), True), (128, 16, 2, 70, (2,), False),
+                                                     (48, 16, 3, 40, (), True)])
 def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
     lib()
     gen = torch.Generator().manual_seed(400 + n)
@@ -134,8 +138,9 @@ def test_fp32_random_shapes(seed):
     cls = of3pair.TriangleMultiplicationOutgoing if outgoing else of3pair.TriangleMultiplicationIncoming
     got = _load(cls(c, ch), pm)(z.to(DEV), mask=None if mask is None else mask.to(DEV))
     _maxerr("trimul fp32 random", got, orc.trimul_update(z, mask, pm, outgoing))
-    pa = orc.make_triattn_params(gen, c, 32, heads)
-    got = _load(of3pair.TriangleAttention(c, 32, heads, starting=starting), pa)(z.to(DEV), mask=None if mask is None else mask.to(DEV))
+    d = 16 if seed % 3 == 2 else 32
+    pa = orc.make_triattn_params(gen, c, d, heads)
+    got = _load(of3pair.TriangleAttention(c, d, heads, starting=starting), pa)(z.to(DEV), mask=None if mask is None else mask.to(DEV))
     _maxerr("triattn fp32 random", got, orc.triattn_update(z, mask, pa, heads, starting=starting))
 
 
