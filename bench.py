@@ -32,6 +32,10 @@ with inplace_safe, where z drifts from step to step, for comparison) the line ca
                 the same N, for orientation; not part of `value`;
   fp32_block_ms  wall clock of the same pair-stack block in fp32 (the reference's default inference
                 precision; of3pair.PairStack on fp32 tensors), for orientation; not part of `value`;
+  fp32_pairformer_block_ms  wall clock of the whole PairFormerBlock in fp32, for orientation;
+  template_block_ms  {"bf16", "fp32"}: wall clock of one block of the template pair stack (of3pair.PairBlock,
+                4 templates, N = 512, c_t = 64, 4 heads x 16, transition n = 2, padded tails: the benchmark's
+                fourth configuration whatever --n says), for orientation;
   cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path) on the host
                 cores for the same workload: one warm-up run, then the median of three.
 """
@@ -58,7 +62,7 @@ CAL_BYTES = 256 << 20      # size of the calibration copy
 # scaled by what the same counter reads for the calibration copy; the summaries are kept in
 # profiles/.  Keyed by (N, tile variant the library picks for that shape): a figure measured
 # on one kernel variant is not reported for another; None for any other workload.
-MEASURED_TRAFFIC = {(768, 1): 539701909, (768, 4): 500864558}
+MEASURED_TRAFFIC = {(768, 1): 539701909, (768, 4): 499742378}
 
 TRANSITION_N = 4           # hidden width factor of the pair transition (AF3 configuration)
 PAIR_BIAS_HEADS = 16       # heads of the pairformer's single-representation attention
@@ -98,6 +102,49 @@ def kernel_model(B, N, C, CH, H, D):
     }
 
 
+def extra_legs(of3pair, orc, pf, s_pf, z32, sm, m32, fp32_reps, dev):
+    """Legs beside the headline workload, wall clock, informative: the whole PairFormerBlock in fp32 and one
+    block of the template pair stack at its own shape in both precisions."""
+    import torch
+
+    bf = torch.bfloat16
+    # ---- the whole PairFormerBlock in fp32, wall clock; informative
+    pf32 = of3pair.PairFormerBlock(C_S, 128, C_HEAD_S, PAIR_BIAS_HEADS, 128, 32, 4, "swiglu", TRANSITION_N, 0.25, False, 1e9)
+    pf32.load_state_dict(pf.state_dict())
+    pf32 = pf32.to(dev).float().eval()
+    s32 = s_pf.float()
+    pf32(s32, z32, sm, m32)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(fp32_reps):
+        pf32(s32, z32, sm, m32)
+    torch.cuda.synchronize()
+    fp32_pairformer_block_ms = (time.perf_counter() - t0) * 1e3 / fp32_reps
+
+    # ---- one block of the template pair stack at its own shape (4 templates, N = 512, c_t = 64, 4 x 16), both
+    # precisions, wall clock; informative
+    template_block_ms = {}
+    t_gen = torch.Generator().manual_seed(3)
+    t_params = dict(orc.make_block_params(30, 64, 64, 16, 4))
+    t_params.update({"pair_transition." + k_: v for k_, v in orc.make_transition_params(t_gen, 64, 2).items()})
+    t_host = orc.make_pair_input(3, (4,), 512, 64)
+    t_mask = orc.tail_padding_mask((4,), 512, torch.tensor([0, 20, 51, 102])).to(dev)
+    for name, dt in (("bf16", bf), ("fp32", torch.float32)):
+        tb_ = of3pair.PairBlock(64, 64, 16, 4, "swiglu", 2, 0.0, False, 1e9)
+        tb_.load_state_dict(t_params, strict=True)
+        tb_ = tb_.to(dev).to(dt).eval()
+        t_in = t_host.to(dev).to(dt)
+        tb_(t_in, t_mask)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(fp32_reps):
+            tb_(t_in, t_mask)
+        torch.cuda.synchronize()
+        template_block_ms[name] = round((time.perf_counter() - t0) * 1e3 / fp32_reps, 3)
+        del tb_, t_in
+    return fp32_pairformer_block_ms, template_block_ms
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -105,6 +152,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--n", type=int, default=768, help="N_token (768 = the headline configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the fp32 PairFormerBlock and the template-block legs (profiles of the headline workload)")
     ap.add_argument("--contract-variant", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -338,6 +387,10 @@ def main():
     torch.cuda.synchronize()
     fp32_block_ms = (time.perf_counter() - t0) * 1e3 / fp32_reps
 
+    fp32_pairformer_block_ms, template_block_ms = None, None
+    if not args.no_extras:
+        fp32_pairformer_block_ms, template_block_ms = extra_legs(of3pair, orc, pf, s_pf, z32, sm, m32, fp32_reps, dev)
+
     # ---- CPU baseline: the oracle on the host cores, one block of the same workload; one warm-up
     # run (thread pool, allocator), then the median of three
     cpu = None
@@ -375,6 +428,8 @@ def main():
                                "c_z=128, c_hidden_mul=128, 4 heads x 32, all-ones mask" % N},
         "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
         "pairformer_block_ms": round(pairformer_block_ms, 4), "fp32_block_ms": round(fp32_block_ms, 3),
+        "fp32_pairformer_block_ms": None if fp32_pairformer_block_ms is None else round(fp32_pairformer_block_ms, 3),
+        "template_block_ms": template_block_ms,
     }
     print(json.dumps(line))
 
