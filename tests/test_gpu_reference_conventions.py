@@ -6,7 +6,10 @@ against the fp32 CPU oracle (openfold3/tests/test_kernels.py):
     triangle multiplication on N(0,1) inputs, seq_len 84, c_z = c_hidden = 128, all-ones mask,
     several templates), every Linear re-initialised N(0, 1/fan_in) (:381-385);
   * a whole PairFormer block: mean-abs difference < 2e-2 after F.layer_norm over the channel
-    dimension (:469-492), inputs uniform [0, 1), masks random 0/1.
+    dimension (:469-492), inputs uniform [0, 1), masks random 0/1;
+  * the template embedder: max-abs difference < 2e-2 on its output, 3 templates, n_token = 200, a
+    random 0/1 pair mask (:652-725; here from the output of the feature embedding on, which is where
+    the replaced part begins).
 
 These sit beside the stricter rms / noise-floor criteria of tests/test_gpu_parity.py; the achieved
 figures are written to the parity summary."""
@@ -102,3 +105,50 @@ def test_pairformer_block_mean_abs_after_layer_norm(dtype):
         rec = record_parity("pairformer block %s after layer_norm (reference convention)" % name, g, w, None,
                             "mean|err| < 2e-2")
         assert rec["mean_abs_err"] < EPS, rec
+
+
+STACK_CFG = dict(c_t=64, c_hidden_tri_att=16, c_hidden_tri_mul=64, no_blocks=2, no_heads=4,
+                 transition_type="swiglu", pair_transition_n=2, dropout_rate=0.25, tri_mul_first=True,
+                 fuse_projection_weights=False, blocks_per_ckpt=None, inf=1e9, use_reentrant=False,
+                 tune_chunk_size=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_template_embedder_max_abs(dtype):
+    lib()
+    n, nt, ct, cz = 200, 3, 64, 128
+    gen = torch.Generator().manual_seed(2027)
+    blocks = []
+    for seed in range(2):
+        b = dict(orc.make_block_params(60 + seed, ct, ct, 16, 4))
+        b.update({"pair_transition." + k: v for k, v in orc.make_transition_params(gen, ct, 2).items()})
+        blocks.append(_params(b, dtype))
+    tail = _params(orc.make_template_tail_params(gen, ct, cz), dtype)
+    (emb,) = _inputs(dtype, torch.rand(1, nt, n, n, ct, generator=gen))
+    pair_mask = torch.randint(0, 2, (1, n, n), generator=gen).float()
+    core = of3pair.TemplateEmbedderCore(ct, cz, STACK_CFG)
+    sd = {}
+    for i, b in enumerate(blocks):
+        sd.update({"template_pair_stack.blocks.%d.%s" % (i, k): v for k, v in b.items()})
+    sd.update(tail)
+    core.load_state_dict(sd, strict=True)
+    core = core.to(DEV).to(dtype).eval()
+    got = core(emb.to(DEV).to(dtype), pair_mask.to(DEV))
+    tn = orc.template_stack(emb, pair_mask[:, None], blocks, tail["template_pair_stack.layer_norm.weight"],
+                            tail["template_pair_stack.layer_norm.bias"], 4)
+    want = orc.template_tail(tn, tail["linear_t.weight"])
+    rec = record_parity("template embedder output (reference convention)", got, want, None,
+                        "max|err| < 2e-2 (bf16: or the bf16 path's)")
+    bound = EPS
+    if dtype == torch.bfloat16:
+        # as for the triangle multiplication above: where the reference's own bf16 path (the oracle's
+        # operations run in bfloat16) lies above 2e-2, it is the yardstick
+        bf = torch.bfloat16
+        b16 = [{k: v.to(bf) for k, v in b.items()} for b in blocks]
+        t16 = {k: v.to(bf) for k, v in tail.items()}
+        tn16 = orc.template_stack(emb.to(bf), pair_mask[:, None].to(bf), b16, t16["template_pair_stack.layer_norm.weight"],
+                                  t16["template_pair_stack.layer_norm.bias"], 4)
+        ref16 = orc.template_tail(tn16, t16["linear_t.weight"])
+        bound = max(EPS, float((ref16.float() - want).abs().max()))
+        print("bf16 reference path max|err| = %.4g, HIP path %.4g" % (bound, rec["max_abs_err"]), flush=True)
+    assert rec["max_abs_err"] <= bound, rec
