@@ -58,7 +58,7 @@
  * of3_transition_fwd / of3_pair_bias_fwd / of3_layer_norm_fwd / of3_template_tail_fwd /
  * of3_attn_pair_bias_fwd / of3_transition_rows_fwd only:
  * every tensor and parameter is fp32, pointers 4-byte aligned, strides any positive
- * element counts, any N, C and CH <= 256, H*D <= 256 with D in {16, 32, 64}; fp32-grade
+ * element counts, any N, C and CH <= 256, H*D <= 256 with D <= 64; fp32-grade
  * arithmetic in the reference's order of operations.  With channel counts in multiples of
  * 16 the two triangle modules compute every fp32 product from three bf16 terms per operand
  * on the bf16 matrix instructions (six exact products, summed in fp32; the workspace holds

@@ -78,8 +78,7 @@ inline bool f32_trimul_dims_ok(int64_t B, int64_t N, int64_t C, int64_t CH) {
   return positions_ok(B, N) && N <= (1 << 16) && C >= 1 && C <= 256 && CH >= 1 && CH <= 256;
 }
 inline bool f32_triattn_dims_ok(int64_t B, int64_t N, int64_t C, int64_t H, int64_t D) {
-  return positions_ok(B, N) && N <= (1 << 16) && C >= 1 && C <= 256 && H >= 1 && (D == 16 || D == 32 || D == 64) &&
-         H * D <= 256;
+  return positions_ok(B, N) && N <= (1 << 16) && C >= 1 && C <= 256 && H >= 1 && D >= 1 && D <= 64 && H * D <= 256;
 }
 inline int64_t f32_triattn_qkv_bytes(int64_t B, int64_t N, int64_t H, int64_t D) {
   const int64_t fp32 = 3 * align256(B * N * N * H * D * 4), split = align256((int64_t)of3::triattn_qkv_split_bytes(B, N, H, D));

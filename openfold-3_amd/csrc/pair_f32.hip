@@ -1695,11 +1695,12 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
 //   O^T = V^T P^T rows = head channels; the weights go from the S^T accumulator registers straight
 //                 into the B operand: MFMA step v pairs the keys acc_row(v, 0) and acc_row(v, 1)
 // Logits in the reference's order: q.k, then the mask bias, then the triangle bias.
-template <int D>
+template <int DP>
 __global__ __launch_bounds__(kThreads, 2) void triattn_core_f32(TriattnF32 p, int qgroups) {
-  static_assert(D % 8 == 0 && D <= 64, "head widths 16, 32, 64");
-  constexpr int KC = 32, LD = D + 4;  // padded rows: the 16 lanes of a float4 read phase cover all banks
-  constexpr int OB = (D + 31) / 32;   // 32-channel blocks of the output
+  static_assert(DP % 8 == 0 && DP <= 64, "head widths up to 64, rounded up to a multiple of 8");
+  constexpr int KC = 32, LD = DP + 4;  // padded rows: the 16 lanes of a float4 read phase cover all banks
+  constexpr int OB = (DP + 31) / 32;   // 32-channel blocks of the output
+  const int D = p.D;                   // the head width itself: channels D .. DP - 1 are zeros in LDS
   static_assert(kThreads == 256, "four waves of 32 queries");
   __shared__ __align__(16) float ks[KC * LD];
   __shared__ float vs[KC * LD], mbs[KC];
@@ -1713,11 +1714,14 @@ __global__ __launch_bounds__(kThreads, 2) void triattn_core_f32(TriattnF32 p, in
   const bool active = qi < N;
   const size_t bih = (((size_t)b * N + i) * H + h) * N;
   // B operands of S^T: MFMA step 4j+e pairs d = 8j+e (lanes 0-31) with d = 8j+4+e (lanes 32-63)
-  float qv[D / 8][4];
+  float qv[DP / 8][4];
 #pragma unroll
-  for (int j = 0; j < D / 8; ++j)
+  for (int j = 0; j < DP / 8; ++j)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) qv[j][e] = active ? p.q[(bih + qi) * D + 8 * j + 4 * lh + e] : 0.f;
+    for (int e = 0; e < 4; ++e) {
+      const int d = 8 * j + 4 * lh + e;
+      qv[j][e] = active && d < D ? p.q[(bih + qi) * D + d] : 0.f;
+    }
   f32x16_t oacc[OB];
 #pragma unroll
   for (int ob = 0; ob < OB; ++ob) oacc[ob] = zero16();
@@ -1725,13 +1729,13 @@ __global__ __launch_bounds__(kThreads, 2) void triattn_core_f32(TriattnF32 p, in
   float m = -__builtin_inff(), l = 0.f;
   // a chunk's K, V, bias slice and mask values travel global -> registers while the previous chunk
   // is being computed, and registers -> LDS between two barriers
-  constexpr int KVI = KC * D / kThreads, TBI = 128 * KC / kThreads;
+  constexpr int KVI = KC * DP / kThreads, TBI = 128 * KC / kThreads;
   float k_r[KVI], v_r[KVI], tb_r[TBI], mb_r = 0.f;
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int it = 0; it < KVI; ++it) {
-      const int e = threadIdx.x + it * kThreads, kk = e / D, d = e % D;
-      const bool in = k0 + kk < N;
+      const int e = threadIdx.x + it * kThreads, kk = e / DP, d = e % DP;
+      const bool in = k0 + kk < N && d < D;
       k_r[it] = in ? p.k[(bih + k0 + kk) * D + d] : 0.f;
       v_r[it] = in ? p.v[(bih + k0 + kk) * D + d] : 0.f;
     }
@@ -1752,7 +1756,7 @@ __global__ __launch_bounds__(kThreads, 2) void triattn_core_f32(TriattnF32 p, in
     __syncthreads();
 #pragma unroll
     for (int it = 0; it < KVI; ++it) {
-      const int e = threadIdx.x + it * kThreads, kk = e / D, d = e % D;
+      const int e = threadIdx.x + it * kThreads, kk = e / DP, d = e % DP;
       ks[kk * LD + d] = k_r[it];
       vs[kk * LD + d] = v_r[it];
     }
@@ -1767,7 +1771,7 @@ __global__ __launch_bounds__(kThreads, 2) void triattn_core_f32(TriattnF32 p, in
     const int kn = N - k0 < KC ? N - k0 : KC;
     f32x16_t s = zero16();
 #pragma unroll
-    for (int j = 0; j < D / 8; ++j) {
+    for (int j = 0; j < DP / 8; ++j) {
       const float4 kk = *reinterpret_cast<const float4*>(ks + l32 * LD + 8 * j + 4 * lh);
       s = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.x, qv[j][0], s, 0, 0, 0);
       s = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.y, qv[j][1], s, 0, 0, 0);
@@ -1802,7 +1806,7 @@ __global__ __launch_bounds__(kThreads, 2) void triattn_core_f32(TriattnF32 p, in
     }
 #pragma unroll
     for (int ob = 0; ob < OB; ++ob) {
-      const int ch = 32 * ob + l32 < D ? 32 * ob + l32 : D - 1;  // rows past D are computed and dropped
+      const int ch = 32 * ob + l32 < DP ? 32 * ob + l32 : DP - 1;  // rows past D are computed and dropped
 #pragma unroll
       for (int v = 0; v < 16; ++v)
         oacc[ob] = __builtin_amdgcn_mfma_f32_32x32x2f32(vs[acc_row(v, lh) * LD + ch], s[v], oacc[ob], 0, 0, 0);
@@ -2474,14 +2478,22 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     const int per_xcd = (int)((total + 7) / 8);
     hipLaunchKernelGGL(a.D == 32 ? triattn_core_x3_f32<2> : triattn_core_x3_f32<1>, dim3(per_xcd * 8), dim3(512), kCoreX3Lds,
                        stream, p, n_qc, n_rg, (int)total, per_xcd);
-  } else if (a.D == 32)
-    hipLaunchKernelGGL(triattn_core_f32<32>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
-  else if (a.D == 16)
-    hipLaunchKernelGGL(triattn_core_f32<16>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
-  else if (a.D == 64)
-    hipLaunchKernelGGL(triattn_core_f32<64>, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
-  else
-    return hipErrorInvalidValue;
+  } else {
+    // any head width up to 64, in LDS rounded up to a multiple of 8
+    void (*core)(TriattnF32, int) = nullptr;
+    switch ((a.D + 7) / 8) {
+      case 1: core = triattn_core_f32<8>; break;
+      case 2: core = triattn_core_f32<16>; break;
+      case 3: core = triattn_core_f32<24>; break;
+      case 4: core = triattn_core_f32<32>; break;
+      case 5: core = triattn_core_f32<40>; break;
+      case 6: core = triattn_core_f32<48>; break;
+      case 7: core = triattn_core_f32<56>; break;
+      case 8: core = triattn_core_f32<64>; break;
+      default: return hipErrorInvalidValue;
+    }
+    hipLaunchKernelGGL(core, dim3((unsigned)cblocks), dim3(kThreads), 0, stream, p, qgroups);
+  }
   if (x3) {
     const int HD = a.H * a.D;
     const size_t lds = tile_bytes_x3(a.C > HD ? a.C : HD, 32 * kXT * kPT);

@@ -177,7 +177,7 @@ def triangle_attention(x, mask, norm_weight, norm_bias, bias_weight, q_weight, k
                              add_residual=add_residual)
     if nbytes < 0:
         raise ValueError("triangle attention: bf16 supports 4 heads with (c_in, c_head) = (128,32) or (64,16), fp32 "
-                         "head widths 16/32/64; got c_in=%d heads=%d c_head=%d in %s" % (C, H, D, x.dtype))
+                         "c_in <= 256, head widths up to 64 and heads * c_head <= 256; got c_in=%d heads=%d c_head=%d in %s" % (C, H, D, x.dtype))
     keep = [_w(t, x.dtype) for t in (norm_weight, norm_bias, bias_weight, q_weight, k_weight, v_weight, g_weight, o_weight)]
     m3, mptr, mstr = _mask_arg(mask, lead, B, N, x.device)
     out4 = x4 if inplace else _out_like(x4)

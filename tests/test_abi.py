@@ -132,7 +132,7 @@ def test_triattn_fwd_rejects_bad_arguments(lib):
     # q, k, v in three bf16 terms (18 bytes per element, more than 3 fp32 arrays), o, the triangle bias, the split weights
     assert need32 == 18 * 64 * 4 * 64 * 32 + 64 * 64 * 128 * 4 + 4 * 64 * 64 * 4 + 6 * 5 * 128 * 128
     assert call(dtype=_lib.OF3_DTYPE_F32, ws_bytes=need32 - 1) == _lib.OF3_ENOSPC
-    assert call(dtype=_lib.OF3_DTYPE_F32, D=24, ws_bytes=need32) == _lib.OF3_EINVAL
+    assert call(dtype=_lib.OF3_DTYPE_F32, D=72, ws_bytes=need32) == _lib.OF3_EINVAL  # head width beyond 64
     assert call(H=8) == _lib.OF3_EINVAL
     assert call(D=64) == _lib.OF3_EINVAL
     assert call(ws_bytes=ws_need - 1) == _lib.OF3_ENOSPC

@@ -57,7 +57,11 @@ def test_trimul_fp32(outgoing, c, ch, n, batch, masked):
                                                      # head width 16: the template stack's; several query groups; an odd
                                                      # number of heads (no pair of heads per 32-channel tile)
                                                      (64, 16, 4, 150, (), True), (128, 16, 2, 70, (2,), False),
-                                                     (48, 16, 3, 40, (), True)])
+                                                     (48, 16, 3, 40, (), True),
+                                                     # the reference's unit test (test_triangular_attention.py:24-45):
+                                                     # c_z = 128, head width 12, 4 heads, n_res = 22, batch 2, no mask;
+                                                     # and other widths that are no multiples of 8
+                                                     (128, 12, 4, 22, (2,), False), (40, 20, 2, 35, (), True), (64, 7, 3, 19, (), True)])
 def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
     lib()
     gen = torch.Generator().manual_seed(400 + n)
@@ -71,6 +75,20 @@ def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
     m = _load(of3pair.TriangleAttention(c, d, heads, starting=starting), p)
     got = m(x.to(DEV), mask=None if mask is None else mask.to(DEV))
     _maxerr("triattn fp32", got, orc.triattn_update(x, mask, p, heads, starting=starting))
+
+
+def test_trimul_fp32_reference_unit_test_shape():
+    """The reference's own unit test of the module (test_triangular_multiplicative_update.py:28-52): c_z = 128,
+    hidden width 11, batch 2, n_res = 128, uniform inputs and an integer 0/1 mask; here with the values checked."""
+    lib()
+    gen = torch.Generator().manual_seed(511)
+    p = orc.make_trimul_params(gen, 128, 11)
+    x = torch.rand(2, 128, 128, 128, generator=gen)
+    mask = torch.randint(0, 2, (2, 128, 128), generator=gen)
+    m = _load(of3pair.TriangleMultiplicationOutgoing(128, 11), p)
+    got = m(x.to(DEV), mask.to(DEV))
+    assert got.shape == x.shape
+    _maxerr("trimul fp32 c_hidden=11", got, orc.trimul_update(x, mask.float(), p, True))
 
 
 def test_block_config1_fp32():
