@@ -123,6 +123,39 @@ def test_pairformer_block_fp32():
         assert rec["max_abs_err"] <= 1e-4, rec
 
 
+def test_pairformer_stack_reference_unit_test_shape():
+    """The reference's own unit test of the stack (test_pairformer.py:24-75), here with the values checked:
+    fp32, batch 2, n_res = 22, c_s = 384, c_z = 128, pair-bias attention 3 heads of 12 (36 channels, not c_s),
+    hidden width 19 in the triangle multiplication, 7 heads of 14 in the triangle attention, transition
+    n = 2, two blocks, integer 0/1 masks, chunk_size = 4."""
+    lib()
+    n, cs, cz = 22, 384, 128
+    blocks = [orc.make_pairformer_block_params(70 + i, cs, cz, 19, 14, 7, 12, 3, 2) for i in range(2)]
+    gen = torch.Generator().manual_seed(99)
+    s = torch.rand(2, n, cs, generator=gen)
+    z = torch.rand(2, n, n, cz, generator=gen)
+    single_mask = torch.randint(0, 2, (2, n), generator=gen)
+    pair_mask = torch.randint(0, 2, (2, n, n), generator=gen)
+    stack = of3pair.PairFormerStack(c_s=cs, c_z=cz, c_hidden_pair_bias=12, no_heads_pair_bias=3, c_hidden_mul=19,
+                                    c_hidden_pair_att=14, no_heads_pair=7, no_blocks=2, transition_type="swiglu",
+                                    transition_n=2, pair_dropout=0.25, fuse_projection_weights=False,
+                                    blocks_per_ckpt=None, inf=1e9)
+    sd = {}
+    for i, p in enumerate(blocks):
+        sd.update({"blocks.%d.%s" % (i, k): v for k, v in p.items()})
+    stack.load_state_dict(sd, strict=True)
+    stack = stack.to(DEV).eval()
+    s_got, z_got = stack(s.to(DEV), z.to(DEV), single_mask=single_mask.to(DEV), pair_mask=pair_mask.to(DEV), chunk_size=4)
+    assert s_got.shape == s.shape and z_got.shape == z.shape
+    s_want, z_want = s, z
+    for p in blocks:
+        s_want, z_want = orc.pairformer_block(s_want, z_want, single_mask.float(), pair_mask.float(), p, 7, 3)
+    for name, got, want in (("z", z_got, z_want), ("s", s_got, s_want)):
+        rec = record_parity("pairformer stack, reference unit-test shape, fp32 " + name, got, want, None,
+                            "fp32: max|err| <= 1e-4")
+        assert rec["max_abs_err"] <= 1e-4, rec
+
+
 @pytest.mark.parametrize("mask_trans", [True, False])
 def test_pairformer_block(mask_trans):
     """One PairFormerBlock of the AF3 trunk shape at N = 72 with a padded tail: (s, z) against the
