@@ -247,6 +247,14 @@ def _swiglu_transition_rows(x, mask, norm_weight, norm_bias, a_weight, b_weight,
             mask = mask.expand(*x.shape[:-1])
         m = mask.to(torch.float32).contiguous()
     need = lib.of3_transition_rows_workspace_bytes_for(code, rows, C, HID)
+    if need < 0 and code == _lib.OF3_DTYPE_BF16 and lib.of3_transition_rows_workspace_bytes_for(_lib.OF3_DTYPE_F32, rows, C, HID) >= 0:
+        # widths the bf16 kernels do not serve: the fp32 kernel on widened activations, rounded once at the end
+        upd = _swiglu_transition_rows(x.float(), mask, norm_weight, norm_bias, a_weight, b_weight, out_weight, add_residual,
+                                      False, _lib.OF3_DTYPE_F32).to(torch.bfloat16)
+        if inplace:
+            x.copy_(upd)
+            return x
+        return upd
     if need < 0:
         raise ValueError("single transition: bf16 supports c_in = 384 with a hidden width that is a multiple of 384, "
                          "fp32 c_in <= 512 and hidden <= 2048; got hidden=%d in %s" % (HID, x.dtype))
@@ -281,6 +289,9 @@ def pair_bias(z, norm_weight, norm_bias, weight):
         st = lib.of3_pair_bias_fwd(z4.data_ptr(), _lib.strides3(z4.stride()[:3]), nw.data_ptr(),
                                    None if nb is None else nb.data_ptr(), w.data_ptr(), out.data_ptr(), B, N, C, H,
                                    code, _stream(z))
+    if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and C <= 256 and H <= 64:
+        # widths the bf16 kernel does not serve: the fp32 kernel on widened activations, rounded once at the end
+        return pair_bias(z.float(), norm_weight, norm_bias, weight).to(torch.bfloat16)
     if st == _lib.OF3_EINVAL:
         raise ValueError("pair bias: bf16 supports c_z 64 or 128 and up to 32 heads, fp32 c_z <= 256 and up to 64 "
                          "heads; got c_z=%d heads=%d in %s" % (C, H, z.dtype))
@@ -343,14 +354,16 @@ def template_tail(t, norm_weight, norm_bias, linear_t_weight, apply_layer_norm: 
 
 def attention_pair_bias(a, z, mask, norm_a_weight, norm_a_bias, norm_z_weight, norm_z_bias, z_weight, q_weight,
                         q_bias, k_weight, v_weight, g_weight, o_weight, no_heads: int, inf: float = 1e9,
-                        add_residual: bool = False, inplace: bool = False):
+                        add_residual: bool = False, inplace: bool = False, _bias=None):
     """AttentionPairBias.forward of the trunk (attention_pair_bias.py:189-244): attention over
     the single representation a [*, N, C_s] with the pair bias of z [*, N, N, C_z] and the key
     mask [*, N].  Returns the update (or a + update with add_residual; inplace writes into a).
     bf16: C_s = no_heads * head width = 384; fp32: C_s <= 512."""
     code = _require_gpu(a, "a")
     lib = _lib.load()
-    bias = pair_bias(z, norm_z_weight, norm_z_bias, z_weight)  # [*, H, N, N]
+    bias = _bias if _bias is not None else pair_bias(z, norm_z_weight, norm_z_bias, z_weight)  # [*, H, N, N]
+    if bias.dtype != a.dtype:
+        bias = bias.to(a.dtype)
     lead = a.shape[:-2]
     N, CS = a.shape[-2:]
     B = 1
@@ -369,6 +382,15 @@ def attention_pair_bias(a, z, mask, norm_a_weight, norm_a_bias, norm_z_weight, n
     if mask is not None:
         m = mask.to(torch.float32).expand(*lead, N).contiguous()
     need = lib.of3_attn_pair_bias_workspace_bytes_for(code, B, N, CS, H, D)
+    if need < 0 and code == _lib.OF3_DTYPE_BF16 and lib.of3_attn_pair_bias_workspace_bytes_for(_lib.OF3_DTYPE_F32, B, N, CS, H, D) >= 0:
+        # widths the bf16 kernels do not serve: the fp32 kernels on widened activations, rounded once at the end
+        upd = attention_pair_bias(a.float(), z, mask, norm_a_weight, norm_a_bias, norm_z_weight, norm_z_bias, z_weight,
+                                  q_weight, q_bias, k_weight, v_weight, g_weight, o_weight, no_heads, inf=inf,
+                                  add_residual=add_residual, inplace=False, _bias=bias.float()).to(torch.bfloat16)
+        if inplace:
+            a.copy_(upd)
+            return a
+        return upd
     if need < 0:
         raise ValueError("attention_pair_bias: bf16 supports C_s = no_heads * c = 384 with c a multiple of 8 up to "
                          "24, fp32 C_s <= 512 and c <= 64; got C_s=%d heads=%d c=%d in %s" % (CS, H, D, a.dtype))

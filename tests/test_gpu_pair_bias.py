@@ -86,5 +86,22 @@ def test_pair_bias_fp32(c, h, n, batch, offset):
 def test_pair_bias_rejects_unsupported():
     lib()
     z = torch.zeros(1, 8, 8, 128, device=DEV, dtype=torch.bfloat16)
-    with pytest.raises(ValueError):  # 40 heads: more than one MFMA tile of heads
-        F3.pair_bias(z, torch.ones(128, device=DEV), None, torch.zeros(40, 128, device=DEV))
+    with pytest.raises(ValueError):  # 80 heads: beyond both the bf16 kernel (32) and the fp32 kernels (64)
+        F3.pair_bias(z, torch.ones(128, device=DEV), None, torch.zeros(80, 128, device=DEV))
+    with pytest.raises(ValueError):  # 320 channels: beyond the fp32 kernels too
+        F3.pair_bias(torch.zeros(1, 8, 8, 320, device=DEV, dtype=torch.bfloat16), torch.ones(320, device=DEV), None,
+                     torch.zeros(4, 320, device=DEV))
+
+
+def test_pair_bias_bf16_shape_outside_the_bf16_kernel():
+    """40 heads (more than one MFMA tile of heads) and 96 channels in bf16: the fp32 kernel on widened
+    activations, rounded to bf16 once."""
+    lib()
+    for c, h in ((128, 40), (96, 5)):
+        gen = torch.Generator().manual_seed(930 + h)
+        p = {k: orc.round_bf16(v) for k, v in orc.make_pair_bias_params(gen, c, h, offset=True).items()}
+        z = orc.round_bf16(orc.make_pair_input(23, (2,), 19, c))
+        got = _module(c, h, p, torch.bfloat16)(z.to(DEV).to(torch.bfloat16))
+        assert got.dtype == torch.bfloat16 and tuple(got.shape) == (2, h, 19, 19)
+        want = orc.pair_bias(z, p)
+        report("pair bias, bf16 through fp32", got.float().cpu(), want, atol=2e-2 * float(want.abs().max()), rtol=0.0)

@@ -156,6 +156,32 @@ def test_pairformer_stack_reference_unit_test_shape():
         assert rec["max_abs_err"] <= 1e-4, rec
 
 
+def test_pairformer_block_bf16_widths_outside_the_bf16_kernels():
+    """The same odd widths in bf16: every module of the block falls back to the fp32 kernels on widened
+    activations and rounds its result to bf16 once (pair modules, pair bias, attention over s, transitions)."""
+    lib()
+    n, cs, cz = 22, 384, 128
+    p = _round(orc.make_pairformer_block_params(72, cs, cz, 19, 14, 7, 12, 3, 2))
+    gen = torch.Generator().manual_seed(100)
+    s = orc.round_bf16(torch.rand(2, n, cs, generator=gen))
+    z = orc.round_bf16(torch.rand(2, n, n, cz, generator=gen))
+    single_mask = torch.randint(0, 2, (2, n), generator=gen).float()
+    pair_mask = torch.randint(0, 2, (2, n, n), generator=gen).float()
+    blk = of3pair.PairFormerBlock(c_s=cs, c_z=cz, c_hidden_pair_bias=12, no_heads_pair_bias=3, c_hidden_mul=19,
+                                  c_hidden_pair_att=14, no_heads_pair=7, transition_type="swiglu", transition_n=2,
+                                  pair_dropout=0.25, fuse_projection_weights=False, inf=1e9)
+    blk.load_state_dict(p, strict=True)
+    blk = blk.to(DEV).to(torch.bfloat16).eval()
+    sg, zg = s.to(DEV).to(torch.bfloat16), z.to(DEV).to(torch.bfloat16)
+    s_got, z_got = blk(sg, zg, single_mask.to(DEV), pair_mask.to(DEV))
+    assert s_got.dtype == torch.bfloat16 and z_got.dtype == torch.bfloat16
+    s_want, z_want = orc.pairformer_block(s, z, single_mask, pair_mask, p, 7, 3)
+    _check("pairformer block, odd widths in bf16, z", z_got, z_want, rms_rel=1e-2)
+    _check("pairformer block, odd widths in bf16, s", s_got, s_want, rms_rel=1e-2)
+    s2, z2 = blk(sg.clone(), zg.clone(), single_mask.to(DEV), pair_mask.to(DEV), inplace_safe=True)
+    assert torch.equal(s2, s_got) and torch.equal(z2, z_got)
+
+
 @pytest.mark.parametrize("mask_trans", [True, False])
 def test_pairformer_block(mask_trans):
     """One PairFormerBlock of the AF3 trunk shape at N = 72 with a padded tail: (s, z) against the

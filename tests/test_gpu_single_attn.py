@@ -100,14 +100,37 @@ def test_attention_pair_bias_rejects_unsupported():
     lib()
     with pytest.raises(ValueError):
         of3pair.AttentionPairBias(384, 384, 384, 384, 128, 24, 16, use_ada_layer_norm=True)
-    m = of3pair.AttentionPairBias(128, 128, 128, 128, 128, 32, 4).to(DEV).to(torch.bfloat16)  # c_s = 128
-    a = torch.zeros(8, 128, device=DEV, dtype=torch.bfloat16)
-    z = torch.zeros(8, 8, 128, device=DEV, dtype=torch.bfloat16)
-    with pytest.raises(ValueError):
-        m(a, z)
     m2 = of3pair.AttentionPairBias(768, 768, 768, 768, C_Z, 48, 16).to(DEV)  # c_s beyond the fp32 kernels
     with pytest.raises(ValueError):
         m2(torch.zeros(8, 768, device=DEV), torch.zeros(8, 8, C_Z, device=DEV))
+    with pytest.raises(ValueError):  # ... in bf16 too: there is no fp32 kernel to fall back to
+        m2.to(torch.bfloat16)(torch.zeros(8, 768, device=DEV, dtype=torch.bfloat16),
+                              torch.zeros(8, 8, C_Z, device=DEV, dtype=torch.bfloat16))
+
+
+def test_attention_pair_bias_bf16_width_outside_the_bf16_kernels():
+    """c_s = 128 with 4 heads of 32 in bf16: not a shape of the bf16 kernels; served by the fp32 kernels on
+    widened activations, rounded to bf16 once."""
+    lib()
+    n, c_s, c_head, heads = 29, 128, 32, 4
+    gen = torch.Generator().manual_seed(870)
+    p = {k: orc.round_bf16(v) for k, v in orc.make_attention_pair_bias_params(gen, c_s, 64, c_head, heads).items()}
+    a = orc.round_bf16(torch.randn(n, c_s, generator=gen))
+    z = orc.round_bf16(orc.make_pair_input(871, (), n, 64))
+    mask = torch.ones(n)
+    mask[-4:] = 0
+    m = of3pair.AttentionPairBias(c_s, c_s, c_s, c_s, 64, c_head, heads)
+    m.load_state_dict(p, strict=True)
+    m = m.to(DEV).to(torch.bfloat16).eval()
+    got = m(a.to(DEV).to(torch.bfloat16), z.to(DEV).to(torch.bfloat16), mask=mask.to(DEV))
+    assert got.dtype == torch.bfloat16
+    want = orc.attention_pair_bias(a, z, mask, p, heads)
+    report("attention pair bias, bf16 through fp32", got.float().cpu(), want, atol=2e-2 * float(want.abs().max()), rtol=0.0)
+    ag = a.to(DEV).to(torch.bfloat16)
+    res = m(ag, z.to(DEV).to(torch.bfloat16), mask=mask.to(DEV), _add_residual=True, _inplace=True)
+    assert res.data_ptr() == ag.data_ptr()
+    report("attention pair bias, bf16 through fp32, a+update", res.float().cpu(), a + want,
+           atol=2e-2 * float((a + want).abs().max()), rtol=0.0)
 
 
 @pytest.mark.parametrize("n,batch,c_s,c_head,heads,masked", [(37, (), 384, 24, 16, True), (130, (2,), 96, 12, 8, True),
