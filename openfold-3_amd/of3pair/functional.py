@@ -312,6 +312,8 @@ def layer_norm(x, weight, bias):
     with torch.cuda.device(x.device):
         st = lib.of3_layer_norm_fwd(xc.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(), rows, C, code,
                                     _stream(x))
+    if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and C <= 256:
+        return layer_norm(x.float(), weight, bias).to(torch.bfloat16)  # the fp32 kernel, rounded once at the end
     if st == _lib.OF3_EINVAL:
         raise ValueError("layer norm: bf16 supports 64 or 128 channels, fp32 up to 256; got %d in %s" % (C, x.dtype))
     _lib.check(st, "of3_layer_norm_fwd")
@@ -345,6 +347,9 @@ def template_tail(t, norm_weight, norm_bias, linear_t_weight, apply_layer_norm: 
         st = lib.of3_template_tail_fwd(tc.data_ptr(), None if nw is None else nw.data_ptr(),
                                        None if nb is None else nb.data_ptr(), w.data_ptr(), out.data_ptr(), B, T,
                                        N * N, CT, CZ, 1 if apply_layer_norm else 0, code, _stream(t))
+    if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and CT <= 256:
+        # the fp32 kernel on widened activations, rounded once at the end
+        return template_tail(t.float(), norm_weight, norm_bias, linear_t_weight, apply_layer_norm).to(torch.bfloat16)
     if st == _lib.OF3_EINVAL:
         raise ValueError("template tail: bf16 supports c_t = 64 with c_z = 128, fp32 c_t <= 256; got c_t=%d c_z=%d "
                          "in %s" % (CT, CZ, t.dtype))

@@ -181,9 +181,28 @@ def test_template_tail_full_size_rows():
 
 def test_template_tail_rejects_unsupported():
     lib()
-    t = torch.zeros(2, 8, 8, 32, device=DEV, dtype=torch.bfloat16)  # c_t = 32 has no bf16 kernel
+    t = torch.zeros(2, 8, 8, 320, device=DEV, dtype=torch.bfloat16)  # c_t = 320: beyond the fp32 kernels too
     with pytest.raises(ValueError):
-        F3.template_tail(t, torch.ones(32, device=DEV), torch.zeros(32, device=DEV), torch.zeros(128, 32, device=DEV))
+        F3.template_tail(t, torch.ones(320, device=DEV), torch.zeros(320, device=DEV), torch.zeros(128, 320, device=DEV))
     with pytest.raises(ValueError):
-        F3.layer_norm(torch.zeros(4, 96, device=DEV, dtype=torch.bfloat16), torch.ones(96, device=DEV),
-                      torch.zeros(96, device=DEV))
+        F3.layer_norm(torch.zeros(4, 320, device=DEV, dtype=torch.bfloat16), torch.ones(320, device=DEV),
+                      torch.zeros(320, device=DEV))
+
+
+def test_template_tail_and_layer_norm_bf16_widths_outside_the_bf16_kernels():
+    """c_t = 32 -> c_z = 96 and a LayerNorm over 96 channels in bf16: the fp32 kernels on widened activations,
+    rounded to bf16 once."""
+    lib()
+    gen = torch.Generator().manual_seed(79)
+    p = {k: orc.round_bf16(v) for k, v in orc.make_template_tail_params(gen, 32, 96).items()}
+    g, b, w = p["template_pair_stack.layer_norm.weight"], p["template_pair_stack.layer_norm.bias"], p["linear_t.weight"]
+    t = orc.round_bf16(torch.randn(3, 17, 17, 32, generator=gen))
+    got = F3.template_tail(t.to(DEV).to(torch.bfloat16), g.to(DEV), b.to(DEV), w.to(DEV))
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (17, 17, 96)
+    _check("template tail, bf16 through fp32", got, orc.template_tail(orc.layer_norm(t, g, b), w))
+    gen = torch.Generator().manual_seed(80)
+    x = orc.round_bf16(2.0 * torch.randn(11, 96, generator=gen) + 0.5)
+    gw, gb = orc.round_bf16(1 + 0.1 * torch.randn(96, generator=gen)), orc.round_bf16(0.1 * torch.randn(96, generator=gen))
+    got = F3.layer_norm(x.to(DEV).to(torch.bfloat16), gw.to(DEV), gb.to(DEV))
+    assert got.dtype == torch.bfloat16
+    _check("layer norm, bf16 through fp32", got, orc.layer_norm(x, gw, gb))
