@@ -30,8 +30,9 @@ struct TrimulProjArgs {
 hipError_t trimul_proj_launch(const TrimulProjArgs& args, int C, int CH, hipStream_t stream);
 
 // a, b: k-panel layout [planes][Np/32][Np][32]; x: row-major [planes][Np][Np].
-// variant: 1 = 256x192 output tiles, 2 = 256x128, 3 = 256x256
-hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
+// nk: the k-panels that are summed over, ceil(N / 32) (the later ones hold zeros);
+// variant: 1 = 256x192 output tiles, 2 = 256x128, 3 = 256x256, 4 = 384x192 on eight waves
+hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int nk, int variant,
                                   hipStream_t stream);
 
 struct TrimulOutArgs {

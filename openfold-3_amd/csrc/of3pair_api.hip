@@ -210,7 +210,7 @@ int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_
   if (!a || !b || !x || !aligned16(a) || !aligned16(b) || !aligned16(x)) return OF3_EINVAL;
   const int64_t Np = padded(N);
   if (variant == 0) variant = contract_variant_auto(B * CH, Np);
-  hipError_t e = of3::trimul_contract_launch(bf(a), bf(b), bf(x), (int)(B * CH), (int)Np, variant,
+  hipError_t e = of3::trimul_contract_launch(bf(a), bf(b), bf(x), (int)(B * CH), (int)Np, (int)((N + 31) / 32), variant,
                                              static_cast<hipStream_t>(stream));
   return e == hipSuccess ? OF3_OK : fail_hip(e);
 }

@@ -1591,7 +1591,11 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
   }
   const int tb_key = (l32 >> 1) & 7;
 
+  // a wave of a row past the end, or whose queries all lie past the end, still takes part in the loads and
+  // barriers of its work-group but leaves the arithmetic out; so does a 32-query tile past the end
+  const bool wave_has_work = row_valid && q0 < N;
   auto tile = [&](int buf, float mb) {
+    if (!wave_has_work) return;
     const bool has_mb = __builtin_amdgcn_ballot_w64(mb != 0.f) != 0;
     const u32x4_t* kvb = kv_row + buf * kXKvSlots + lane;
     const u32x4_t* tbuf = tb_lds + buf * kXTbSlots + (64 * qh + l32) * 8;
@@ -1602,6 +1606,7 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
       for (int pl = 0; pl < 3; ++pl) kop[st][pl] = kvb[(st * 3 + pl) * 64];
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
+      if (qt > 0 && q0 + 32 * qt >= N) continue;
       f32x16_t s;
 #pragma unroll
       for (int a = 0; a < 4; ++a) {  // registers 4 a .. 4 a + 3: keys 8 a + 4 lh .. + 3 = chunk 2 a + lh

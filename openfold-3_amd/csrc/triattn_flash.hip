@@ -203,8 +203,13 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
     const u32x2_t a_op = {lo ? 0x3F803F80u : 0u, lo ? 0x3F80u : 0u};
     return mfma_32x32x8(a_op, b_op, acc);
   };
+  // a wave of a row past the end, or whose queries all lie past the end (N not a multiple of 4 or of 64),
+  // still takes part in the loads and barriers of its work-group but leaves the arithmetic out; so does
+  // a 32-query tile past the end.  All of these are wave-uniform.
+  const bool wave_has_work = row_valid && q0 < N;
   auto tile = [&](auto track, int buf, float mb_cur) {
     constexpr bool kTrack = decltype(track)::value;
+    if (!wave_has_work) return;
     const bool has_mb = __builtin_amdgcn_ballot_w64(mb_cur != 0.f) != 0;
     const u32x4_t* tbuf = tb_lds + buf * TBS + tb_row;
     const u32x4_t* kvb = kv_row + buf * KVS;
@@ -219,6 +224,7 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
     }
 #pragma unroll
     for (int rq = 0; rq < kRQ; ++rq) {
+      if (rq > 0 && q0 + 32 * rq >= N) continue;
       f32x16_t s;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {

@@ -64,8 +64,8 @@ __device__ __forceinline__ void wait_vmcnt() {
 template <int BN, int kNS>
 __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restrict__ pm,  // j side planes (b)
                                                           const bf16_t* __restrict__ pn,  // i side planes (a)
-                                                          bf16_t* __restrict__ x, int Np, int tiles_m, int tiles_n,
-                                                          int total_tiles, int tiles_per_xcd) {
+                                                          bf16_t* __restrict__ x, int Np, int nk, int tiles_m,
+                                                          int tiles_n, int total_tiles, int tiles_per_xcd) {
   constexpr int BM = 256;
   constexpr int WM = BM / 2, WN = BN / 2;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
   const int my_tiles = slot_in_xcd < xcd_count ? (xcd_count - slot_in_xcd + wgs_per_xcd - 1) / wgs_per_xcd : 0;
   if (my_tiles == 0) return;
   const int per_plane = tiles_m * tiles_n;
-  const int nk = Np / kBK;
+  // nk: the 32-wide k-panels that hold keys below N (the panels after them hold zeros and are left out)
   const size_t panel_bytes = (size_t)Np * kBK * 2;
 
   auto tile_coords = [&](int t_local, int& plane, int& tm, int& tn) {
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
       // simply allowed to stay outstanding, otherwise the wait would drain the whole ring
       // at every tile boundary.
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): a1/b1 have arrived
-      if (stores_pending && kb < kNS - 1) wait_vmcnt<(kNS - 2) * IPW + 8 * TN>();
+      if (stores_pending && kb < kNS - 1 && nk >= kNS) wait_vmcnt<(kNS - 2) * IPW + 8 * TN>();
       else wait_vmcnt<(kNS - 2) * IPW>();
       compiler_fence();
       __builtin_amdgcn_s_barrier();
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
 }
 
 template <int BN, int kNS>
-hipError_t launch_contract(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, hipStream_t stream) {
+hipError_t launch_contract(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int nk, hipStream_t stream) {
   constexpr int BM = 256;
   auto kern = contract_kernel<BN, kNS>;
   const size_t smem = ((size_t)kNS * (BM + BN) * 4 + 4 * 512) * sizeof(u32x4_t);  // ring + epilogue staging
@@ -328,7 +328,7 @@ hipError_t launch_contract(const bf16_t* a, const bf16_t* b, bf16_t* x, int plan
   int grid = (cus / 8) * 8;  // a multiple of the 8 XCDs
   if (grid < 8) grid = 8;
   // M side (register-contiguous output index j) is b, N side (lane index i) is a
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, stream, b, a, x, Np, tiles_m, tiles_n, total, tiles_per_xcd);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, stream, b, a, x, Np, nk, tiles_m, tiles_n, total, tiles_per_xcd);
   return hipGetLastError();
 }
 
@@ -347,8 +347,8 @@ hipError_t launch_contract(const bf16_t* a, const bf16_t* b, bf16_t* x, int plan
 template <int kNS>
 __global__ __launch_bounds__(512, 1) void contract8_kernel(const bf16_t* __restrict__ pm,  // j side planes (b)
                                                            const bf16_t* __restrict__ pn,  // i side planes (a)
-                                                           bf16_t* __restrict__ x, int Np, int tiles_m, int tiles_n,
-                                                           int total_tiles, int tiles_per_xcd) {
+                                                           bf16_t* __restrict__ x, int Np, int nk, int tiles_m,
+                                                           int tiles_n, int total_tiles, int tiles_per_xcd) {
   constexpr int BM = 384, BN = 192;
   constexpr int WM = 96, WN = 96;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -379,7 +379,7 @@ __global__ __launch_bounds__(512, 1) void contract8_kernel(const bf16_t* __restr
   const int my_tiles = slot_in_xcd < xcd_count ? (xcd_count - slot_in_xcd + wgs_per_xcd - 1) / wgs_per_xcd : 0;
   if (my_tiles == 0) return;
   const int per_plane = tiles_m * tiles_n;
-  const int nk = Np / kBK;
+  // nk: the 32-wide k-panels that hold keys below N (the panels after them hold zeros and are left out)
   const size_t panel_bytes = (size_t)Np * kBK * 2;
 
   auto tile_coords = [&](int t_local, int& plane, int& tm, int& tn) {
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(512, 1) void contract8_kernel(const bf16_t* __restr
       // wave, the newest kNS-2 stages (and a finished tile's stores, for its first stages) may
       // stay in flight
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): a1/b1 have arrived
-      if (stores_pending && kb < kNS - 1)
+      if (stores_pending && kb < kNS - 1 && nk >= kNS)
         wait_stages(std::integral_constant<int, kNS - 2>{}, std::integral_constant<int, STORES>{});
       else
         wait_stages(std::integral_constant<int, kNS - 2>{}, std::integral_constant<int, 0>{});
@@ -562,7 +562,7 @@ __global__ __launch_bounds__(512, 1) void contract8_kernel(const bf16_t* __restr
 }
 
 template <int kNS>
-hipError_t launch_contract8(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, hipStream_t stream) {
+hipError_t launch_contract8(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int nk, hipStream_t stream) {
   constexpr int BM = 384, BN = 192;
   auto kern = contract8_kernel<kNS>;
   const size_t smem = ((size_t)kNS * (BM + BN) * 4 + 8 * 32 * 12) * sizeof(u32x4_t);  // ring + epilogue staging
@@ -582,23 +582,24 @@ hipError_t launch_contract8(const bf16_t* a, const bf16_t* b, bf16_t* x, int pla
   const int tiles_per_xcd = (total + 7) / 8;
   int grid = (cus / 8) * 8;
   if (grid < 8) grid = 8;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), smem, stream, b, a, x, Np, tiles_m, tiles_n, total, tiles_per_xcd);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), smem, stream, b, a, x, Np, nk, tiles_m, tiles_n, total, tiles_per_xcd);
   return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int variant,
+hipError_t trimul_contract_launch(const bf16_t* a, const bf16_t* b, bf16_t* x, int planes, int Np, int nk, int variant,
                                   hipStream_t stream) {
+  if (nk < 1 || nk > Np / kBK) return hipErrorInvalidValue;
   switch (variant) {
     case 1:
-      return launch_contract<192, 4>(a, b, x, planes, Np, stream);
+      return launch_contract<192, 4>(a, b, x, planes, Np, nk, stream);
     case 2:
-      return launch_contract<128, 4>(a, b, x, planes, Np, stream);
+      return launch_contract<128, 4>(a, b, x, planes, Np, nk, stream);
     case 3:
-      return launch_contract<256, 4>(a, b, x, planes, Np, stream);
+      return launch_contract<256, 4>(a, b, x, planes, Np, nk, stream);
     case 4:
-      return launch_contract8<3>(a, b, x, planes, Np, stream);
+      return launch_contract8<3>(a, b, x, planes, Np, nk, stream);
     default:
       return hipErrorInvalidValue;
   }

@@ -15,6 +15,9 @@
 // columns so that a lane finishes 4 consecutive k of one row and channel and stores them as
 // one 8-byte vector.  A tile is 4 consecutive rows r of one 32-wide k-panel: in the k-panel
 // layout these are 256 contiguous bytes per channel, so 32 lanes write whole 128-byte lines.
+// Only the panels that hold a k below N are written (the last one with zeros from N on), and only
+// the rows up to N rounded up to 4: the contraction sums over no other panel, and what it makes of
+// the other rows lands in rows and columns of x that nobody reads.
 #include "of3_device.h"
 #include "of3_kernels.h"
 #include "of3_launch.h"
@@ -219,7 +222,7 @@ hipError_t launch(const TrimulProjArgs& a, hipStream_t stream) {
   int grid_cap = 0;
   hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 512, dev, v); }, &grid_cap);
   if (e != hipSuccess) return e;
-  const int panels = a.Np / 32;
+  const int panels = (a.N + 31) / 32;  // the panels that hold a k below N; the contraction reads no others
   const long total = (long)a.B * ((a.N + 3) / 4) * panels;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, panels, (int)total);

@@ -55,6 +55,30 @@ def test_contract(variant, n):
     report("contract", x, want, atol=2e-2 * math.sqrt(np_) , rtol=1e-2)
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("n", [70, 200, 333])
+def test_contract_ragged_n(variant, n):
+    """N off the multiples of 32 and 128: the sum runs over the ceil(N / 32) panels that hold a k below N (fewer
+    of them than the pipeline has stages at N = 70), the panels after them are never read (they hold NaN here)."""
+    L = lib()
+    gen = _gen(500 + n + variant)
+    planes, B, CH = 64, 1, 64
+    np_ = L.of3_padded_n(n)
+    kk = (n + 31) // 32 * 32
+    a = bf(_randn(gen, planes, np_, np_))
+    b = bf(_randn(gen, planes, np_, np_))
+    a[:, :, kk:] = float("nan")
+    b[:, :, kk:] = float("nan")
+    x = torch.full((planes, np_, np_), float("nan"), dtype=torch.bfloat16, device=DEV)
+    print("contract ragged variant", variant, "n", n, flush=True)
+    ap, bp = _to_panels(a), _to_panels(b)
+    st = L.of3_trimul_contract(ap.data_ptr(), bp.data_ptr(), x.data_ptr(), B, n, CH, variant, stream())
+    assert st == 0, L.of3_status_string(st)
+    torch.cuda.synchronize()
+    want = torch.bmm(a[:, :, :kk].float(), b[:, :, :kk].float().transpose(1, 2))
+    report("contract ragged", x[:, :n, :n], want[:, :n, :n], atol=2e-2 * math.sqrt(kk), rtol=1e-2)
+
+
 def _trimul_weights(gen, C, CH):
     w = {
         "ln_in_w": 1 + 0.1 * torch.randn(C, generator=gen), "ln_in_b": 0.1 * torch.randn(C, generator=gen),
@@ -93,8 +117,12 @@ def test_trimul_proj(outgoing, C, n, B):
         # expected [b][c][r][k]: outgoing (r,k) = (i,k); incoming (r,k) from ref[b,k,r,c]
         want = ref.permute(0, 3, 1, 2) if outgoing else ref.permute(0, 3, 2, 1)
         report("trimul_proj %s valid" % name, got[:, :, :n, :n], want, atol=2e-2, rtol=1e-2)
-        pad = got[:, :, :n, n:]
+        # the contraction sums over the panels that hold a k below n: the last of them is padded with zeros,
+        # the panels after it are not written at all
+        kk = (n + 31) // 32 * 32
+        pad = got[:, :, :n, n:kk]
         assert (pad.float() == 0).all(), "k-padding of %s must be zero" % name
+        assert torch.isnan(got[:, :, :n, kk:].float()).all(), "panels past the last k of %s are left alone" % name
 
 
 @pytest.mark.parametrize("add_residual", [0, 1])
