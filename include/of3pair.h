@@ -100,14 +100,16 @@ int64_t of3_trimul_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t 
 
 /* a, b: gated, masked projections, channel-major in "k-panels" of 32 contracted indices:
  * shape [B][CH][NP/32][NP][32], a[b][c][k/32][i][k%32] = a_ref[b,i,k,c] (outgoing) or
- * a_ref[b,k,i,c] (incoming); entries with k >= N are zero, rows i >= N are left untouched. */
+ * a_ref[b,k,i,c] (incoming).  Written: the ceil(N/32) panels that hold a k < N, their entries with k >= N
+ * as zeros, rows i up to N rounded up to 4; the other panels and rows are left untouched. */
 int of3_trimul_proj(const void* z, const int64_t z_strides[3], const float* mask, const int64_t mask_strides[3],
                     const void* ln_in_w, const void* ln_in_b, const void* w_a_p, const void* w_a_g,
                     const void* w_b_p, const void* w_b_g, void* a, void* b, int64_t B, int64_t N, int64_t C,
                     int64_t CH, int outgoing, void* stream);
 
-/* x[b][c][i][j] = sum_k a[b][c][i][k] * b[b][c][j][k] over the padded planes; a, b in the
- * k-panel layout above, x row-major [B][CH][NP][NP].
+/* x[b][c][i][j] = sum_k a[b][c][i][k] * b[b][c][j][k], the sum over the ceil(N/32) panels that hold a
+ * k < N (entries with k >= N in the last of them must be zero; later panels are not read); a, b in the
+ * k-panel layout above, x row-major [B][CH][NP][NP], of which rows and columns below N are meaningful.
  * variant: 0 = automatic; 1 / 2 / 3 / 4 = 256x192 / 256x128 / 256x256 / 384x192 output tiles. */
 int of3_trimul_contract(const void* a, const void* b, void* x, int64_t B, int64_t N, int64_t CH, int variant,
                         void* stream);
