@@ -139,9 +139,15 @@ int of3_trimul_fwd(const void* z, const int64_t z_strides[3], const float* mask,
  * workspace: a, b and x live in a scratch array built into the library, OF3_STATIC_SCRATCH_BYTES
  * per GPU, which every GPU the library runs on holds until the process ends.  The call allocates
  * and frees nothing.  Problems with of3_trimul_workspace_bytes_for(dtype, B, N, C, CH) above that
- * size return OF3_ESTATIC before anything is launched (bf16: B*CH*NP*NP <= 2^23, e.g. B = 1,
- * C = CH = 128, N <= 256; fp32: B*CH*N*N <= 2^22).  All calls on one GPU share that GPU's array:
- * calls that overlap on one GPU (two streams, two threads) race; calls on one stream are ordered. */
+ * size return OF3_ESTATIC before anything is launched: the rule is exactly
+ * of3_trimul_workspace_bytes_for(dtype, B, N, C, CH) <= OF3_STATIC_SCRATCH_BYTES (bf16:
+ * B*CH*NP*NP <= 2^23, e.g. B = 1, C = CH = 128, N <= 256; fp32, whose scratch also holds the operands
+ * split into bf16 terms and the split weights: B = 1, C = CH = 128 fits up to N = 142).  All calls on one
+ * GPU share that GPU's array: calls that overlap on one GPU (two streams, two threads) race; calls on
+ * one stream are ordered.  The first call on a device looks up the array's address and the kernels'
+ * launch geometry (hipGetSymbolAddress, occupancy and attribute queries), which a stream capture does
+ * not allow: make one eager call per device (any size) before capturing a graph that contains this
+ * entry point; every later call issues kernel launches only. */
 #define OF3_STATIC_SCRATCH_BYTES (48u << 20)
 int of3_trimul_fwd_static(const void* z, const int64_t z_strides[3], const float* mask,
                           const int64_t mask_strides[3], const void* ln_in_w, const void* ln_in_b, const void* ln_out_w,

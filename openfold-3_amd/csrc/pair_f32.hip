@@ -284,9 +284,10 @@ struct WeightSplitter {
     ++j.n;
     w += 3 * dst.plane;
   }
-  void launch(hipStream_t stream) const {
+  hipError_t launch(hipStream_t stream) const {
     const long items = j.first[j.n];
     hipLaunchKernelGGL(split_weights_f32, dim3((unsigned)((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, j);
+    return hipGetLastError();
   }
 };
 
@@ -2335,7 +2336,7 @@ hipError_t trimul_fwd_f32(const TrimulF32Args& a, hipStream_t stream) {
     splitter.add(a.w_bg, a.CH, a.C, p.s_bg);
     splitter.add(a.w_g, a.C, a.C, p.s_g);
     splitter.add(a.w_z, a.C, a.CH, p.s_z);
-    splitter.launch(stream);
+    if (hipError_t es = splitter.launch(stream); es != hipSuccess) return es;  // no kernel may read unsplit weights
     auto proj = split_ab ? (fast ? trimul_proj_x3_f32<kXT, kPT, true, true> : trimul_proj_x3_f32<kXT, kPT, false, true>)
                          : (fast ? trimul_proj_x3_f32<kXT, kPT, true, false> : trimul_proj_x3_f32<kXT, kPT, false, false>);
     hipError_t e = allow_lds<trimul_proj_x3_f32<kXT, kPT, false, false>>(kLdsLimit);
@@ -2452,7 +2453,7 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     splitter.add(a.w_v, HD, a.C, p.s_v);
     splitter.add(a.w_g, HD, a.C, p.s_g);
     splitter.add(a.w_o, a.C, HD, p.s_o);
-    splitter.launch(stream);
+    if (hipError_t es = splitter.launch(stream); es != hipSuccess) return es;  // no kernel may read unsplit weights
     auto proj = core_x3 ? (fast ? triattn_proj_x3_f32<kXT, kPT, true, true> : triattn_proj_x3_f32<kXT, kPT, true, false>)
                         : (fast ? triattn_proj_x3_f32<kXT, kPT, false, true> : triattn_proj_x3_f32<kXT, kPT, false, false>);
     hipError_t e = allow_lds<triattn_proj_x3_f32<kXT, kPT, false, false>>(kLdsLimit);
@@ -2538,7 +2539,7 @@ hipError_t transition_fwd_f32(const TransitionF32Args& a, hipStream_t stream) {
     splitter.add(a.w_a, a.HID, a.C, p.s_a);
     splitter.add(a.w_b, a.HID, a.C, p.s_b);
     splitter.add(a.w_out, a.C, a.HID, p.s_out);
-    splitter.launch(stream);
+    if (hipError_t es = splitter.launch(stream); es != hipSuccess) return es;  // no kernel may read unsplit weights
     const bool fast = a.C % 64 == 0 && (reinterpret_cast<uintptr_t>(a.x) & 7u) == 0 && even_strides(a.x_view);
     const bool wide = a.C > 128;
     auto kern = wide ? (fast ? transition_x3_f32<true, true> : transition_x3_f32<true, false>)

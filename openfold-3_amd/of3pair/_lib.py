@@ -9,6 +9,7 @@ import ctypes
 import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 
+from . import build as _build
 from .build import LIB_PATH
 
 OF3_OK, OF3_EINVAL, OF3_ENOSPC, OF3_EHIP, OF3_ESTATIC = 0, -1, -2, -3, -4
@@ -67,6 +68,10 @@ def load() -> ctypes.CDLL:
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(
                 "libof3pair.so is not built (%s); build it with `python -m of3pair.build`" % LIB_PATH)
+        if LIB_PATH == _build.LIB_PATH and _build.is_stale():
+            raise RuntimeError(
+                "libof3pair.so is older than its sources (%s was edited after the build); rebuild it with "
+                "`python -m of3pair.build`" % _build.CSRC)
         lib = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)

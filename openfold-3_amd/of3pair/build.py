@@ -7,6 +7,7 @@ installed outside the tree.
 """
 from __future__ import annotations
 
+import hashlib
 import os
 import subprocess
 import sys
@@ -17,6 +18,8 @@ ROOT = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(ROOT, "csrc")
 LIB_DIR = os.path.join(ROOT, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libof3pair.so")
+STAMP_PATH = os.path.join(LIB_DIR, "libof3pair.sources.sha256")
+INCLUDE_DIR = os.path.join(os.path.dirname(ROOT), "include")
 
 SOURCES = [
     "of3pair_api.hip",
@@ -58,8 +61,25 @@ def _run(cmd):
     return out
 
 
+def source_digest() -> str:
+    """sha256 over everything the library is compiled from: the kernel sources and headers, the public
+    header and the compiler flags."""
+    h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
+    files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".h"))]
+    if os.path.isdir(INCLUDE_DIR):
+        files += [os.path.join(INCLUDE_DIR, f) for f in sorted(os.listdir(INCLUDE_DIR)) if f.endswith(".h")]
+    for path in files:
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
 def build(verbose: bool = False, jobs: int = 4) -> str:
     os.makedirs(LIB_DIR, exist_ok=True)
+    digest = source_digest()
+    if os.path.exists(STAMP_PATH):
+        os.remove(STAMP_PATH)  # no stamp while the objects are in flux
     objs = []
 
     def compile_one(src):
@@ -72,11 +92,24 @@ def build(verbose: bool = False, jobs: int = 4) -> str:
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(compile_one, SOURCES))
     _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs])
+    with open(STAMP_PATH, "w") as fh:
+        fh.write(digest + "\n")
     return LIB_PATH
 
 
 def is_built() -> bool:
-    return os.path.exists(LIB_PATH)
+    """True when the library exists and was built from the sources as they are now (the stamp
+    written next to it holds the digest of the sources of that build)."""
+    return os.path.exists(LIB_PATH) and not is_stale()
+
+
+def is_stale() -> bool:
+    """True when a library exists whose sources are known to have changed since it was built (a
+    library without a stamp, e.g. one copied in from elsewhere, cannot be judged and is accepted)."""
+    if not os.path.exists(LIB_PATH) or not os.path.exists(STAMP_PATH):
+        return False
+    with open(STAMP_PATH) as fh:
+        return fh.read().strip() != source_digest()
 
 
 if __name__ == "__main__":

@@ -16,22 +16,32 @@ import torch
 from . import _lib
 
 _workspaces: dict = {}
+_in_graph: set = set()  # keys of the buffers a stream capture has handed to kernels
 _retired: list = []
 
 
 def _workspace(device, nbytes: int) -> torch.Tensor:
     """Grow-only scratch per (device, current stream), owned by this Python layer (the library
     allocates nothing).  Kernels on one stream are ordered, so all modules running on a stream share
-    its buffer; another stream gets a buffer of its own.  A buffer that is outgrown is kept alive
-    until release_workspaces(): a HIP graph captured earlier still replays kernels that point into
-    it, and the caching allocator must not hand that memory to another tensor."""
+    its buffer; another stream gets a buffer of its own.  A buffer that is outgrown is freed, unless a
+    stream capture has used it: a HIP graph captured earlier still replays kernels that point into it
+    and the caching allocator must not hand that memory to another tensor, so such a buffer is kept
+    alive until release_workspaces()."""
     key = (device, torch.cuda.current_stream(device).cuda_stream)
+    capturing = torch.cuda.is_current_stream_capturing()
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        if buf is not None:
+        if buf is not None and key in _in_graph:
             _retired.append(buf)
+        _in_graph.discard(key)
+        # an eager buffer goes back to the allocator before its successor is requested (kernels already
+        # queued on this stream keep it valid: the allocator reuses it for later work of the stream only)
+        _workspaces.pop(key, None)
+        del buf
         buf = torch.empty(int(nbytes), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
+    if capturing:
+        _in_graph.add(key)
     return buf
 
 
@@ -39,6 +49,7 @@ def release_workspaces():
     """Drops every scratch buffer, current and outgrown.  Only when no captured graph that used them
     will be replayed again."""
     _workspaces.clear()
+    _in_graph.clear()
     _retired.clear()
 
 
@@ -208,6 +219,14 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
     HID = a_weight.shape[0]
     if tuple(a_weight.shape) != (HID, C) or tuple(b_weight.shape) != (HID, C) or tuple(out_weight.shape) != (C, HID):
         raise ValueError("transition weights must be [n*C, C], [n*C, C] and [C, n*C]")
+    # which kernels serve these widths is decided from the shape alone: any other refusal of the
+    # library (alignment, strides, null pointers) is the caller's error and is raised
+    bf16_widths = C in (64, 128) and HID >= 128 and HID % 32 == 0 and HID <= (1 << 16)
+    fp32_widths = 1 <= C <= 256 and 1 <= HID <= 1024
+    if code == _lib.OF3_DTYPE_BF16 and not bf16_widths and fp32_widths:
+        return _through_fp32(swiglu_transition, x, inplace, mask, norm_weight, norm_bias, a_weight, b_weight, out_weight,
+                             add_residual=add_residual)
+    served = bf16_widths if code == _lib.OF3_DTYPE_BF16 else fp32_widths
     keep = [_w(t, x.dtype) for t in (norm_weight, norm_bias, a_weight, b_weight, out_weight)]
     m3, mptr, mstr = _mask_arg(mask, lead, B, N, x.device)
     out4 = x4 if inplace else _out_like(x4)
@@ -218,10 +237,7 @@ def swiglu_transition(x, mask, norm_weight, norm_bias, a_weight, b_weight, out_w
                                        *[k.data_ptr() for k in keep], out4.data_ptr(), B, N, C, HID,
                                        int(bool(add_residual)), ws.data_ptr() if ws is not None else None,
                                        need if ws is not None else 0, code, _stream(x))
-    if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and C <= 256 and HID <= 1024:
-        return _through_fp32(swiglu_transition, x, inplace, mask, norm_weight, norm_bias, a_weight, b_weight, out_weight,
-                             add_residual=add_residual)
-    if st == _lib.OF3_EINVAL:
+    if st == _lib.OF3_EINVAL and not served:
         raise ValueError("pair transition: bf16 supports c_in 64 or 128 with a hidden width n*c_in that is a multiple "
                          "of 32 and at least 128, fp32 c_in <= 256 and n*c_in <= 1024; got c_in=%d hidden=%d in %s"
                          % (C, HID, x.dtype))
@@ -282,6 +298,12 @@ def pair_bias(z, norm_weight, norm_bias, weight):
     H = weight.shape[0]
     if tuple(weight.shape) != (H, C):
         raise ValueError("pair-bias weight must be [no_heads, c_z]")
+    bf16_widths = C in (64, 128) and H <= 32
+    fp32_widths = C <= 256 and H <= 64
+    if code == _lib.OF3_DTYPE_BF16 and not bf16_widths and fp32_widths:
+        # widths the bf16 kernel does not serve: the fp32 kernel on widened activations, rounded once at the end
+        return pair_bias(z.float(), norm_weight, norm_bias, weight).to(torch.bfloat16)
+    served = bf16_widths if code == _lib.OF3_DTYPE_BF16 else fp32_widths
     nw, w = _w(norm_weight, z.dtype), _w(weight, z.dtype)
     nb = None if norm_bias is None else _w(norm_bias, z.dtype)
     out = torch.empty(B, H, N, N, dtype=z.dtype, device=z.device)
@@ -289,10 +311,7 @@ def pair_bias(z, norm_weight, norm_bias, weight):
         st = lib.of3_pair_bias_fwd(z4.data_ptr(), _lib.strides3(z4.stride()[:3]), nw.data_ptr(),
                                    None if nb is None else nb.data_ptr(), w.data_ptr(), out.data_ptr(), B, N, C, H,
                                    code, _stream(z))
-    if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and C <= 256 and H <= 64:
-        # widths the bf16 kernel does not serve: the fp32 kernel on widened activations, rounded once at the end
-        return pair_bias(z.float(), norm_weight, norm_bias, weight).to(torch.bfloat16)
-    if st == _lib.OF3_EINVAL:
+    if st == _lib.OF3_EINVAL and not served:
         raise ValueError("pair bias: bf16 supports c_z 64 or 128 and up to 32 heads, fp32 c_z <= 256 and up to 64 "
                          "heads; got c_z=%d heads=%d in %s" % (C, H, z.dtype))
     _lib.check(st, "of3_pair_bias_fwd")
@@ -304,17 +323,19 @@ def layer_norm(x, weight, bias):
     (template_module.py:376).  Returns a new contiguous tensor of x's shape and dtype."""
     code = _require_gpu(x, "x")
     lib = _lib.load()
+    C = x.shape[-1]
+    bf16_widths = C in (64, 128)
+    if code == _lib.OF3_DTYPE_BF16 and not bf16_widths and C <= 256:
+        return layer_norm(x.float(), weight, bias).to(torch.bfloat16)  # the fp32 kernel, rounded once at the end
+    served = bf16_widths if code == _lib.OF3_DTYPE_BF16 else C <= 256
     xc = x.contiguous()
-    C = xc.shape[-1]
     rows = xc.numel() // C
     out = torch.empty_like(xc)
     w, b = _w(weight, x.dtype), _w(bias, x.dtype)
     with torch.cuda.device(x.device):
         st = lib.of3_layer_norm_fwd(xc.data_ptr(), w.data_ptr(), b.data_ptr(), out.data_ptr(), rows, C, code,
                                     _stream(x))
-    if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and C <= 256:
-        return layer_norm(x.float(), weight, bias).to(torch.bfloat16)  # the fp32 kernel, rounded once at the end
-    if st == _lib.OF3_EINVAL:
+    if st == _lib.OF3_EINVAL and not served:
         raise ValueError("layer norm: bf16 supports 64 or 128 channels, fp32 up to 256; got %d in %s" % (C, x.dtype))
     _lib.check(st, "of3_layer_norm_fwd")
     return out
@@ -339,6 +360,12 @@ def template_tail(t, norm_weight, norm_bias, linear_t_weight, apply_layer_norm: 
     CZ = linear_t_weight.shape[0]
     if tuple(linear_t_weight.shape) != (CZ, CT):
         raise ValueError("linear_t weight must be [c_z, c_t]")
+    bf16_widths = CT == 64 and CZ == 128
+    fp32_widths = CT <= 256 and CZ <= 4096
+    if code == _lib.OF3_DTYPE_BF16 and not bf16_widths and fp32_widths:
+        # the fp32 kernel on widened activations, rounded once at the end
+        return template_tail(t.float(), norm_weight, norm_bias, linear_t_weight, apply_layer_norm).to(torch.bfloat16)
+    served = bf16_widths if code == _lib.OF3_DTYPE_BF16 else fp32_widths
     w = _w(linear_t_weight, t.dtype)
     nw = _w(norm_weight, t.dtype) if apply_layer_norm else None
     nb = _w(norm_bias, t.dtype) if apply_layer_norm else None
@@ -347,10 +374,7 @@ def template_tail(t, norm_weight, norm_bias, linear_t_weight, apply_layer_norm: 
         st = lib.of3_template_tail_fwd(tc.data_ptr(), None if nw is None else nw.data_ptr(),
                                        None if nb is None else nb.data_ptr(), w.data_ptr(), out.data_ptr(), B, T,
                                        N * N, CT, CZ, 1 if apply_layer_norm else 0, code, _stream(t))
-    if st == _lib.OF3_EINVAL and code == _lib.OF3_DTYPE_BF16 and CT <= 256:
-        # the fp32 kernel on widened activations, rounded once at the end
-        return template_tail(t.float(), norm_weight, norm_bias, linear_t_weight, apply_layer_norm).to(torch.bfloat16)
-    if st == _lib.OF3_EINVAL:
+    if st == _lib.OF3_EINVAL and not served:
         raise ValueError("template tail: bf16 supports c_t = 64 with c_z = 128, fp32 c_t <= 256; got c_t=%d c_z=%d "
                          "in %s" % (CT, CZ, t.dtype))
     _lib.check(st, "of3_template_tail_fwd")

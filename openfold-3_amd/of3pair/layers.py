@@ -18,6 +18,7 @@ import torch
 import torch.nn as nn
 
 from . import functional as F3
+from ._guard import forward_only
 
 
 def _truncated_normal_(weight: torch.Tensor, scale: float = 1.0):
@@ -93,7 +94,7 @@ class TriangleMultiplicativeUpdate(nn.Module):
         for name, default in TRI_MUL_INIT.items():
             _init_linear(getattr(self, name), _init_name(linear_init_params, name, default))
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, z, mask=None, inplace_safe=False, use_cueq_triangle_kernels=False,
                 _add_with_inplace=False, _inplace_chunk_size=256):
         """z [*, N, N, C_z], mask [*, N, N] -> [*, N, N, C_z].
@@ -162,7 +163,7 @@ class TriangleAttention(nn.Module):
             mha_init = linear_init_params["mha"] if "mha" in linear_init_params else None
         self.mha = _GatedAttentionParams(c_in, c_hidden, no_heads, mha_init)
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, x, mask=None, chunk_size=None, use_deepspeed_evo_attention=False,
                 use_cueq_triangle_kernels=False, use_lma=False, inplace_safe=False,
                 _add_residual=False):
@@ -227,7 +228,7 @@ class SwiGLUTransition(nn.Module):
         self.linear_out = nn.Linear(n * c_in, c_in, bias=False)
         _init_linear(self.linear_out, _init_name(linear_init_params, "linear_out", SWIGLU_TRANSITION_INIT["linear_out"]))
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, x, mask=None, chunk_size=None, ckpt_chunk_size=None, _add_residual=False, _inplace=False):
         """x [*, N, N, C_in], mask [*, N, N] or None (all ones, transition.py:106-107) -> the
         update.  chunk_size / ckpt_chunk_size of the reference are accepted and ignored: the
@@ -254,7 +255,7 @@ class PairBiasProjection(nn.Module):
         self.linear_z = nn.Linear(c_z, no_heads, bias=False)
         _init_linear(self.linear_z, linear_init)
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, z):
         return F3.pair_bias(z, self.layer_norm_z.weight, self.layer_norm_z.bias, self.linear_z.weight)
 
@@ -308,7 +309,7 @@ class AttentionPairBias(nn.Module):
         _init_linear(self.linear_z, _init_name(linear_init_params, "linear_z", "default"))
         self.mha = _PairBiasAttentionParams(c_q, c_hidden, no_heads, mha_init)
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, a, z, s=None, mask=None, use_deepspeed_evo_attention=False, use_cueq_triangle_kernels=False,
                 use_lma=False, use_high_precision_attention=False, _add_residual: bool = False,
                 _inplace: bool = False):

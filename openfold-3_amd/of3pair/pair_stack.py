@@ -13,6 +13,7 @@ import torch
 import torch.nn as nn
 
 from . import functional as F3
+from ._guard import forward_only
 from .layers import (SwiGLUTransition, TriangleAttention, TriangleMultiplicationIncoming,
                      TriangleMultiplicationOutgoing)
 
@@ -55,14 +56,14 @@ class PairStack(nn.Module):
             module.mha.linear_g.weight, module.mha.linear_o.weight,
             no_heads=module.no_heads, inf=module.inf, add_residual=True, inplace=inplace)
 
-    @torch.no_grad()
+    @forward_only
     def tri_mul_out_in(self, z, pair_mask, inplace_safe: bool = False, use_cueq_triangle_kernels: bool = False):
         """base_blocks.py:307-351.  Without inplace_safe the caller's tensor is left intact:
         the first z + update lands in a new tensor, which the second module then overwrites."""
         z = self._mul(self.tri_mul_out, z, pair_mask, inplace=inplace_safe)
         return self._mul(self.tri_mul_in, z, pair_mask, inplace=True)
 
-    @torch.no_grad()
+    @forward_only
     def tri_att_start_end(self, z, pair_mask, _attn_chunk_size=None, use_deepspeed_evo_attention=False,
                           use_cueq_triangle_kernels=False, use_lma=False, inplace_safe: bool = False):
         """base_blocks.py:353-406; the ending node is the starting-node module run on the
@@ -73,7 +74,7 @@ class PairStack(nn.Module):
         zt = self._att(self.tri_att_end, zt, mt, inplace=True)
         return zt.transpose(-2, -3)
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, z, pair_mask, chunk_size=None, use_deepspeed_evo_attention=False,
                 use_cueq_triangle_kernels=False, use_lma=False, inplace_safe: bool = False,
                 _attn_chunk_size=None):
@@ -108,7 +109,7 @@ class PairBlock(PairStack):
         self.pair_transition = SwiGLUTransition(c_z, transition_n, linear_init_params=pt)
         self.pair_dropout = pair_dropout
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, z, pair_mask, chunk_size=None, use_deepspeed_evo_attention=False,
                 use_cueq_triangle_kernels=False, use_lma=False, inplace_safe: bool = False,
                 _mask_trans: bool = True, _attn_chunk_size=None):

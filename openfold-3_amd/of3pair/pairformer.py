@@ -9,6 +9,7 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from ._guard import forward_only
 from .layers import AttentionPairBias, SwiGLUTransition
 from .pair_stack import PairBlock
 
@@ -41,7 +42,7 @@ class PairFormerBlock(nn.Module):
             tr = tr["swiglu"]
         self.single_transition = SwiGLUTransition(c_in=c_s, n=transition_n, linear_init_params=tr)
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, s, z, single_mask, pair_mask, chunk_size=None, use_deepspeed_evo_attention=False,
                 use_cueq_triangle_kernels=False, use_lma=False, inplace_safe: bool = False, _mask_trans: bool = True,
                 _attn_chunk_size=None):
@@ -76,7 +77,7 @@ class PairFormerStack(nn.Module):
             for _ in range(no_blocks)
         ])
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, s, z, single_mask, pair_mask, chunk_size=None, use_deepspeed_evo_attention=False,
                 use_cueq_triangle_kernels=False, use_lma=False, inplace_safe: bool = False, _mask_trans: bool = True):
         """s [*, N, C_s], z [*, N, N, C_z], single_mask [*, N], pair_mask [*, N, N] -> (s, z)

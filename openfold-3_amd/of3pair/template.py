@@ -13,6 +13,7 @@ import torch
 import torch.nn as nn
 
 from . import functional as F3
+from ._guard import forward_only
 from .layers import _init_linear, _init_name
 from .pair_stack import PairBlock
 
@@ -31,7 +32,7 @@ class TemplatePairBlock(PairBlock):
                          linear_init_params=linear_init_params)
         self.tri_mul_first = tri_mul_first
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, z, mask, chunk_size=None, use_deepspeed_evo_attention=False, use_cueq_triangle_kernels=False,
                 use_lma=False, inplace_safe: bool = False, _mask_trans: bool = True, _attn_chunk_size=None):
         """z [*, N_templ, N, N, C_t], mask [*, N_templ, N, N] -> updated z.  Without inplace_safe
@@ -75,7 +76,7 @@ class TemplatePairStack(nn.Module):
             mask = mask.expand(*shape)
         return mask
 
-    @torch.no_grad()
+    @forward_only
     def run_blocks(self, t, mask, inplace_safe: bool = False, _mask_trans: bool = True):
         """The blocks without the closing LayerNorm (the embedder fuses it into its tail)."""
         mask = self._expand_mask(t, mask)
@@ -84,7 +85,7 @@ class TemplatePairStack(nn.Module):
             t = blk(t, mask, inplace_safe=inplace_safe or i > 0, _mask_trans=_mask_trans)
         return t
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, t, mask, chunk_size=None, use_deepspeed_evo_attention=False, use_cueq_triangle_kernels=False,
                 use_lma=False, inplace_safe: bool = False, _mask_trans: bool = True):
         """t [*, N_templ, N, N, C_t], mask [*, N_templ, N, N] or [*, 1, N, N] -> LayerNorm of the
@@ -106,7 +107,7 @@ class TemplateEmbedderCore(nn.Module):
         self.linear_t = nn.Linear(c_t, c_z, bias=False)
         _init_linear(self.linear_t, _init_name(linear_init_params, "linear_t", "default"))
 
-    @torch.no_grad()
+    @forward_only
     def forward(self, template_embeds, pair_mask, chunk_size=None, _mask_trans: bool = True,
                 use_deepspeed_evo_attention=False, use_cueq_triangle_kernels=False, use_lma=False,
                 inplace_safe: bool = False):

@@ -132,9 +132,10 @@ def test_pair_block_in_a_hip_graph_replays_like_eager():
 
 
 def test_outgrown_workspace_stays_valid_for_a_captured_graph():
-    """A graph captured at a small N keeps pointing into the scratch buffer of its capture; later
-    eager calls at a larger N need more scratch.  The outgrown buffer must stay alive (and the graph's
-    own buffer untouched), so the replay still reproduces the eager result of the small problem."""
+    """A graph captured at a small N keeps pointing into the scratch buffer of its capture (the capture
+    stream has a buffer of its own); later eager calls at a larger N need more scratch on their stream.
+    The eager buffer they outgrow was never handed to a capture and is freed, not hoarded; the graph's
+    buffer is untouched, so the replay still reproduces the eager result of the small problem."""
     from of3pair import functional as F3
 
     lib()
@@ -149,11 +150,11 @@ def test_outgrown_workspace_stays_valid_for_a_captured_graph():
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         out_static = blk(z_static, m_small)
-    retired_before = len(F3._retired)
-    z_big = orc.round_bf16(orc.make_pair_input(32, (1,), 160, 128)).to(DEV).to(torch.bfloat16)
-    big = blk(z_big, torch.ones(1, 160, 160, device=DEV))  # grows the eager stream's scratch
-    assert torch.isfinite(big).all()
-    assert len(F3._retired) > retired_before, "the outgrown buffer is kept until release_workspaces()"
+    for n in (96, 160, 224):  # eager calls of rising length: each outgrows the eager stream's scratch
+        z_big = orc.round_bf16(orc.make_pair_input(32, (1,), n, 128)).to(DEV).to(torch.bfloat16)
+        big = blk(z_big, torch.ones(1, n, n, device=DEV))
+        assert torch.isfinite(big).all()
+        assert len(F3._retired) == 0, "an eager buffer no capture has used is freed when it is outgrown"
     filler = torch.full((64 << 20,), 7, dtype=torch.uint8, device=DEV)  # would land in freed scratch memory
     for rep in range(2):
         z_static.copy_(z_small)
@@ -161,6 +162,46 @@ def test_outgrown_workspace_stays_valid_for_a_captured_graph():
         torch.cuda.synchronize()
         assert torch.equal(out_static, eager_small), "replay %d after the workspace grew" % rep
     assert int(filler[0]) == 7
+
+
+def test_workspace_used_by_a_capture_is_kept_when_outgrown():
+    """Warm-up and capture on one side stream share that stream's scratch buffer, so the graph points
+    into it.  A larger eager call on the same stream outgrows it: the buffer must be kept alive (retired,
+    not freed) until release_workspaces(), and the replay must still give the small problem's result."""
+    from of3pair import functional as F3
+
+    lib()
+    torch.cuda.synchronize()
+    F3.release_workspaces()
+    blk, _ = _block(128, 32, seed=6)
+    z_small = orc.round_bf16(orc.make_pair_input(33, (1,), 40, 128)).to(DEV).to(torch.bfloat16)
+    m_small = torch.ones(1, 40, 40, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        eager_small = blk(z_small, m_small)  # allocates the side stream's scratch, eagerly
+    side.synchronize()
+    z_static = z_small.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out_static = blk(z_static, m_small)  # same stream, same buffer: now referenced by the graph
+    assert len(F3._retired) == 0
+    with torch.cuda.stream(side):
+        z_big = orc.round_bf16(orc.make_pair_input(34, (1,), 160, 128)).to(DEV).to(torch.bfloat16)
+        big = blk(z_big, torch.ones(1, 160, 160, device=DEV))
+    side.synchronize()
+    assert torch.isfinite(big).all()
+    assert len(F3._retired) == 1, "a buffer a captured graph points into is kept until release_workspaces()"
+    filler = torch.full((64 << 20,), 7, dtype=torch.uint8, device=DEV)
+    for rep in range(2):
+        z_static.copy_(z_small)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, eager_small), "replay %d after the workspace grew" % rep
+    assert int(filler[0]) == 7
+    del graph
+    F3.release_workspaces()
 
 
 def test_bf16_widths_outside_the_mfma_kernels_run_on_the_fp32_kernels():

@@ -80,15 +80,15 @@ def test_pair_stack_submodule_names():
 
 def test_no_cpu_fallback():
     """The shipped path has no CPU implementation: CPU tensors are refused loudly."""
-    m = of3pair.TriangleMultiplicationOutgoing(128, 128).to(torch.bfloat16)
+    m = of3pair.TriangleMultiplicationOutgoing(128, 128).to(torch.bfloat16).eval()
     z = torch.zeros(1, 8, 8, 128, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="GPU"):
         m(z)
-    a = of3pair.TriangleAttention(128, 32, 4).to(torch.bfloat16)
+    a = of3pair.TriangleAttention(128, 32, 4).to(torch.bfloat16).eval()
     with pytest.raises(RuntimeError, match="GPU"):
         a(z)
     with pytest.raises(RuntimeError, match="GPU"):  # fp32 has no CPU path either
-        of3pair.TriangleMultiplicationOutgoing(128, 128)(z.float())
+        of3pair.TriangleMultiplicationOutgoing(128, 128).eval()(z.float())
 
 
 def test_package_does_not_import_the_oracle():
@@ -250,3 +250,45 @@ def test_whole_pairformer_stack_loads_from_a_model_state_dict():
         assert torch.equal(v, sd["model.pairformer_stack." + k])
     with pytest.raises(KeyError):
         ck.load_pairformer_stack(of3pair.PairFormerStack(**dict(cfg, no_blocks=3)), sd)
+
+
+def test_modules_refuse_training_mode_and_inputs_that_want_gradients():
+    """The kernels are the inference forward pass: no dropout, no autograd.  A module left in training
+    mode (where the reference would apply pair_dropout and record gradients) or an input that requires
+    a gradient must raise instead of silently returning an un-dropped, non-differentiable result."""
+    blk = of3pair.PairBlock(64, 64, 16, 4, "swiglu", 2, 0.25, False, 1e9)
+    z = torch.zeros(1, 8, 8, 64)
+    mask = torch.ones(1, 8, 8)
+    assert blk.training
+    with pytest.raises(RuntimeError, match="forward-only"):
+        blk(z, mask)
+    with torch.no_grad(), pytest.raises(RuntimeError, match="forward-only"):
+        blk(z, mask)  # train mode without autograd would still skip the dropout
+    blk.eval()
+    with pytest.raises(RuntimeError, match="requires a gradient"):
+        blk(z.clone().requires_grad_(True), mask)
+    for m in (of3pair.TriangleMultiplicationOutgoing(64, 64), of3pair.TriangleAttention(64, 16, 4),
+              of3pair.SwiGLUTransition(64, 2), of3pair.PairBiasProjection(64, 16)):
+        with pytest.raises(RuntimeError, match="forward-only"):
+            m(z) if isinstance(m, of3pair.PairBiasProjection) else m(z, mask)
+    # in eval mode the only refusal left is the missing device (no CPU path)
+    with pytest.raises(RuntimeError, match="GPU"):
+        blk(z, mask)
+
+
+def test_build_stamp_detects_edited_sources(tmp_path, monkeypatch):
+    """is_built() is more than a file-exists test: the digest written at build time must match the
+    sources as they are now, and the loader refuses a library whose sources changed."""
+    from of3pair import build as B
+
+    lib = tmp_path / "libof3pair.so"
+    stamp = tmp_path / "libof3pair.sources.sha256"
+    monkeypatch.setattr(B, "LIB_PATH", str(lib))
+    monkeypatch.setattr(B, "STAMP_PATH", str(stamp))
+    assert not B.is_built() and not B.is_stale()
+    lib.write_bytes(b"\x7fELF")
+    assert B.is_built()  # no stamp: cannot be judged, accepted
+    stamp.write_text(B.source_digest() + "\n")
+    assert B.is_built() and not B.is_stale()
+    stamp.write_text("0" * 64 + "\n")
+    assert B.is_stale() and not B.is_built()

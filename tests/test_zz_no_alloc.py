@@ -65,6 +65,45 @@ def test_static_scratch_matches_workspace_entry_point_twice():
     _both(L, 1, 40, 128, torch.float32, 0, seed=15)
 
 
+@pytest.mark.gpu
+def test_static_entry_point_under_graph_capture_after_an_eager_call():
+    """The callers the entry point is for include code under stream capture.  The first call on a device
+    does look-ups that a capture does not allow, so one eager call comes first; after it the entry point
+    issues kernel launches only and can be captured.  Every replay (with eager work and synchronisations
+    in between) must reproduce the eager result bit for bit."""
+    L = lib()
+    B, N, C = 1, 96, 128
+    code = _lib.OF3_DTYPE_BF16
+    z, mask, dp, _ = _case(21, B, N, C, torch.bfloat16, 1)
+    w = [t.data_ptr() for t in dp]
+    eager = torch.empty_like(z)
+    print("trimul static under capture: B=%d N=%d C=%d" % (B, N, C), flush=True)
+    st = L.of3_trimul_fwd_static(z.data_ptr(), s3(z), mask.data_ptr(), s3(mask), *w, eager.data_ptr(), B, N, C, C, 1, 1,
+                                 code, stream())
+    _lib.check(st, "of3_trimul_fwd_static (eager warm-up)")
+    torch.cuda.synchronize()
+    z_static = z.clone()
+    out_static = torch.empty_like(z)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        st = L.of3_trimul_fwd_static(z_static.data_ptr(), s3(z_static), mask.data_ptr(), s3(mask), *w,
+                                     out_static.data_ptr(), B, N, C, C, 1, 1, code, stream())
+    _lib.check(st, "of3_trimul_fwd_static (captured)")
+    for rep in range(3):
+        # eager work between the replays that also uses the built-in scratch (a smaller problem)
+        z2, m2, dp2, _ = _case(22 + rep, 1, 40, C, torch.bfloat16, 0)
+        o2 = torch.empty_like(z2)
+        st = L.of3_trimul_fwd_static(z2.data_ptr(), s3(z2), m2.data_ptr(), s3(m2), *[t.data_ptr() for t in dp2],
+                                     o2.data_ptr(), 1, 40, C, C, 0, 1, code, stream())
+        _lib.check(st, "of3_trimul_fwd_static (eager between replays)")
+        torch.cuda.synchronize()
+        out_static.zero_()
+        z_static.copy_(z)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, eager), "replay %d differs from the eager call" % rep
+
+
 def test_static_scratch_rejects_what_does_not_fit():
     """No GPU needed: sizes are checked before the first HIP call."""
     L = lib()
@@ -78,6 +117,12 @@ def test_static_scratch_rejects_what_does_not_fit():
     assert call(257) == _lib.OF3_ESTATIC
     assert call(384) == _lib.OF3_ESTATIC
     assert call(200, dtype=_lib.OF3_DTYPE_F32) == _lib.OF3_ESTATIC
+    # fp32 at C = CH = 128: the rule is the workspace size, not B*CH*N*N (N = 143..160 are below 2^22 there)
+    f32 = _lib.OF3_DTYPE_F32
+    assert L.of3_trimul_workspace_bytes_for(f32, 1, 142, 128, 128) <= _lib.OF3_STATIC_SCRATCH_BYTES
+    assert L.of3_trimul_workspace_bytes_for(f32, 1, 143, 128, 128) > _lib.OF3_STATIC_SCRATCH_BYTES
+    assert call(143, dtype=f32) == _lib.OF3_ESTATIC
+    assert call(160, dtype=f32) == _lib.OF3_ESTATIC
     assert call(64, C=96) == _lib.OF3_EINVAL
     assert call(64, dtype=5) == _lib.OF3_EINVAL
     assert b"OF3_STATIC_SCRATCH_BYTES" in L.of3_status_string(_lib.OF3_ESTATIC)
