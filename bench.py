@@ -36,6 +36,10 @@ with inplace_safe, where z drifts from step to step, for comparison) the line ca
   template_block_ms  {"bf16", "fp32"}: wall clock of one block of the template pair stack (of3pair.PairBlock,
                 4 templates, N = 512, c_t = 64, 4 heads x 16, transition n = 2, padded tails: the benchmark's
                 fourth configuration whatever --n says), for orientation;
+  configs       the benchmark's configurations 2, 4 and 5 (N = 384 with a padded tail; the 2-block template
+                pair stack over 4 templates at N = 512, c_t = 64, 4 x 16; 4 stacked blocks in place at N = 2048):
+                wall clock through the modules ("ms", "ms_per_block") and the block's six kernels against their
+                roofs, measured like `kernels`; not part of `value` (--configs '' leaves them out);
   cpu_baseline  the CPU oracle (fp32 PyTorch restatement of the reference's stock path) on the host
                 cores for the same workload: one warm-up run, then the median of three.
 """
@@ -72,8 +76,9 @@ C_S, C_HEAD_S = 384, 24    # single representation and head width of its attenti
 METRIC = "ms per Pairformer pair-stack block at N=768 bf16; % of MFMA peak & HBM GB/s"
 
 
-def kernel_model(B, N, C, CH, H, D):
+def kernel_model(B, N, C, CH, H, D, transition_n=None):
     """Algorithmic work per launch.  U = one bf16 pass over z."""
+    transition_n = TRANSITION_N if transition_n is None else transition_n
     U = B * N * N * C * 2
     hd = H * D
     return {
@@ -90,7 +95,7 @@ def kernel_model(B, N, C, CH, H, D):
         # reads o and x, writes out
         "triattn_out": {"bound": "hbm", "bytes": B * N * N * hd * 2 + 2 * U},
         # the transition after the block (n = 4): three C x 4C products per position
-        "pair_transition": {"bound": "mfma", "flops": 6 * B * N * N * C * (TRANSITION_N * C)},
+        "pair_transition": {"bound": "mfma", "flops": 6 * B * N * N * C * (transition_n * C)},
         # reads z, writes the [PAIR_BIAS_HEADS, N, N] bias
         "pair_bias_proj": {"bound": "hbm", "bytes": U + B * PAIR_BIAS_HEADS * N * N * 2},
         # LayerNorm + q, k, v, g projections, QK^T and PV over 16 heads of 24, output projection
@@ -100,6 +105,202 @@ def kernel_model(B, N, C, CH, H, D):
         # reads the TEMPLATES planes of c_t channels, writes one c_z plane
         "template_tail": {"bound": "hbm", "bytes": B * N * N * 2 * (TEMPLATES * C_T + C)},
     }
+
+
+def block_stage_launches(lib, _lib, torch, dp, zz, mask, dims, contract_variant=0):
+    """The pair-stack block issued kernel by kernel through the stage entry points of the C ABI, in the
+    order the block runs them (trimul out, trimul in, tri-attn start, tri-attn end), in place on zz.
+    dp: device parameters under the PairStack names; returns [(kernel name, launch function)] and the
+    intermediates and stride arrays that have to stay alive."""
+    B, N, C, CH, H, D = dims
+    dev, bf = zz.device, torch.bfloat16
+    s = torch.cuda.current_stream().cuda_stream
+    Np = lib.of3_padded_n(N)
+    sb, si, sj = zz.stride()[:3]
+    z_fwd, z_tr = _lib.strides3((sb, si, sj)), _lib.strides3((sb, sj, si))
+    mb_, mi, mj = mask.stride()
+    m_fwd, m_tr = _lib.strides3((mb_, mi, mj)), _lib.strides3((mb_, mj, mi))
+    a = torch.zeros(B, CH, Np, Np, dtype=bf, device=dev)
+    b = torch.zeros_like(a)
+    x = torch.zeros_like(a)
+    q = torch.zeros(B, N, H, Np, D, dtype=bf, device=dev)
+    k = torch.zeros_like(q)
+    vt = torch.zeros(B, N, H, D, Np, dtype=bf, device=dev)
+    tb = torch.zeros(B, H, N, Np, device=dev)
+    mb = torch.zeros(B, N, Np, device=dev)
+    o = torch.zeros(B, N, N, H * D, dtype=bf, device=dev)
+    P = lambda t: t.data_ptr()  # noqa: E731
+
+    def ck(st):
+        _lib.check(st, "bench stage")
+
+    def trimul(prefix, outgoing):
+        w = lambda name: P(dp[prefix + name])  # noqa: E731
+        return [
+            ("trimul_proj", lambda: ck(lib.of3_trimul_proj(
+                P(zz), z_fwd, P(mask), m_fwd, w("layer_norm_in.weight"), w("layer_norm_in.bias"),
+                w("linear_a_p.weight"), w("linear_a_g.weight"), w("linear_b_p.weight"), w("linear_b_g.weight"),
+                P(a), P(b), B, N, C, CH, outgoing, s))),
+            ("trimul_contract", lambda: ck(lib.of3_trimul_contract(P(a), P(b), P(x), B, N, CH, contract_variant, s))),
+            ("trimul_out", lambda: ck(lib.of3_trimul_out(
+                P(x), P(zz), z_fwd, P(zz), w("layer_norm_in.weight"), w("layer_norm_in.bias"),
+                w("layer_norm_out.weight"), w("layer_norm_out.bias"), w("linear_g.weight"), w("linear_z.weight"),
+                B, N, C, CH, 1, s))),
+        ]
+
+    def triattn(prefix, zs, ms_):
+        w = lambda name: P(dp[prefix + name])  # noqa: E731
+        return [
+            ("triattn_proj", lambda: ck(lib.of3_triattn_proj(
+                P(zz), zs, P(mask), ms_, w("layer_norm.weight"), w("layer_norm.bias"), w("mha.linear_q.weight"),
+                w("mha.linear_k.weight"), w("mha.linear_v.weight"), w("linear_z.weight"),
+                P(q), P(k), P(vt), P(tb), P(mb), B, N, C, H, D, 1e9, s))),
+            ("triattn_flash", lambda: ck(lib.of3_triattn_flash(P(q), P(k), P(vt), P(tb), P(mb), P(o), B, N, H, D, s))),
+            ("triattn_out", lambda: ck(lib.of3_triattn_out(
+                P(o), P(zz), zs, P(zz), w("layer_norm.weight"), w("layer_norm.bias"), w("mha.linear_g.weight"),
+                w("mha.linear_o.weight"), B, N, C, H, D, 1, s))),
+        ]
+
+    stage_list = (trimul("tri_mul_out.", 1) + trimul("tri_mul_in.", 0)
+                  + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr))
+    return stage_list, (a, b, x, q, k, vt, tb, mb, o, z_fwd, z_tr, m_fwd, m_tr)
+
+
+def time_launches(torch, launches, steps, warmup):
+    """Every launch bracketed by its own pair of events on the launch stream: {name: [ms per launch]}."""
+    for _ in range(max(warmup, 1)):
+        for _, fn in launches:
+            fn()
+    torch.cuda.synchronize()
+    marks = []
+    for _ in range(steps):
+        for name, fn in launches:
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            marks.append((name, e0, e1))
+    torch.cuda.synchronize()
+    durations = {}
+    for name, e0, e1 in marks:
+        durations.setdefault(name, []).append(e0.elapsed_time(e1))
+    return durations
+
+
+def kernel_figures(durations, model):
+    """Mean launch duration of every kernel against the roof that bounds it."""
+    kernels = {}
+    for name, vals in durations.items():
+        ms = sum(vals) / len(vals)
+        m = model[name]
+        if m["bound"] == "mfma":
+            ach = m["flops"] / (ms * 1e-3) / 1e12
+            kernels[name] = {"bound": "mfma", "ms": round(ms, 4), "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
+                             "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4)}
+        else:
+            ach = m["bytes"] / (ms * 1e-3) / 1e9
+            kernels[name] = {"bound": "hbm", "ms": round(ms, 4), "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
+                             "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4)}
+    return kernels
+
+
+def other_configs(of3pair, lib, _lib, orc, torch, dev, which):
+    """The benchmark's configurations 2, 4 and 5 (configuration 3 is `value`; configuration 1 is the CPU
+    plumbing case): wall clock through the module interface and the block's six kernels one by one, each
+    against its roof.  Not part of `value`.
+
+      2  one pair-stack block, B = 1, N = 384, c_z = 128, the last 10 % of the tokens masked
+      4  the template pair stack: 2 TemplatePairBlocks (pair stack + transition n = 2) over 4 templates,
+         N = 512, c_t = 64, 4 heads x 16, per-template padding of 0-20 %
+      5  4 stacked pair-stack blocks in place at N = 2048, c_z = 128, the last 256 tokens masked
+    """
+    bf = torch.bfloat16
+    out = {}
+
+    def wall(fn, reps, warm):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / reps
+
+    def stage_figures(params, zz, mask, dims, reps, warm):
+        dp = {k_: v.to(dev).to(bf).contiguous() for k_, v in params.items()}
+        stage_list, keep = block_stage_launches(lib, _lib, torch, dp, zz, mask, dims)
+        fig = kernel_figures(time_launches(torch, stage_list, reps, warm), kernel_model(*dims))
+        del stage_list, keep
+        return fig
+
+    if 2 in which:
+        B, N, C, CH, H, D = dims = (1, 384, 128, 128, 4, 32)
+        params = {k_: orc.round_bf16(v) for k_, v in orc.make_block_params(0, C, CH, D, H).items()}
+        blk = of3pair.PairStack(C, CH, D, H)
+        blk.load_state_dict(params)
+        blk = blk.to(dev).to(bf).eval()
+        z = orc.round_bf16(orc.make_pair_input(2, (B,), N, C)).to(dev).to(bf)
+        mask = orc.tail_padding_mask((B,), N, N // 10).to(dev)
+        ms = wall(lambda: blk(z, mask), 30, 10)
+        out["2"] = {"workload": "pair-stack block, B=1, N_token=384, c_z=128, last 10% of tokens masked",
+                    "blocks": 1, "ms": round(ms, 4), "ms_per_block": round(ms, 4),
+                    "kernels": stage_figures(params, z.clone(), mask, dims, 20, 5)}
+        del blk, z, mask
+    if 4 in which:
+        B, N, C, CH, H, D = dims = (4, 512, 64, 64, 4, 16)
+        gen = torch.Generator().manual_seed(3)
+        sd, first = {}, None
+        for i in range(2):
+            bp = dict(orc.make_block_params(30 + i, C, CH, D, H))
+            bp.update({"pair_transition." + k_: v for k_, v in orc.make_transition_params(gen, C, 2).items()})
+            bp = {k_: orc.round_bf16(v) for k_, v in bp.items()}
+            first = first or bp
+            sd.update({"blocks.%d.%s" % (i, k_): v for k_, v in bp.items()})
+        sd["layer_norm.weight"], sd["layer_norm.bias"] = torch.ones(C), torch.zeros(C)
+        stack = of3pair.TemplatePairStack(c_t=C, c_hidden_tri_att=D, c_hidden_tri_mul=CH, no_blocks=2, no_heads=H,
+                                          pair_transition_n=2, dropout_rate=0.25, tri_mul_first=True)
+        stack.load_state_dict(sd, strict=True)
+        stack = stack.to(dev).to(bf).eval()
+        t = orc.round_bf16(orc.make_pair_input(3, (B,), N, C)).to(dev).to(bf)
+        mask = orc.tail_padding_mask((B,), N, torch.tensor([0, 20, 51, 102])).to(dev)
+        ms = wall(lambda: stack.run_blocks(t, mask), 10, 3)
+        out["4"] = {"workload": "template pair stack: 2 blocks (pair stack + transition n=2), 4 templates, N_token=512, "
+                                "c_t=64, c_hidden_mul=64, 4 heads x 16, per-template padding 0-20%",
+                    "blocks": 2, "ms": round(ms, 4), "ms_per_block": round(ms / 2, 4),
+                    "kernels": stage_figures(first, t.clone(), mask, dims, 10, 3)}
+        del stack, t, mask
+    if 5 in which:
+        B, N, C, CH, H, D = dims = (1, 2048, 128, 128, 4, 32)
+        blocks, params = [], None
+        for i in range(4):
+            params = {k_: orc.round_bf16(v) for k_, v in orc.make_block_params(50 + i, C, CH, D, H).items()}
+            blk = of3pair.PairStack(C, CH, D, H)
+            blk.load_state_dict(params)
+            blocks.append(blk.to(dev).to(bf).eval())
+        z0 = torch.randn(B, N, N, C, generator=torch.Generator().manual_seed(5)).to(bf).to(dev)
+        mask = orc.tail_padding_mask((B,), N, 256).to(dev)
+        zw = torch.empty_like(z0)
+
+        def four_blocks():
+            zw.copy_(z0)  # the stack runs in place on a fresh copy (a 1 GB device copy, counted: ~0.4 ms of ~100)
+            zz = zw
+            for blk_ in blocks:
+                zz = blk_(zz, mask, inplace_safe=True)
+
+        ms = wall(four_blocks, 3, 1)
+        del blocks
+        from of3pair import functional as F3
+        F3.release_workspaces()
+        torch.cuda.empty_cache()
+        fig = stage_figures(params, zw, mask, dims, 3, 1)
+        out["5"] = {"workload": "4 stacked pair-stack blocks in place, B=1, N_token=2048, c_z=128, last 256 tokens "
+                                "masked (~1 GB pair representation)",
+                    "blocks": 4, "ms": round(ms, 3), "ms_per_block": round(ms / 4, 3), "kernels": fig}
+        del z0, zw, mask
+    torch.cuda.empty_cache()
+    return out
 
 
 def extra_legs(of3pair, orc, pf, s_pf, z32, sm, m32, fp32_reps, dev):
@@ -155,6 +356,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the fp32 PairFormerBlock and the template-block legs (profiles of the headline workload)")
     ap.add_argument("--contract-variant", type=int, default=0)
+    ap.add_argument("--configs", default="2,4,5",
+                    help="which of the other benchmark configurations (2, 4, 5) to time as well; '' for none")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build is single-GPU (one pair-stack block on one MI355X); run with --gpus 1")
@@ -232,55 +435,15 @@ def main():
     # the caches by its producer, clocks as in the block) and not in a back-to-back loop
     lib = _lib.load()
     s = torch.cuda.current_stream().cuda_stream
-    Np = lib.of3_padded_n(N)
     bf = torch.bfloat16
     zz = z_host.to(dev).to(bf)
-    sb, si, sj = zz.stride()[:3]
-    z_fwd, z_tr = _lib.strides3((sb, si, sj)), _lib.strides3((sb, sj, si))
-    mb_, mi, mj = mask.stride()
-    m_fwd, m_tr = _lib.strides3((mb_, mi, mj)), _lib.strides3((mb_, mj, mi))
     dp = {k: v.to(dev).to(bf).contiguous() for k, v in params.items()}
-    a = torch.zeros(B, CH, Np, Np, dtype=bf, device=dev)
-    b = torch.zeros_like(a)
-    x = torch.zeros_like(a)
-    q = torch.zeros(B, N, H, Np, D, dtype=bf, device=dev)
-    k = torch.zeros_like(q)
-    vt = torch.zeros(B, N, H, D, Np, dtype=bf, device=dev)
-    tb = torch.zeros(B, H, N, Np, device=dev)
-    mb = torch.zeros(B, N, Np, device=dev)
-    o = torch.zeros(B, N, N, H * D, dtype=bf, device=dev)
+    block_launches, keep = block_stage_launches(lib, _lib, torch, dp, zz, mask, (B, N, C, CH, H, D), args.contract_variant)
+    z_fwd, m_fwd = keep[-4], keep[-2]
     P = lambda t: t.data_ptr()  # noqa: E731
 
     def ck(st):
         _lib.check(st, "bench stage")
-
-    def trimul(prefix, outgoing):
-        w = lambda name: P(dp[prefix + name])  # noqa: E731
-        return [
-            ("trimul_proj", lambda: ck(lib.of3_trimul_proj(
-                P(zz), z_fwd, P(mask), m_fwd, w("layer_norm_in.weight"), w("layer_norm_in.bias"),
-                w("linear_a_p.weight"), w("linear_a_g.weight"), w("linear_b_p.weight"), w("linear_b_g.weight"),
-                P(a), P(b), B, N, C, CH, outgoing, s))),
-            ("trimul_contract", lambda: ck(lib.of3_trimul_contract(P(a), P(b), P(x), B, N, CH,
-                                                                    args.contract_variant, s))),
-            ("trimul_out", lambda: ck(lib.of3_trimul_out(
-                P(x), P(zz), z_fwd, P(zz), w("layer_norm_in.weight"), w("layer_norm_in.bias"),
-                w("layer_norm_out.weight"), w("layer_norm_out.bias"), w("linear_g.weight"), w("linear_z.weight"),
-                B, N, C, CH, 1, s))),
-        ]
-
-    def triattn(prefix, zs, ms_):
-        w = lambda name: P(dp[prefix + name])  # noqa: E731
-        return [
-            ("triattn_proj", lambda: ck(lib.of3_triattn_proj(
-                P(zz), zs, P(mask), ms_, w("layer_norm.weight"), w("layer_norm.bias"), w("mha.linear_q.weight"),
-                w("mha.linear_k.weight"), w("mha.linear_v.weight"), w("linear_z.weight"),
-                P(q), P(k), P(vt), P(tb), P(mb), B, N, C, H, D, 1e9, s))),
-            ("triattn_flash", lambda: ck(lib.of3_triattn_flash(P(q), P(k), P(vt), P(tb), P(mb), P(o), B, N, H, D, s))),
-            ("triattn_out", lambda: ck(lib.of3_triattn_out(
-                P(o), P(zz), zs, P(zz), w("layer_norm.weight"), w("layer_norm.bias"), w("mha.linear_g.weight"),
-                w("mha.linear_o.weight"), B, N, C, H, D, 1, s))),
-        ]
 
     tgen = torch.Generator().manual_seed(7)
     tp = {k_: v.to(dev).to(bf).contiguous() for k_, v in orc.make_transition_params(tgen, C, TRANSITION_N).items()}
@@ -317,39 +480,9 @@ def main():
         P(s_in), None, P(stp["layer_norm.weight"]), P(stp["layer_norm.bias"]), P(stp["swiglu.linear_a.weight"]),
         P(stp["swiglu.linear_b.weight"]), P(stp["linear_out.weight"]), P(s_out), B * N, C_S, TRANSITION_N * C_S, 0,
         P(st_ws), st_ws.numel(), _lib.OF3_DTYPE_BF16, s)))]
-    launches = (trimul("tri_mul_out.", 1) + trimul("tri_mul_in.", 0)
-                + triattn("tri_att_start.", z_fwd, m_fwd) + triattn("tri_att_end.", z_tr, m_tr) + transition
-                + pair_bias + attn_pair_bias + single_transition + template_tail)
-    for _ in range(max(args.warmup, 1)):
-        for _, fn in launches:
-            fn()
-    torch.cuda.synchronize()
-    marks = []
-    for _ in range(args.steps):
-        for name, fn in launches:
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
-            e0.record()
-            fn()
-            e1.record()
-            marks.append((name, e0, e1))
-    torch.cuda.synchronize()
-    durations = {}
-    for name, e0, e1 in marks:
-        durations.setdefault(name, []).append(e0.elapsed_time(e1))
-    model = kernel_model(B, N, C, CH, H, D)
-    kernels = {}
-    for name, vals in durations.items():
-        ms = sum(vals) / len(vals)
-        m = model[name]
-        if m["bound"] == "mfma":
-            ach = m["flops"] / (ms * 1e-3) / 1e12
-            kernels[name] = {"bound": "mfma", "ms": round(ms, 4), "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS,
-                             "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4)}
-        else:
-            ach = m["bytes"] / (ms * 1e-3) / 1e9
-            kernels[name] = {"bound": "hbm", "ms": round(ms, 4), "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
-                             "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4)}
+    launches = (block_launches + transition + pair_bias + attn_pair_bias + single_transition + template_tail)
+    durations = time_launches(torch, launches, args.steps, args.warmup)
+    kernels = kernel_figures(durations, kernel_model(B, N, C, CH, H, D))
     dom = kernels["trimul_contract"]
     roofline = {"kernel": "trimul_contract", "bound": "mfma", "achieved": dom["achieved"], "peak": PEAK_BF16_TFLOPS,
                 "unit": "TFLOP/s", "frac": dom["frac"],
@@ -390,6 +523,10 @@ def main():
     fp32_pairformer_block_ms, template_block_ms = None, None
     if not args.no_extras:
         fp32_pairformer_block_ms, template_block_ms = extra_legs(of3pair, orc, pf, s_pf, z32, sm, m32, fp32_reps, dev)
+    del pf, ps32, z32, m32, launches, block_launches, keep
+    torch.cuda.empty_cache()
+    which = [int(c) for c in args.configs.split(",") if c]
+    configs = other_configs(of3pair, lib, _lib, orc, torch, dev, which) if which else None
 
     # ---- CPU baseline: the oracle on the host cores, one block of the same workload; one warm-up
     # run (thread pool, allocator), then the median of three
@@ -429,7 +566,7 @@ def main():
         "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
         "pairformer_block_ms": round(pairformer_block_ms, 4), "fp32_block_ms": round(fp32_block_ms, 3),
         "fp32_pairformer_block_ms": None if fp32_pairformer_block_ms is None else round(fp32_pairformer_block_ms, 3),
-        "template_block_ms": template_block_ms,
+        "template_block_ms": template_block_ms, "configs": configs,
     }
     print(json.dumps(line))
 

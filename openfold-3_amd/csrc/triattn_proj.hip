@@ -16,6 +16,13 @@
 #include "of3_kernels.h"
 #include "of3_launch.h"
 
+// Waves per work-group of the C = 128 kernel: 8 (two per SIMD, 248 registers) or 16 (four per SIMD,
+// 118 registers, one matrix per wave).  Measured at N = 768 inside the block: 126 us against 128 us,
+// stand-alone 150 against 158: more waves in flight do not help this pass, the shipped form is 8.
+#ifndef OF3_TP_WAVES
+#define OF3_TP_WAVES 8
+#endif
+
 namespace of3 {
 
 namespace {
@@ -30,24 +37,27 @@ __device__ __forceinline__ int proj_slot(int pos, int chunk) {
   return pos * NCH + (chunk ^ key);
 }
 
-template <int C, int D>
-__global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, int tiles_per_row, int total_tiles) {
+template <int C, int D, int NW>
+__global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p, int tiles_per_row, int total_tiles) {
   constexpr int H = 4;
   constexpr int HD = H * D;
   constexpr int NCH = C / 8;
   constexpr int LPP = NCH;
   constexpr int PPI = 64 / LPP;
   constexpr int TP = 128;
-  constexpr int NW = 8;                // waves per work-group
   constexpr int LN_ITERS = (TP / NW) / PPI;
   constexpr int KS = C / 16;
   constexpr int NT = HD / 32;          // 32-row output tiles per matrix (4 or 2)
   constexpr bool WIDE = (NT == 4);
-  // WIDE (H*D = 128): waves 0..3 own output tile w of q and of k, waves 4..7 own tile w-4 of
-  //   v plus the bias of position tile w-4; waves w and w+4 share a SIMD, so every SIMD
+  constexpr bool W16 = (NW == 16);
+  // WIDE (H*D = 128), 8 waves: waves 0..3 own output tile w of q and of k, waves 4..7 own tile
+  //   w-4 of v plus the bias of position tile w-4; waves w and w+4 share a SIMD, so every SIMD
   //   carries the same MFMA load.
+  // WIDE, 16 waves (four per SIMD at 128 registers): waves 0..3 own tile w of q, 4..7 of k, 8..11
+  //   of v, 12..15 the bias of position tile w-12; waves w, w+4, w+8, w+12 share a SIMD.
   // else (H*D = 64): waves 0..5 own one (matrix, tile) job, waves 6 and 7 do the bias of two
   //   position tiles each.
+  static_assert(!W16 || WIDE, "the sixteen-wave form is built for H*D = 128");
   constexpr int TPW = 4;               // every wave visits all four position tiles
   static_assert(NT == 4 || NT == 2, "H*D must be 128 or 64");
 
@@ -115,9 +125,9 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
   // depends on a branch).
   auto run = [&](auto role_tag) {
     constexpr int ROLE = decltype(role_tag)::value;
-    constexpr int NJ = (ROLE == 0 && WIDE) ? 2 : (ROLE == 2 ? 0 : 1);
+    constexpr int NJ = (ROLE == 0 && WIDE && !W16) ? 2 : (ROLE == 2 ? 0 : 1);
     const int ot = WIDE ? wave % 4 : wave % 2;
-    const int m0 = ROLE == 1 ? 2 : (WIDE ? 0 : wave / 2);  // matrix of job 0: 0 q, 1 k, 2 v
+    const int m0 = ROLE == 1 ? 2 : (WIDE ? (W16 ? wave / 4 : 0) : wave / 2);  // matrix of job 0: 0 q, 1 k, 2 v
 
     u32x4_t wj[NJ > 0 ? NJ : 1][KS];
 #pragma unroll
@@ -166,8 +176,12 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
         }
       };
       if (ROLE == 2) {
-        bias_tile(2 * (wave - 6));
-        bias_tile(2 * (wave - 6) + 1);
+        if (W16) {
+          bias_tile(wave - 12);
+        } else {
+          bias_tile(2 * (wave - 6));
+          bias_tile(2 * (wave - 6) + 1);
+        }
         return;
       }
 #pragma unroll
@@ -215,7 +229,7 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
           *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
         }
       }
-      if (ROLE == 1 && WIDE) bias_tile(wave - 4);
+      if (ROLE == 1 && WIDE && !W16) bias_tile(wave - 4);
     };
 
     int tile_id = blockIdx.x;
@@ -229,7 +243,11 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
     for (; tile_id < total_tiles; tile_id += gridDim.x, buf ^= 1) do_tile(tile_id, buf);
   };
 
-  if (WIDE) {
+  if (W16) {
+    if (wave < 8) run(std::integral_constant<int, 0>{});
+    else if (wave < 12) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, 2>{});
+  } else if (WIDE) {
     if (wave < 4) run(std::integral_constant<int, 0>{});
     else run(std::integral_constant<int, 1>{});
   } else {
@@ -239,17 +257,17 @@ __global__ __launch_bounds__(512) void triattn_proj_kernel(TriattnProjArgs p, in
   }
 }
 
-template <int C, int D>
+template <int C, int D, int NW>
 hipError_t launch(const TriattnProjArgs& a, hipStream_t stream) {
-  auto kern = triattn_proj_kernel<C, D>;
+  auto kern = triattn_proj_kernel<C, D, NW>;
   static int cache[kMaxDevices];
   int grid_cap = 0;
-  hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 512, dev, v); }, &grid_cap);
+  hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 64 * NW, dev, v); }, &grid_cap);
   if (e != hipSuccess) return e;
   const int tiles_per_row = a.Jp / 128;
   const long total = (long)a.B * a.N * tiles_per_row;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, tiles_per_row, (int)total);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), 0, stream, a, tiles_per_row, (int)total);
   return hipGetLastError();
 }
 
@@ -257,8 +275,8 @@ hipError_t launch(const TriattnProjArgs& a, hipStream_t stream) {
 
 hipError_t triattn_proj_launch(const TriattnProjArgs& args, int C, int D, hipStream_t stream) {
   if (args.H != 4) return hipErrorInvalidValue;
-  if (C == 128 && D == 32) return launch<128, 32>(args, stream);
-  if (C == 64 && D == 16) return launch<64, 16>(args, stream);
+  if (C == 128 && D == 32) return launch<128, 32, OF3_TP_WAVES>(args, stream);
+  if (C == 64 && D == 16) return launch<64, 16, 8>(args, stream);
   return hipErrorInvalidValue;
 }
 

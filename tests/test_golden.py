@@ -59,7 +59,7 @@ def test_gpu_trimul_reproduces_fixture(fx, outgoing):
     cls = of3pair.TriangleMultiplicationOutgoing if outgoing else of3pair.TriangleMultiplicationIncoming
     m = cls(c, ch)
     m.load_state_dict(tm)
-    m = m.to("cuda", torch.bfloat16)
+    m = m.to("cuda", torch.bfloat16).eval()
     got = m(z.to("cuda", torch.bfloat16)[None], mask=mask.cuda()[None])[0].float().cpu().numpy()
     _bound(got, d["trimul_outgoing" if outgoing else "trimul_incoming"])
 
@@ -73,6 +73,6 @@ def test_gpu_triattn_reproduces_fixture(fx, starting):
     _, c, _, heads, hd = (int(v) for v in d["dims"])
     m = of3pair.TriangleAttention(c, hd, heads, starting=starting)
     m.load_state_dict(ta)
-    m = m.to("cuda", torch.bfloat16)
+    m = m.to("cuda", torch.bfloat16).eval()
     got = m(z.to("cuda", torch.bfloat16)[None], mask=mask.cuda()[None])[0].float().cpu().numpy()
     _bound(got, d["triattn_starting" if starting else "triattn_ending"])

@@ -100,7 +100,7 @@ def test_attention_pair_bias_rejects_unsupported():
     lib()
     with pytest.raises(ValueError):
         of3pair.AttentionPairBias(384, 384, 384, 384, 128, 24, 16, use_ada_layer_norm=True)
-    m2 = of3pair.AttentionPairBias(768, 768, 768, 768, C_Z, 48, 16).to(DEV)  # c_s beyond the fp32 kernels
+    m2 = of3pair.AttentionPairBias(768, 768, 768, 768, C_Z, 48, 16).to(DEV).eval()  # c_s beyond the fp32 kernels
     with pytest.raises(ValueError):
         m2(torch.zeros(8, 768, device=DEV), torch.zeros(8, 8, C_Z, device=DEV))
     with pytest.raises(ValueError):  # ... in bf16 too: there is no fp32 kernel to fall back to
