@@ -32,6 +32,14 @@
 //    32) carry -inf, and a fully masked row degenerates to a uniform average over all real
 //    keys exactly as the reference's does (-1e9 absorbs the logits in fp32).  A key tile whose
 //    32 mask biases are all zero (checked wave-wide once per tile) skips that k-step.
+//  * padding costs no arithmetic in the first pass: a key tile whose 32 keys are all masked or padded
+//    contributes exp2(-1.44e9 + logit) = 0 exactly to every sum, so the wave leaves that tile out (its
+//    loads and barriers go on).  A row without any unmasked key (a padded token) thereby sits the first
+//    pass out, ends it with the row sum 0 and takes the pass with running maxima, which gives the
+//    reference's uniform average (padded tokens come in runs, so the four rows of a work-group mostly
+//    agree and few other rows are dragged into a second pass).
+//  * head width 16 leaves rows 16..31 of the V^T operand free: row 16 holds ones, so the PV product
+//    itself accumulates the row sum (of the bf16 weights it multiplies) and the 16 additions per tile go.
 #include "of3_device.h"
 #include "of3_kernels.h"
 #include "of3_launch.h"
@@ -58,6 +66,7 @@ __device__ __forceinline__ int key2(int row) { return (row >> 4) & 1; }  // 2 ch
 constexpr int kRows = 4, kRQ = 2, kWaves = 8, kStages = 2;
 constexpr float kRaise = 64.0f;  // the offset of a query is raised only when a logit exceeds it by 2^64 ...
 constexpr float kSnap = 32.0f;   // ... and an offset within +-32 is replaced by 0
+constexpr float kMaskedBelow = -1e8f;  // a mask bias below this sends exp2 of any sane logit to exactly 0
 
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
@@ -210,6 +219,10 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
   auto tile = [&](auto track, int buf, float mb_cur) {
     constexpr bool kTrack = decltype(track)::value;
     if (!wave_has_work) return;
+    // first pass: a tile whose keys are all masked or padded adds exp2(-1.44e9 + logit) = 0 exactly to
+    // every sum and is left out (a row without any unmasked key thus does nothing here, ends with the
+    // row sum 0 and takes the second pass, as it has to anyway)
+    if (!kTrack && __builtin_amdgcn_ballot_w64(mb_cur > kMaskedBelow) == 0) return;
     const bool has_mb = __builtin_amdgcn_ballot_w64(mb_cur != 0.f) != 0;
     const u32x4_t* tbuf = tb_lds + buf * TBS + tb_row;
     const u32x4_t* kvb = kv_row + buf * KVS;
@@ -219,7 +232,9 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) {
       const u32x4_t v = kvb[v_rd[s2]];
-      const u32x4_t z = {0u, 0u, 0u, 0u};
+      // head width 16: rows 16..31 of the operand are free; row 16 is ones (the row sum), the rest zeros
+      const uint32_t fill = (krow == 16) ? 0x3F803F80u : 0u;
+      const u32x4_t z = {fill, fill, fill, fill};
       vc[s2] = (D == 32 || vvalid) ? v : z;
     }
 #pragma unroll
@@ -266,16 +281,20 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const float e0 = fast_exp2(s[2 * w]), e1 = fast_exp2(s[2 * w + 1]);
-        rs += e0;
-        rs += e1;
+        if (D == 32) {
+          rs += e0;
+          rs += e1;
+        }
         pop0[w] = pack_bf16(e0, e1);
       }
       oacc[rq] = mfma_32x32x16(vc[0], pop0, oacc[rq]);
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const float e0 = fast_exp2(s[8 + 2 * w]), e1 = fast_exp2(s[8 + 2 * w + 1]);
-        rs += e0;
-        rs += e1;
+        if (D == 32) {
+          rs += e0;
+          rs += e1;
+        }
         pop1[w] = pack_bf16(e0, e1);
       }
       oacc[rq] = mfma_32x32x16(vc[1], pop1, oacc[rq]);
@@ -310,7 +329,15 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
     }
     wait_vmcnt<0>();  // the loads issued past the end must not outlive the pass (or the work-group's LDS)
 #pragma unroll
-    for (int rq = 0; rq < kRQ; ++rq) l_tot[rq] = l_run[rq] + xhalf(l_run[rq]);
+    for (int rq = 0; rq < kRQ; ++rq) {
+      if (D == 32) {
+        l_tot[rq] = l_run[rq] + xhalf(l_run[rq]);
+      } else {
+        // V^T row 16 (ones) is result row 16: register 0 of the upper lane half, same query column
+        const float mine = oacc[rq][0], other = xhalf(mine);
+        l_tot[rq] = lh ? mine : other;
+      }
+    }
   };
 
   // First pass: offset 0 for every query, no running maximum.  It is exact whenever a query's

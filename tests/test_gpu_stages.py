@@ -283,6 +283,57 @@ def test_triattn_flash_random_shapes(seed):
     report("flash o (random shapes)", o, want, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("D,n,B,pads", [(32, 200, 2, "tail"), (16, 200, 2, "tail"), (32, 160, 1, "head"),
+                                        (16, 97, 1, "middle"), (32, 300, 1, "outer")])
+def test_triattn_flash_padding_masks(D, n, B, pads):
+    """Block-shaped masks as padding produces them: runs of 32 and more masked keys (key tiles the
+    kernel leaves out for rows that have an unmasked key) and rows whose keys are all masked (padded
+    tokens: the reference's -1e9 absorbs the logits and the row becomes a uniform average; the kernel
+    gets there in its first pass with the row's mask bias as the offset)."""
+    L = lib()
+    H = 4
+    gen = _gen(911 + n + D)
+    np_ = L.of3_padded_n(n)
+    q = bf(_randn(gen, B, n, H, np_, D))
+    k = bf(_randn(gen, B, n, H, np_, D))
+    vt = bf(_randn(gen, B, n, H, D, np_))
+    tb = _randn(gen, B, H, n, np_).contiguous()
+    tok = torch.ones(B, n)
+    if pads == "tail":
+        tok[0, n - 70:] = 0
+        if B > 1:
+            tok[1, n - 33:] = 0
+    elif pads == "head":
+        tok[:, :45] = 0
+    elif pads == "middle":
+        tok[:, 20:60] = 0
+    mask = (tok[:, :, None] * tok[:, None, :]).to(DEV)  # outer product: padded rows have no unmasked key
+    if pads == "outer":  # keys masked in long runs for some rows only, every row keeps a key
+        mask = torch.ones(B, n, n, device=DEV)
+        mask[:, ::3, 64:200] = 0
+        mask[:, 1::3, :96] = 0
+    mb = torch.full((B, n, np_), float("-inf"), device=DEV)
+    mb[..., :n] = LOG2E * 1e9 * (mask - 1)
+    o = torch.full((B, n, n, H * D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    print("triattn_flash padding", D, n, B, pads, flush=True)
+    vtp = _to_panels(vt)
+    st = L.of3_triattn_flash(q.data_ptr(), k.data_ptr(), vtp.data_ptr(), tb.data_ptr(), mb.data_ptr(), o.data_ptr(),
+                             B, n, H, D, stream())
+    assert st == 0, L.of3_status_string(st)
+    torch.cuda.synchronize()
+    qf, kf, vf = q[:, :, :, :n].float(), k[:, :, :, :n].float(), vt[..., :n].float()
+    s = torch.einsum("bihqd,bihkd->bihqk", qf, kf)
+    s = (s + mb[:, :, None, None, :n]) + tb[:, None, :, :, :n]
+    p = torch.softmax(s * math.log(2.0), dim=-1)
+    want = torch.einsum("bihqk,bihdk->biqhd", p, vf).reshape(B, n, n, H * D)
+    report("flash o (padding masks)", o, want, atol=2e-2, rtol=2e-2)
+    if pads != "outer":  # a padded row is the plain average of v over all keys, for every query
+        i_pad = int((tok[0] == 0).nonzero()[0])
+        mean_v = vf[0, i_pad].mean(dim=-1)  # [h][d]
+        got = o[0, i_pad].float().reshape(n, H, D)
+        assert (got - mean_v[None]).abs().max() < 2e-2
+
+
 @pytest.mark.parametrize("transposed,add_residual", [(False, 0), (True, 1)])
 @pytest.mark.parametrize("C,D,n,B", [(128, 32, 70, 2), (64, 16, 130, 1)])
 def test_triattn_out(transposed, add_residual, C, D, n, B):
