@@ -1480,8 +1480,10 @@ __global__ __launch_bounds__(kThreads * PT) void triattn_out_x3_f32(TriattnF32 p
 // direct-to-LDS buffer loads, one tile ahead, into double buffers: no registers are held for data in
 // flight, and the only wait is one vmcnt(0) + barrier per key tile, a whole tile of arithmetic after
 // the loads were issued.  The bias slice is XOR-swizzled on the global side (a lane picks which
-// 16-byte chunk it fetches for its fixed LDS slot).  Online softmax; keys past N carry a mask bias
-// of -inf.
+// 16-byte chunk it fetches for its fixed LDS slot).  Softmax as in the bf16 core: a first pass with
+// the offset 0 for every query that leaves out key tiles whose keys are all masked or padded, and a
+// second pass with running maxima for the work-groups whose row sums say the first was not exact;
+// keys past N carry a mask bias of -inf.
 constexpr int kXRows = 4;
 constexpr int kXTbSlots = 128 * 8;                     // bias slice [128 queries][32 keys] fp32 in 16-byte slots
 constexpr int kXKvSlots = 12 * 64;                     // K step 0, 1 (h m l each), then V^T step 0, 1
@@ -1583,20 +1585,18 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
   };
 
   f32x16_t oacc[QT];
-  float m_run[QT], l_run[QT];
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt) {
-    oacc[qt] = zero16();
-    m_run[qt] = -__builtin_inff();
-    l_run[qt] = 0.f;
-  }
+  float m_run[QT], l_run[QT], l_tot[QT];
   const int tb_key = (l32 >> 1) & 7;
 
   // a wave of a row past the end, or whose queries all lie past the end, still takes part in the loads and
   // barriers of its work-group but leaves the arithmetic out; so does a 32-query tile past the end
   const bool wave_has_work = row_valid && q0 < N;
-  auto tile = [&](int buf, float mb) {
+  // track = false: the first pass, offset 0 for every query (no maximum, no rescaling); track = true: running maxima
+  auto tile = [&](auto track, int buf, float mb) {
+    constexpr bool kTrack = decltype(track)::value;
     if (!wave_has_work) return;
+    // first pass: a tile whose keys are all masked or padded adds exp(-1e9 + logit) = 0 exactly to every sum
+    if (!kTrack && __builtin_amdgcn_ballot_w64(mb > -1e8f) == 0) return;
     const bool has_mb = __builtin_amdgcn_ballot_w64(mb != 0.f) != 0;
     const u32x4_t* kvb = kv_row + buf * kXKvSlots + lane;
     const u32x4_t* tbuf = tb_lds + buf * kXTbSlots + (64 * qh + l32) * 8;
@@ -1625,22 +1625,31 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
         s = mfma_32x32x16(kop[st][0], qop[qt][st][1], s);
         s = mfma_32x32x16(kop[st][0], qop[qt][st][0], s);
       }
-      float cmax = s[0];
-#pragma unroll
-      for (int v = 1; v < 16; ++v) cmax = fmaxf(cmax, s[v]);
-      cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));  // the other half of the query's keys
-      const float m_new = fmaxf(m_run[qt], cmax);    // finite: every tile holds a key below N
-      const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_new) * kLog2eF32);
-      m_run[qt] = m_new;
       float lsum = 0.f;
+      if constexpr (kTrack) {
+        float cmax = s[0];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        s[v] = __builtin_amdgcn_exp2f((s[v] - m_new) * kLog2eF32);
-        lsum += s[v];
+        for (int v = 1; v < 16; ++v) cmax = fmaxf(cmax, s[v]);
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));  // the other half of the query's keys
+        const float m_new = fmaxf(m_run[qt], cmax);    // finite: every tile holds a key below N
+        const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_new) * kLog2eF32);
+        m_run[qt] = m_new;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          s[v] = __builtin_amdgcn_exp2f((s[v] - m_new) * kLog2eF32);
+          lsum += s[v];
+        }
+        l_run[qt] = l_run[qt] * alpha + lsum;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[qt][v] *= alpha;
+      } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          s[v] = __builtin_amdgcn_exp2f(s[v] * kLog2eF32);
+          lsum += s[v];
+        }
+        l_run[qt] += lsum;
       }
-      l_run[qt] = l_run[qt] * alpha + lsum;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) oacc[qt][v] *= alpha;
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
         float x[8];
@@ -1659,32 +1668,57 @@ __global__ __launch_bounds__(512) void triattn_core_x3_f32(TriattnF32 p, int n_q
     }
   };
 
-  float mv_next = load_mask(0);
-  issue_loads(0, 0);
-  auto step = [&](int kt, int buf) {  // buf is a constant at both call sites: LDS addresses are immediates
-    wait_vmcnt<0>();               // this wave's loads of tile kt (and its mask values) have landed ...
-    __builtin_amdgcn_s_barrier();  // ... and everybody's; nobody reads tile kt - 1's buffers any more
-    compiler_fence();
-    const float mb = mask_bias(kt, mv_next);
-    const int ktn = kt + 1 < nkt ? kt + 1 : nkt - 1;
-    mv_next = load_mask(ktn);
-    issue_loads(ktn, buf ^ 1);
-    tile(buf, mb);
-    compiler_fence();
+  auto pass = [&](auto track) {
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      oacc[qt] = zero16();
+      m_run[qt] = -__builtin_inff();
+      l_run[qt] = 0.f;
+    }
+    float mv_next = load_mask(0);
+    issue_loads(0, 0);
+    auto step = [&](int kt, int buf) {  // buf is a constant at both call sites: LDS addresses are immediates
+      wait_vmcnt<0>();               // this wave's loads of tile kt (and its mask values) have landed ...
+      __builtin_amdgcn_s_barrier();  // ... and everybody's; nobody reads tile kt - 1's buffers any more
+      compiler_fence();
+      const float mb = mask_bias(kt, mv_next);
+      const int ktn = kt + 1 < nkt ? kt + 1 : nkt - 1;
+      mv_next = load_mask(ktn);
+      issue_loads(ktn, buf ^ 1);
+      tile(track, buf, mb);
+      compiler_fence();
+    };
+    for (int kt = 0; kt < nkt; kt += 2) {
+      step(kt, 0);
+      if (kt + 1 < nkt) step(kt + 1, 1);
+    }
+    wait_vmcnt<0>();  // the loads issued past the end must not outlive the pass (or the work-group's LDS)
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) l_tot[qt] = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
   };
-  for (int kt = 0; kt < nkt; kt += 2) {
-    step(kt, 0);
-    if (kt + 1 < nkt) step(kt + 1, 1);
+
+  // First pass: offset 0 for every query (any common offset gives the same softmax): a logit costs one
+  // multiplication, one exp2 and one addition, no maximum and no rescaling of the accumulator.  It is exact
+  // whenever the exponentials neither overflowed nor lost the row's largest terms, which the row sum tells:
+  // 2^-60 <= sum <= 2^60 (an overflow leaves +inf, a row of masked keys leaves 0).  A work-group with a query
+  // outside that range (its loads and barriers are collective) runs the pass again with running maxima.
+  pass(std::false_type{});
+  {
+    bool bad = false;
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      const bool in_range = l_tot[qt] >= 0x1p-60f && l_tot[qt] <= 0x1p60f;  // false for NaN too
+      bad |= row_valid && (q0 + 32 * qt + l32 < N) && !in_range;
+    }
+    if (__syncthreads_or(bad)) pass(std::true_type{});
   }
-  wait_vmcnt<0>();  // the loads issued past the end must not outlive the work-group's LDS
 
   if (row_valid) {
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
       const int q = q0 + 32 * qt + l32;
-      const float l_tot = l_run[qt] + __shfl_xor(l_run[qt], 32, 64);
       if (q >= N) continue;
-      const float inv = 1.0f / l_tot;
+      const float inv = 1.0f / l_tot[qt];
       float* dst = p.o + ((((size_t)b * N + i) * N + q) * H + h) * D + 4 * lh;
 #pragma unroll
       for (int a = 0; a < D / 8; ++a)  // registers 4 a .. 4 a + 3 are head channels 8 a + 4 lh .. + 3
@@ -2464,8 +2498,9 @@ hipError_t triattn_fwd_f32(const TriattnF32Args& a, hipStream_t stream) {
     if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, true, false>>(kLdsLimit);
     if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, false, true>>(kLdsLimit);
     if (e == hipSuccess) e = allow_lds<triattn_out_x3_f32<kXT, kPT, true, true>>(kLdsLimit);
-    if (e == hipSuccess) e = allow_lds<triattn_core_x3_f32<1>>(kLdsLimit);
-    if (e == hipSuccess) e = allow_lds<triattn_core_x3_f32<2>>(kLdsLimit);
+    // the cores also hold a few static bytes (the work-group vote): ask for what they use, not for the limit
+    if (e == hipSuccess) e = allow_lds<triattn_core_x3_f32<1>>(kCoreX3Lds);
+    if (e == hipSuccess) e = allow_lds<triattn_core_x3_f32<2>>(kCoreX3Lds);
     if (e != hipSuccess) return e;
     const size_t lds = tile_bytes_x3(a.C, 32 * kXT * kPT) + (size_t)a.H * 32 * kXT * kPT * sizeof(float);
     hipLaunchKernelGGL(proj, dim3(xblocks), dim3(kThreads * kPT), lds, stream, p, xgroups);

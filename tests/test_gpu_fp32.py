@@ -77,6 +77,28 @@ def test_triattn_fp32(starting, c, d, heads, n, batch, masked):
     _maxerr("triattn fp32", got, orc.triattn_update(x, mask, p, heads, starting=starting))
 
 
+@pytest.mark.parametrize("d,heads,pads", [(32, 2, 0), (16, 4, 0), (32, 2, 50)])
+def test_triattn_fp32_large_logits_and_padding(d, heads, pads):
+    """Logits far outside the range in which a softmax with the offset 0 is exact (queries whose largest
+    logit lies beyond +-60 in base 2): the work-groups concerned must repeat the pass with running
+    maxima, next to work-groups that never need it; with a padded tail (runs of masked keys the first
+    pass leaves out, padded rows that only the second pass serves)."""
+    lib()
+    c, n = 64, 150
+    gen = torch.Generator().manual_seed(4400 + d + pads)
+    p = orc.make_triattn_params(gen, c, d, heads)
+    p["mha.linear_q.weight"] = p["mha.linear_q.weight"] * 14.0   # q.k / sqrt(d) of +-40 and more
+    p["linear_z.weight"][0] = p["linear_z.weight"][0] * 40.0     # head 0: a triangle bias of +-100
+    x = torch.randn(n, n, c, generator=gen)
+    mask = orc.tail_padding_mask((), n, pads) if pads else (torch.rand(n, n, generator=gen) > 0.2).float()
+    m = _load(of3pair.TriangleAttention(c, d, heads), p)
+    got = m(x.to(DEV), mask=mask.to(DEV))
+    want = orc.triattn_update(x, mask, p, heads)
+    if pads:  # padded rows: -1e9 absorbs moderate logits only, and these are not moderate; compare the real rows
+        got, want = got[: n - pads], want[: n - pads]
+    _maxerr("triattn fp32 large logits", got, want)
+
+
 def test_trimul_fp32_reference_unit_test_shape():
     """The reference's own unit test of the module (test_triangular_multiplicative_update.py:28-52): c_z = 128,
     hidden width 11, batch 2, n_res = 128, uniform inputs and an integer 0/1 mask; here with the values checked."""
