@@ -109,12 +109,26 @@ inline of3::PairView mask_view(const float* mask, const int64_t s[3], bool swap)
 inline const of3::bf16_t* bf(const void* p) { return static_cast<const of3::bf16_t*>(p); }
 inline of3::bf16_t* bf(void* p) { return static_cast<of3::bf16_t*>(p); }
 
+// compute units of the current device (one persistent work-group of the contraction each); 256, the
+// MI355X, when no device can be asked (the shape queries are also answered without a GPU)
+inline int64_t current_cu_count() {
+  static int cache[of3::kMaxDevices];
+  int cus = 0;
+  hipError_t e = of3::per_device(cache, [](int dev, int* v) { return of3::cu_count(dev, v); }, &cus);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // a shape query must not leave an error behind for the next HIP call
+    return 256;
+  }
+  return cus >= 8 ? (cus / 8) * 8 : 8;
+}
+
 inline int contract_variant_auto(int64_t planes, int64_t Np) {
-  // Cheapest of the four output tile shapes for this problem on the 256 CUs of an MI355X:
-  // rounds of persistent work-groups x padded tile area, with a small bonus for the wider
+  // Cheapest of the four output tile shapes for this problem on the device's compute units (256 on
+  // an MI355X): rounds of persistent work-groups x padded tile area, with a small bonus for the wider
   // tiles, which move fewer operand bytes per flop.  (768: 384x192 gives every work-group
   // exactly 4 tiles and every XCD whole planes per round; 512, 1024, 2048: 256x256 divides the
   // plane without waste.)
+  const int64_t cus = current_cu_count();
   const int64_t bm[4] = {256, 256, 256, 384};
   const int64_t bn[4] = {192, 128, 256, 192};
   const double eff[4] = {0.97, 0.90, 1.00, 1.00};
@@ -122,7 +136,7 @@ inline int contract_variant_auto(int64_t planes, int64_t Np) {
   double best_cost = 0;
   for (int v = 0; v < 4; ++v) {
     const int64_t tiles = planes * ((Np + bm[v] - 1) / bm[v]) * ((Np + bn[v] - 1) / bn[v]);
-    const double cost = (double)((tiles + 255) / 256) * (double)(bm[v] * bn[v]) / eff[v];
+    const double cost = (double)((tiles + cus - 1) / cus) * (double)(bm[v] * bn[v]) / eff[v];
     if (v == 0 || cost < best_cost) {
       best = v + 1;
       best_cost = cost;

@@ -46,11 +46,24 @@
 
 #include <type_traits>
 
+// Token count from which the 16-wave form (256 queries per work-group, one work-group per CU) is used.
+// Measured against the 8-wave form (two work-groups per CU): N = 768 395 vs 375 us, N = 2048 7.57 vs
+// 6.95 ms, 4 x 512 with head width 16 474 vs 400 us: the K / V^T loads it saves cost less than the second
+// independent work-group hides, so the default is never.
+#ifndef OF3_FLASH_WIDE_FROM
+#define OF3_FLASH_WIDE_FROM (1 << 30)
+#endif
+
 namespace of3 {
 
 namespace {
 
 __device__ __forceinline__ float xhalf(float v) { return __shfl_xor(v, 32, 64); }
+
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+__device__ __forceinline__ f32x4_t mfma_16x16x32(u32x4_t a, u32x4_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
 
 // swizzle keys of the K / V^T tiles in LDS: rows are read in the order rowperm16(lane), i.e.
 // {x..x+3, x+16..x+19, x+4..x+7, x+20..x+23} per 16 lanes; (row & 1, key) must differ inside
@@ -63,7 +76,7 @@ __device__ __forceinline__ int key2(int row) { return (row >> 4) & 1; }  // 2 ch
 // Every iteration of the tile loop issues the same loads (indices past the end are clamped, their
 // data is never read), so that the compiler can count the loads in flight and its own waits do not
 // drain the ring.
-constexpr int kRows = 4, kRQ = 2, kWaves = 8, kStages = 2;
+constexpr int kRows = 4, kRQ = 2, kStages = 2;
 constexpr float kRaise = 64.0f;  // the offset of a query is raised only when a logit exceeds it by 2^64 ...
 constexpr float kSnap = 32.0f;   // ... and an offset within +-32 is replaced by 0
 constexpr float kMaskedBelow = -1e8f;  // a mask bias below this sends exp2 of any sane logit to exactly 0
@@ -74,9 +87,14 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   return r;
 }
 
-template <int D>
-__global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFlashArgs p, int n_qc, int n_rg,
-                                                                          int total, int per_xcd) {
+// QW = waves per row: 2 (work-group = 8 waves = 4 rows x 128 queries, two work-groups per CU) or 4 (16 waves
+// = 4 rows x 256 queries, one work-group per CU: a row's K and V^T tiles, the loads that miss L2, are brought
+// in for twice as many queries).
+template <int D, int QW>
+__global__ __launch_bounds__(64 * kRows * QW, 4) void triattn_flash_kernel(TriattnFlashArgs p, int n_qc, int n_rg,
+                                                                             int total, int per_xcd) {
+  constexpr int kWaves = kRows * QW;
+  constexpr int QWG = 64 * QW;  // queries per work-group
   constexpr int H = 4;
   constexpr int HD = H * D;
   constexpr int KSQ = D / 16;
@@ -85,9 +103,12 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
   constexpr int VSLOTS = D * 4;
   constexpr int KVS = KSLOTS + VSLOTS;
   constexpr int KI = KSLOTS / 64, VI = VSLOTS / 64;
-  static_assert(KI == VI, "the two waves of a row issue the same number of loads per tile");
-  constexpr int TBS = 128 * 8;  // [128 q][32 k] fp32 in 16-byte slots
-  constexpr int TBI = TBS / 64 / kWaves;  // bias instructions per wave and tile
+  static_assert(KI == VI, "a row's K and V^T tiles take the same number of load instructions");
+  constexpr int KVI = KI + VI;                       // 1-KB load instructions per row and tile: K0, (K1), V0, (V1)
+  constexpr int SPW = KVI / QW > 0 ? KVI / QW : 1;   // of which a wave issues this many (waves beyond KVI: none)
+  constexpr int TBS = QWG * 8;  // [QWG q][32 k] fp32 in 16-byte slots
+  constexpr int TBI = 2;  // bias instructions per wave and tile
+  static_assert(TBI * 64 * kWaves == TBS, "the waves share the bias slice evenly");
   constexpr int LPT = TBI + KI;
 
   extern __shared__ u32x4_t lds[];
@@ -96,7 +117,7 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int row = wave >> 1, qh = wave & 1;
+  const int row = wave / QW, qq = wave % QW;
   const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
   const int N = p.N, Jp = p.Jp;
   const int logical = xcd_logical_block(blockIdx.x, per_xcd);
@@ -108,8 +129,8 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
   const bool row_valid = i_raw < N;  // wave-uniform; idle waves still take part in the loads and barriers
   const int i = row_valid ? i_raw : N - 1;
   const int b = bh / H, h = bh % H;
-  const int qwg = qc * 128;
-  const int q0 = qwg + 64 * qh;
+  const int qwg = qc * QWG;
+  const int q0 = qwg + 64 * qq;
 
   const size_t bih = ((size_t)b * N + i) * H + h;
   const bf16_t* Q = p.q + bih * Jp * D;
@@ -140,36 +161,43 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
     qrow = qrow < N ? qrow : N - 1;
     tb_off[n] = (uint32_t)(((size_t)qrow * Jp + 4 * chunk) * sizeof(float));
   }
-  // the wave's share of its row's stage: the K tile (qh = 0) or the V^T tile (qh = 1)
-  // (with two instructions per tile, the second one's rows are 16 further on, which flips bit 1 of
-  // key4: its offset is (kv_off ^ 32) + 1024)
+  // the wave's share of its row's stage: SPW of the row's KVI load instructions, all of the K tile or all
+  // of the V^T tile (the second instruction of a tile takes rows 16 further on, which flips bit 1 of
+  // key4: its offset is (first ^ 32) + 1024)
   static_assert(KI == 1 || (KI == 2 && QCH == 4), "offset rule of the second instruction");
+  const int slot0 = qq * SPW;               // first instruction slot of this wave
+  const bool has_kv = slot0 < KVI;          // wave-uniform
+  const bool is_v = slot0 >= KI;
+  const int idx0 = is_v ? slot0 - KI : slot0;
   uint32_t kv_off;
-  if (qh == 0) {
+  if (!is_v) {
     const int r = lane / QCH, chunk = (lane % QCH) ^ (QCH == 4 ? key4(r) : key2(r));
     kv_off = (uint32_t)((r * D + 8 * chunk) * sizeof(bf16_t));
   } else {
     const int r = lane >> 2, chunk = (lane & 3) ^ key4(r);
     kv_off = (uint32_t)((r * 32 + 8 * chunk) * sizeof(bf16_t));
   }
+  if (idx0 == 1) kv_off = (kv_off ^ 32u) + 1024u;
   u32x4_t* kv_row = kv_lds + row * (kStages * KVS);
   // Loads go through buffer descriptors (scalar base, 32-bit lane offset, scalar tile offset): the
   // addresses cost one register per stream, and a load beyond its range would return zeros.
   const __amdgpu_buffer_rsrc_t tb_rsrc = buffer_rsrc(tb, (size_t)N * Jp * sizeof(float));
-  const __amdgpu_buffer_rsrc_t kv_rsrc = buffer_rsrc(qh == 0 ? K : Vt, (size_t)Jp * D * sizeof(bf16_t));
+  const __amdgpu_buffer_rsrc_t kv_rsrc = buffer_rsrc(is_v ? Vt : K, (size_t)Jp * D * sizeof(bf16_t));
   const __amdgpu_buffer_rsrc_t mb_rsrc = buffer_rsrc(mb, (size_t)Jp * sizeof(float));
   auto issue_loads = [&](int kt, int buf) {  // buf is a constant at every call site
     u32x4_t* tdst = tb_lds + buf * TBS + 64 * TBI * wave;
-    u32x4_t* kdst = kv_row + buf * KVS + (qh == 0 ? 0 : KSLOTS);
+    u32x4_t* kdst = kv_row + buf * KVS + (is_v ? KSLOTS : 0) + 64 * idx0;
 #pragma unroll
     for (int n = 0; n < TBI; ++n)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(tb_rsrc, (void OF3_LDS_AS*)(tdst + 64 * n), 16, tb_off[n],
                                                kt * (32 * (int)sizeof(float)), 0, 0);
     const int kv_tile = kt * (32 * D * (int)sizeof(bf16_t));
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(kv_rsrc, (void OF3_LDS_AS*)kdst, 16, kv_off, kv_tile, 0, 0);
-    if (KI == 2)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(kv_rsrc, (void OF3_LDS_AS*)(kdst + 64), 16, (kv_off ^ 32u) + 1024u,
-                                               kv_tile, 0, 0);
+    if (has_kv) {  // wave-uniform and the same in every tile: the number of loads per tile stays a constant of the wave
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kv_rsrc, (void OF3_LDS_AS*)kdst, 16, kv_off, kv_tile, 0, 0);
+      if (SPW == 2)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(kv_rsrc, (void OF3_LDS_AS*)(kdst + 64), 16, (kv_off ^ 32u) + 1024u,
+                                                 kv_tile, 0, 0);
+    }
   };
   auto load_mb = [&](int kt, uint32_t lane_off) {
     return __builtin_amdgcn_raw_buffer_load_b32(mb_rsrc, lane_off, kt * (32 * (int)sizeof(float)), 0);
@@ -186,10 +214,20 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
     v_rd[s2] = KSLOTS + vr * 4 + ((2 * lh + s2) ^ key4(vr));
   }
   const int tb_key = (l32 >> 1) & 7;
-  const int tb_row = (2 * qh) * 256 + l32 * 8;
+  const int tb_row = (2 * qq) * 256 + l32 * 8;
 
   float m_run[kRQ], l_run[kRQ], l_tot[kRQ];
   f32x16_t oacc[kRQ];
+  // Head width 32, first pass: the row sums come from the matrix pipe as well.  The weights of a tile sit
+  // in the B-operand registers of the P V product: lane 16 g + n holds 8 keys of query 16 (g % 2) + n.
+  // Read as the B operand of a 16 x 16 x 32 product, lane 16 g + n is column n, k-group g; with an A
+  // operand whose row 0 is ones over the k-groups 0 and 2 and whose row 1 is ones over the k-groups 1 and 3,
+  // row 0 of the result sums query n and row 1 query 16 + n (registers 0 and 1 of lanes 0..15), over the
+  // keys of both lane halves.  Two such products per tile replace sixteen additions on the vector pipe,
+  // which is the busier one; the sums are those of the bf16 weights the P V product multiplies.
+  f32x4_t lsum[kRQ];
+  const uint32_t ones_pat = (lane == 0 || lane == 32 || lane == 17 || lane == 49) ? 0x3F803F80u : 0u;
+  const u32x4_t ones_a = {ones_pat, ones_pat, ones_pat, ones_pat};
 
   // mask-bias k-step on the 8-deep MFMA (two registers per operand): A = [mb[key], 0, 0, 0], B = [1, 0, 0, 0],
   // both built where they are used (few tiles hold a masked or padded key)
@@ -281,23 +319,25 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const float e0 = fast_exp2(s[2 * w]), e1 = fast_exp2(s[2 * w + 1]);
-        if (D == 32) {
+        if (D == 32 && kTrack) {
           rs += e0;
           rs += e1;
         }
         pop0[w] = pack_bf16(e0, e1);
       }
       oacc[rq] = mfma_32x32x16(vc[0], pop0, oacc[rq]);
+      if (D == 32 && !kTrack) lsum[rq] = mfma_16x16x32(ones_a, pop0, lsum[rq]);
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const float e0 = fast_exp2(s[8 + 2 * w]), e1 = fast_exp2(s[8 + 2 * w + 1]);
-        if (D == 32) {
+        if (D == 32 && kTrack) {
           rs += e0;
           rs += e1;
         }
         pop1[w] = pack_bf16(e0, e1);
       }
       oacc[rq] = mfma_32x32x16(vc[1], pop1, oacc[rq]);
+      if (D == 32 && !kTrack) lsum[rq] = mfma_16x16x32(ones_a, pop1, lsum[rq]);
       l_run[rq] = rs;
     }
   };
@@ -309,6 +349,7 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
       m_run[rq] = decltype(track)::value ? -__builtin_inff() : 0.f;
       l_run[rq] = 0.f;
       oacc[rq] = zero16();
+      lsum[rq] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
     float mb_next = __uint_as_float(load_mb(0, mb_off));
     issue_loads(0, 0);
@@ -330,8 +371,11 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
     wait_vmcnt<0>();  // the loads issued past the end must not outlive the pass (or the work-group's LDS)
 #pragma unroll
     for (int rq = 0; rq < kRQ; ++rq) {
-      if (D == 32) {
+      if (D == 32 && decltype(track)::value) {
         l_tot[rq] = l_run[rq] + xhalf(l_run[rq]);
+      } else if (D == 32) {
+        const float lo = __shfl(lsum[rq][0], l32 & 15, 64), hi = __shfl(lsum[rq][1], l32 & 15, 64);
+        l_tot[rq] = (l32 & 16) ? hi : lo;
       } else {
         // V^T row 16 (ones) is result row 16: register 0 of the upper lane half, same query column
         const float mine = oacc[rq][0], other = xhalf(mine);
@@ -376,30 +420,30 @@ __global__ __launch_bounds__(64 * kWaves, 4) void triattn_flash_kernel(TriattnFl
 }
 
 
-template <int D>
+template <int D, int QW>
 constexpr int lds_bytes() {
-  return (kStages * 128 * 8 + kRows * kStages * (32 * (D / 8) + D * 4)) * 16;
+  return (kStages * 64 * QW * 8 + kRows * kStages * (32 * (D / 8) + D * 4)) * 16;
 }
 
-template <int D>
+template <int D, int QW>
 hipError_t launch(const TriattnFlashArgs& a, hipStream_t stream) {
-  auto kern = triattn_flash_kernel<D>;
   static int cache[kMaxDevices];
   int configured = 0;
   hipError_t e = per_device(
       cache,
       [&](int, int* v) {
         *v = 1;
-        return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   lds_bytes<D>());
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(&triattn_flash_kernel<D, QW>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (lds_bytes<D, QW>()));
       },
       &configured);
   if (e != hipSuccess) return e;
-  const int n_qc = (a.N + 127) / 128, n_rg = (a.N + kRows - 1) / kRows;
+  const int n_qc = (a.N + 64 * QW - 1) / (64 * QW), n_rg = (a.N + kRows - 1) / kRows;
   const long total = (long)n_qc * n_rg * a.B * a.H;
   const int per_xcd = (int)((total + 7) / 8);
-  hipLaunchKernelGGL(kern, dim3(per_xcd * 8), dim3(64 * kWaves), lds_bytes<D>(), stream, a, n_qc, n_rg, (int)total,
-                     per_xcd);
+  constexpr int kLds = lds_bytes<D, QW>();
+  triattn_flash_kernel<D, QW><<<dim3(per_xcd * 8), dim3(64 * kRows * QW), kLds, stream>>>(a, n_qc, n_rg, (int)total,
+                                                                                          per_xcd);
   return hipGetLastError();
 }
 
@@ -407,8 +451,9 @@ hipError_t launch(const TriattnFlashArgs& a, hipStream_t stream) {
 
 hipError_t triattn_flash_launch(const TriattnFlashArgs& args, int D, hipStream_t stream) {
   if (args.H != 4) return hipErrorInvalidValue;
-  if (D == 32) return launch<32>(args, stream);
-  if (D == 16) return launch<16>(args, stream);
+  const bool wide = args.N >= OF3_FLASH_WIDE_FROM;
+  if (D == 32) return wide ? launch<32, 4>(args, stream) : launch<32, 2>(args, stream);
+  if (D == 16) return wide ? launch<16, 4>(args, stream) : launch<16, 2>(args, stream);
   return hipErrorInvalidValue;
 }
 

@@ -48,6 +48,12 @@ HIPCC_FLAGS = [
 ]
 
 
+def _flags():
+    """The compiler flags, plus what OF3_HIPCC_EXTRA adds (e.g. -DOF3_FLASH_WIDE_FROM=1 to run the tests on a
+    kernel variant that the default thresholds would not pick at the tests' sizes)."""
+    return HIPCC_FLAGS + os.environ.get("OF3_HIPCC_EXTRA", "").split()
+
+
 def _hipcc() -> str:
     return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -64,7 +70,7 @@ def _run(cmd):
 def source_digest() -> str:
     """sha256 over everything the library is compiled from: the kernel sources and headers, the public
     header and the compiler flags."""
-    h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
+    h = hashlib.sha256(" ".join(_flags()).encode())
     files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".h"))]
     if os.path.isdir(INCLUDE_DIR):
         files += [os.path.join(INCLUDE_DIR, f) for f in sorted(os.listdir(INCLUDE_DIR)) if f.endswith(".h")]
@@ -84,7 +90,7 @@ def build(verbose: bool = False, jobs: int = 4) -> str:
 
     def compile_one(src):
         obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
-        out = _run([_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        out = _run([_hipcc(), *_flags(), "-c", os.path.join(CSRC, src), "-o", obj])
         if verbose and out.strip():
             print(out)
         return obj
