@@ -358,6 +358,9 @@ def main():
     ap.add_argument("--contract-variant", type=int, default=0)
     ap.add_argument("--configs", default="2,4,5",
                     help="which of the other benchmark configurations (2, 4, 5) to time as well; '' for none")
+    ap.add_argument("--configs-only", action="store_true",
+                    help="time only the configurations named by --configs (kernel traces of one configuration); prints "
+                         "their figures, no headline line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build is single-GPU (one pair-stack block on one MI355X); run with --gpus 1")
@@ -376,6 +379,11 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, N, C, CH, H, D = 1, args.n, 128, 128, 4, 32
+
+    if args.configs_only:
+        which = [int(c) for c in args.configs.split(",") if c]
+        print(json.dumps({"configs": other_configs(of3pair, _lib.load(), _lib, orc, torch, dev, which)}))
+        return
 
     params = {k: orc.round_bf16(v) for k, v in orc.make_block_params(0, C, CH, D, H).items()}
     block = of3pair.PairStack(C, CH, D, H)

@@ -54,7 +54,10 @@ def test_trimul_max_abs(dtype, outgoing):
     m = _load(cls(c, c), p, dtype)
     got = m(z.to(DEV).to(dtype), mask=mask.to(DEV))
     want = orc.trimul_update(z, mask, p, outgoing)
-    rec = record_parity("trimul update (reference convention)", got, want, None, "max|err| < 2e-2 (bf16: or the bf16 path's)")
+    rec = record_parity("trimul update (reference convention)", got, want, None,
+                        "max|err| < 2e-2" if dtype == torch.float32 else
+                        "PASSES ON max|err| <= error of the oracle run in bfloat16 (2.8-3.1e-2), NOT on 2e-2; the "
+                        "reference states this test in fp32 only")
     bound = EPS
     if dtype == torch.bfloat16:
         # The reference states this test in fp32 only.  In bf16 the outputs reach |4|, where half a
@@ -138,7 +141,8 @@ def test_template_embedder_max_abs(dtype):
                             tail["template_pair_stack.layer_norm.bias"], 4)
     want = orc.template_tail(tn, tail["linear_t.weight"])
     rec = record_parity("template embedder output (reference convention)", got, want, None,
-                        "max|err| < 2e-2 (bf16: or the bf16 path's)")
+                        "max|err| < 2e-2" if dtype == torch.float32 else
+                        "PASSES ON max|err| <= error of the oracle run in bfloat16 (5.5e-2), NOT on 2e-2")
     bound = EPS
     if dtype == torch.bfloat16:
         # as for the triangle multiplication above: where the reference's own bf16 path (the oracle's
