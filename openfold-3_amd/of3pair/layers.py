@@ -59,6 +59,10 @@ TRI_ATT_INIT = {
 }
 
 
+# the fused-projection form (default_linear_init_config.py:122-129): bias-free as well
+FUSED_TRI_MUL_INIT = {"linear_ab_p": "default", "linear_ab_g": "gating", "linear_g": "gating", "linear_z": "final"}
+
+
 # default_linear_init_config.py:29-34, :157-162
 SWIGLU_TRANSITION_INIT = {"swiglu": {"linear_a": "relu", "linear_b": "relu"}, "linear_out": "final"}
 
@@ -94,6 +98,12 @@ class TriangleMultiplicativeUpdate(nn.Module):
         for name, default in TRI_MUL_INIT.items():
             _init_linear(getattr(self, name), _init_name(linear_init_params, name, default))
 
+    def _weights(self):
+        """The ten tensors of F3.triangle_multiplicative_update, in its order."""
+        return (self.layer_norm_in.weight, self.layer_norm_in.bias, self.layer_norm_out.weight, self.layer_norm_out.bias,
+                self.linear_a_p.weight, self.linear_a_g.weight, self.linear_b_p.weight, self.linear_b_g.weight,
+                self.linear_g.weight, self.linear_z.weight)
+
     @forward_only
     def forward(self, z, mask=None, inplace_safe=False, use_cueq_triangle_kernels=False,
                 _add_with_inplace=False, _inplace_chunk_size=256):
@@ -124,6 +134,55 @@ class TriangleMultiplicationIncoming(TriangleMultiplicativeUpdate):
     """AF3 Algorithm 13."""
 
     __init__ = partialmethod(TriangleMultiplicativeUpdate.__init__, _outgoing=False)
+
+
+class FusedTriangleMultiplicativeUpdate(nn.Module):
+    """The fused-projection form of the triangle multiplication (tmu.py:522-666): linear_ab_p and
+    linear_ab_g hold the a and b projections stacked, [2 * c_hidden, c_z], rows 0 .. c_hidden - 1 being a
+    (tmu.py:578-580, :646-647).  Same arithmetic as the un-fused module, so the same kernels run it: the
+    two halves of each stacked weight are handed over as the a and b matrices (contiguous row slices, no
+    copy).  State-dict keys: layer_norm_in, layer_norm_out, linear_ab_p, linear_ab_g, linear_g, linear_z.
+    Bias-free Linears only, as in the reference's own initialiser table for this module."""
+
+    def __init__(self, c_z, c_hidden, _outgoing=True, linear_init_params=None):
+        super().__init__()
+        self.c_z = c_z
+        self.c_hidden = c_hidden
+        self._outgoing = _outgoing
+        self.linear_g = nn.Linear(c_z, c_z, bias=False)
+        self.linear_z = nn.Linear(c_hidden, c_z, bias=False)
+        self.layer_norm_in = nn.LayerNorm(c_z, eps=1e-5)
+        self.layer_norm_out = nn.LayerNorm(c_hidden, eps=1e-5)
+        self.linear_ab_p = nn.Linear(c_z, 2 * c_hidden, bias=False)
+        self.linear_ab_g = nn.Linear(c_z, 2 * c_hidden, bias=False)
+        for name, default in FUSED_TRI_MUL_INIT.items():
+            _init_linear(getattr(self, name), _init_name(linear_init_params, name, default))
+
+    def _weights(self):
+        """The ten tensors of F3.triangle_multiplicative_update, in its order."""
+        ch = self.c_hidden
+        p, g = self.linear_ab_p.weight, self.linear_ab_g.weight
+        return (self.layer_norm_in.weight, self.layer_norm_in.bias, self.layer_norm_out.weight, self.layer_norm_out.bias,
+                p[:ch], g[:ch], p[ch:], g[ch:], self.linear_g.weight, self.linear_z.weight)
+
+    @forward_only
+    def forward(self, z, mask=None, inplace_safe=False, use_cueq_triangle_kernels=False,
+                _add_with_inplace=False, _inplace_chunk_size=256):
+        """z [*, N, N, C_z], mask [*, N, N] -> [*, N, N, C_z]; the in-place contract of tmu.py:620-628."""
+        if use_cueq_triangle_kernels:  # tmu.py:612-618
+            raise NotImplementedError("CUEQ triangle multiplicative update kernel not supported for "
+                                      "FusedTriangleMultiplicativeUpdate.")
+        return F3.triangle_multiplicative_update(
+            z, mask, *self._weights(), outgoing=self._outgoing,
+            add_residual=bool(inplace_safe and _add_with_inplace), inplace=bool(inplace_safe))
+
+
+class FusedTriangleMultiplicationOutgoing(FusedTriangleMultiplicativeUpdate):
+    __init__ = partialmethod(FusedTriangleMultiplicativeUpdate.__init__, _outgoing=True)
+
+
+class FusedTriangleMultiplicationIncoming(FusedTriangleMultiplicativeUpdate):
+    __init__ = partialmethod(FusedTriangleMultiplicativeUpdate.__init__, _outgoing=False)
 
 
 class _GatedAttentionParams(nn.Module):

@@ -14,8 +14,8 @@ import torch.nn as nn
 
 from . import functional as F3
 from ._guard import forward_only
-from .layers import (SwiGLUTransition, TriangleAttention, TriangleMultiplicationIncoming,
-                     TriangleMultiplicationOutgoing)
+from .layers import (FusedTriangleMultiplicationIncoming, FusedTriangleMultiplicationOutgoing, SwiGLUTransition,
+                     TriangleAttention, TriangleMultiplicationIncoming, TriangleMultiplicationOutgoing)
 
 
 class PairStack(nn.Module):
@@ -26,12 +26,17 @@ class PairStack(nn.Module):
     PairBlock subclass below."""
 
     def __init__(self, c_z: int, c_hidden_mul: int, c_hidden_pair_att: int, no_heads_pair: int,
-                 inf: float = 1e9, linear_init_params=None):
+                 inf: float = 1e9, linear_init_params=None, fuse_projection_weights: bool = False):
         super().__init__()
-        tm = None if linear_init_params is None else linear_init_params["tri_mul"]
         ta = None if linear_init_params is None else linear_init_params["tri_att"]
-        self.tri_mul_out = TriangleMultiplicationOutgoing(c_z, c_hidden_mul, linear_init_params=tm)
-        self.tri_mul_in = TriangleMultiplicationIncoming(c_z, c_hidden_mul, linear_init_params=tm)
+        if fuse_projection_weights:  # base_blocks.py:260-266
+            tm = None if linear_init_params is None else linear_init_params["fused_tri_mul"]
+            self.tri_mul_out = FusedTriangleMultiplicationOutgoing(c_z, c_hidden_mul, linear_init_params=tm)
+            self.tri_mul_in = FusedTriangleMultiplicationIncoming(c_z, c_hidden_mul, linear_init_params=tm)
+        else:
+            tm = None if linear_init_params is None else linear_init_params["tri_mul"]
+            self.tri_mul_out = TriangleMultiplicationOutgoing(c_z, c_hidden_mul, linear_init_params=tm)
+            self.tri_mul_in = TriangleMultiplicationIncoming(c_z, c_hidden_mul, linear_init_params=tm)
         self.tri_att_start = TriangleAttention(c_z, c_hidden_pair_att, no_heads_pair, inf=inf,
                                                linear_init_params=ta)
         # like the reference, a *starting* module that is handed the transposed tensor
@@ -40,13 +45,8 @@ class PairStack(nn.Module):
 
     @staticmethod
     def _mul(module, z, mask, inplace):
-        return F3.triangle_multiplicative_update(
-            z, mask,
-            module.layer_norm_in.weight, module.layer_norm_in.bias,
-            module.layer_norm_out.weight, module.layer_norm_out.bias,
-            module.linear_a_p.weight, module.linear_a_g.weight, module.linear_b_p.weight, module.linear_b_g.weight,
-            module.linear_g.weight, module.linear_z.weight,
-            outgoing=module._outgoing, add_residual=True, inplace=inplace)
+        return F3.triangle_multiplicative_update(z, mask, *module._weights(), outgoing=module._outgoing,
+                                                 add_residual=True, inplace=inplace)
 
     @staticmethod
     def _att(module, z, mask, inplace):
@@ -90,18 +90,17 @@ class PairBlock(PairStack):
     """The reference's PairBlock (base_blocks.py:218-480): the four triangle updates, then
     z + pair_transition(z, mask).  Same constructor arguments and sub-module names
     (tri_mul_out, tri_mul_in, tri_att_start, tri_att_end, pair_transition).  Only what the
-    AF3 configuration uses is implemented: the SwiGLU transition and un-fused projection
-    weights; pair_dropout is accepted for signature parity (inference: identity)."""
+    AF3 configuration uses is implemented: the SwiGLU transition; fuse_projection_weights selects the
+    fused-projection triangle multiplications (bias-free, as the reference's table initialises them);
+    pair_dropout is accepted for signature parity (inference: identity)."""
 
     def __init__(self, c_z: int, c_hidden_mul: int, c_hidden_pair_att: int, no_heads_pair: int,
                  transition_type: str = "swiglu", transition_n: int = 4, pair_dropout: float = 0.0,
                  fuse_projection_weights: bool = False, inf: float = 1e9, linear_init_params=None):
         if transition_type != "swiglu":
             raise ValueError("Transition type %s is not available (the kernels implement 'swiglu')" % transition_type)
-        if fuse_projection_weights:
-            raise ValueError("fused projection weights are not implemented")
         super().__init__(c_z, c_hidden_mul, c_hidden_pair_att, no_heads_pair, inf=inf,
-                         linear_init_params=linear_init_params)
+                         linear_init_params=linear_init_params, fuse_projection_weights=fuse_projection_weights)
         pt = None
         if linear_init_params is not None and "pair_transition" in linear_init_params:
             pt = linear_init_params["pair_transition"]

@@ -106,6 +106,35 @@ def trimul_update(z, mask, p, outgoing: bool):
     return x * g
 
 
+def fused_trimul_update(z, mask, p, outgoing: bool):
+    """FusedTriangleMultiplicativeUpdate.forward, tmu.py:637-660 (bias-free Linears, as
+    default_linear_init_config.py:122-129 creates them): the a and b projections come stacked out of
+    linear_ab_p / linear_ab_g, [2 * c_hidden, c_z], and are cut apart after gating and masking."""
+    if mask is None:
+        mask = z.new_ones(z.shape[:-1])
+    m = mask.to(z.dtype).unsqueeze(-1)
+    c_hidden = p["linear_ab_p.weight"].shape[0] // 2
+    zn = layer_norm(z, p["layer_norm_in.weight"], p["layer_norm_in.bias"])
+    ab = m
+    ab = ab * torch.sigmoid(linear(zn, p["linear_ab_g.weight"]))
+    ab = ab * linear(zn, p["linear_ab_p.weight"])
+    a = ab[..., :c_hidden]
+    b = ab[..., c_hidden:]
+    x = trimul_contract(a, b, outgoing)
+    x = layer_norm(x, p["layer_norm_out.weight"], p["layer_norm_out.bias"])
+    x = linear(x, p["linear_z.weight"])
+    g = torch.sigmoid(linear(zn, p["linear_g.weight"]))
+    return x * g
+
+
+def fuse_trimul_params(p):
+    """The un-fused parameter set of make_trimul_params under the fused module's names: a on top of b."""
+    q = {k: v for k, v in p.items() if not k.startswith(("linear_a_", "linear_b_"))}
+    q["linear_ab_p.weight"] = torch.cat([p["linear_a_p.weight"], p["linear_b_p.weight"]], dim=0)
+    q["linear_ab_g.weight"] = torch.cat([p["linear_a_g.weight"], p["linear_b_g.weight"]], dim=0)
+    return q
+
+
 # --------------------------------------------------------------------------
 # triangle attention
 # --------------------------------------------------------------------------

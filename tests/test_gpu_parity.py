@@ -228,3 +228,29 @@ def test_config5_four_blocks_run_in_place():
         outs.append(zg.cpu())
         del zg
     assert torch.equal(outs[0], outs[1]), "two runs of the same stack differ bitwise"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("outgoing", [True, False])
+def test_fused_trimul_module(outgoing):
+    """FusedTriangleMultiplicativeUpdate (tmu.py:522-666, bias-free) against the oracle's restatement of
+    its forward, and bit for bit against the un-fused module holding the two halves of the stacked
+    weights (the same kernels on the same numbers); in place with the residual as well."""
+    lib()
+    c, n = 128, 150
+    gen = torch.Generator().manual_seed(88)
+    p = {k: orc.round_bf16(v) for k, v in orc.make_trimul_params(gen, c, c).items()}
+    fp = orc.fuse_trimul_params(p)
+    z = orc.round_bf16(orc.make_pair_input(89, (2,), n, c))
+    mask = orc.tail_padding_mask((2,), n, torch.tensor([13, 0]))
+    cls = of3pair.FusedTriangleMultiplicationOutgoing if outgoing else of3pair.FusedTriangleMultiplicationIncoming
+    ucls = of3pair.TriangleMultiplicationOutgoing if outgoing else of3pair.TriangleMultiplicationIncoming
+    m, u = _load(cls(c, c), fp), _load(ucls(c, c), p)
+    zg = z.to(DEV).to(torch.bfloat16)
+    got = m(zg, mask=mask.to(DEV))
+    assert torch.equal(got, u(zg, mask=mask.to(DEV)))
+    want = orc.fused_trimul_update(z, mask, fp, outgoing)
+    _check("fused trimul update", got, want, rms_rel=5e-3)
+    res = m(zg, mask=mask.to(DEV), inplace_safe=True, _add_with_inplace=True)
+    assert res.data_ptr() == zg.data_ptr()
+    _check("fused trimul in place", res, z + want, rms_rel=5e-3)

@@ -292,3 +292,29 @@ def test_build_stamp_detects_edited_sources(tmp_path, monkeypatch):
     assert B.is_built() and not B.is_stale()
     stamp.write_text("0" * 64 + "\n")
     assert B.is_stale() and not B.is_built()
+
+
+def test_fused_trimul_state_dict_names_and_pair_block_switch():
+    """fuse_projection_weights=True builds the reference's FusedTriangleMultiplication modules
+    (base_blocks.py:260-266; keys linear_ab_p / linear_ab_g with stacked [2 * c_hidden, c_z] weights)."""
+    m = of3pair.FusedTriangleMultiplicationOutgoing(128, 128)
+    want = {
+        "layer_norm_in.weight": (128,), "layer_norm_in.bias": (128,),
+        "layer_norm_out.weight": (128,), "layer_norm_out.bias": (128,),
+        "linear_ab_p.weight": (256, 128), "linear_ab_g.weight": (256, 128),
+        "linear_g.weight": (128, 128), "linear_z.weight": (128, 128),
+    }
+    assert {k: tuple(v.shape) for k, v in m.state_dict().items()} == want
+    assert m._outgoing and not of3pair.FusedTriangleMultiplicationIncoming(64, 64)._outgoing
+    assert m.linear_ab_g.weight.abs().max() == 0 and m.linear_z.weight.abs().max() == 0 and m.linear_ab_p.weight.std() > 0
+    w = m._weights()
+    assert w[4].data_ptr() == m.linear_ab_p.weight.data_ptr() and w[4].shape == (128, 128) and w[4].is_contiguous()
+    assert w[6].data_ptr() == m.linear_ab_p.weight[128:].data_ptr() and w[6].is_contiguous()
+    blk = of3pair.PairBlock(64, 64, 16, 4, "swiglu", 2, 0.0, True, 1e9)
+    assert isinstance(blk.tri_mul_out, of3pair.FusedTriangleMultiplicationOutgoing)
+    assert isinstance(blk.tri_mul_in, of3pair.FusedTriangleMultiplicationIncoming)
+    assert "tri_mul_in.linear_ab_g.weight" in blk.state_dict()
+    with pytest.raises(ValueError):  # the kernels have no bias term
+        of3pair.FusedTriangleMultiplicationOutgoing(64, 64, linear_init_params={"linear_ab_p": {"bias": True, "init": "default"}})
+    with pytest.raises(NotImplementedError):  # tmu.py:612-618
+        m.eval()(torch.zeros(1, 4, 4, 128), use_cueq_triangle_kernels=True)

@@ -33,6 +33,21 @@ def test_trimul_matches_bruteforce(outgoing, seed):
     assert np.abs(got - want).max() < FP32_TOL
 
 
+@pytest.mark.parametrize("outgoing", [True, False])
+def test_fused_trimul_matches_bruteforce(outgoing):
+    """The fused-projection restatement (stacked a/b weights, cut after gating) against the float64 loops
+    run on the two halves of the stacked weights; a swap of the halves (b on top) must lie far outside."""
+    z, mask, tm, _, _ = _tiny(2)
+    fused = orc.fuse_trimul_params(tm)
+    assert fused["linear_ab_p.weight"].shape == (2 * tm["linear_a_p.weight"].shape[0], z.shape[-1])
+    got = orc.fused_trimul_update(z, mask, fused, outgoing).double().numpy()
+    want = bf.trimul_update(z, mask, tm, outgoing)
+    assert np.abs(got - want).max() < FP32_TOL
+    swapped = dict(tm, **{"linear_a_p.weight": tm["linear_b_p.weight"], "linear_b_p.weight": tm["linear_a_p.weight"],
+                          "linear_a_g.weight": tm["linear_b_g.weight"], "linear_b_g.weight": tm["linear_a_g.weight"]})
+    assert np.abs(bf.trimul_update(z, mask, swapped, outgoing) - want).max() > 1e-2
+
+
 def test_trimul_outgoing_differs_from_incoming():
     # guards against the brute force and the oracle both ignoring the direction flag
     z, mask, tm, _, _ = _tiny(3)
