@@ -76,7 +76,14 @@ __device__ __forceinline__ int key2(int row) { return (row >> 4) & 1; }  // 2 ch
 // Every iteration of the tile loop issues the same loads (indices past the end are clamped, their
 // data is never read), so that the compiler can count the loads in flight and its own waits do not
 // drain the ring.
-constexpr int kRows = 4, kRQ = 2, kStages = 2;
+// 32-query tiles per wave: 2 (the shipped form) or 1 (half the accumulators, so that six waves per SIMD fit:
+// measured slower, head width 16 at 4 x 512^2 443 vs 392 us with 76 registers and no spills, head width 32
+// does not fit 80 registers; a K / V^T tile read from LDS then serves half as many logits)
+#ifndef OF3_FLASH_RQ
+#define OF3_FLASH_RQ 2
+#endif
+constexpr int kRows = 4, kRQ = OF3_FLASH_RQ, kStages = 2;
+constexpr int kQW = 32 * kRQ;  // queries per wave
 constexpr float kRaise = 64.0f;  // the offset of a query is raised only when a logit exceeds it by 2^64 ...
 constexpr float kSnap = 32.0f;   // ... and an offset within +-32 is replaced by 0
 constexpr float kMaskedBelow = -1e8f;  // a mask bias below this sends exp2 of any sane logit to exactly 0
@@ -91,10 +98,10 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 // = 4 rows x 256 queries, one work-group per CU: a row's K and V^T tiles, the loads that miss L2, are brought
 // in for twice as many queries).
 template <int D, int QW>
-__global__ __launch_bounds__(64 * kRows * QW, 4) void triattn_flash_kernel(TriattnFlashArgs p, int n_qc, int n_rg,
+__global__ __launch_bounds__(64 * kRows * QW, kRQ == 1 ? 6 : 4) void triattn_flash_kernel(TriattnFlashArgs p, int n_qc, int n_rg,
                                                                              int total, int per_xcd) {
   constexpr int kWaves = kRows * QW;
-  constexpr int QWG = 64 * QW;  // queries per work-group
+  constexpr int QWG = kQW * QW;  // queries per work-group
   constexpr int H = 4;
   constexpr int HD = H * D;
   constexpr int KSQ = D / 16;
@@ -107,7 +114,7 @@ __global__ __launch_bounds__(64 * kRows * QW, 4) void triattn_flash_kernel(Triat
   constexpr int KVI = KI + VI;                       // 1-KB load instructions per row and tile: K0, (K1), V0, (V1)
   constexpr int SPW = KVI / QW > 0 ? KVI / QW : 1;   // of which a wave issues this many (waves beyond KVI: none)
   constexpr int TBS = QWG * 8;  // [QWG q][32 k] fp32 in 16-byte slots
-  constexpr int TBI = 2;  // bias instructions per wave and tile
+  constexpr int TBI = kRQ;  // bias instructions per wave and tile
   static_assert(TBI * 64 * kWaves == TBS, "the waves share the bias slice evenly");
   constexpr int LPT = TBI + KI;
 
@@ -130,7 +137,7 @@ __global__ __launch_bounds__(64 * kRows * QW, 4) void triattn_flash_kernel(Triat
   const int i = row_valid ? i_raw : N - 1;
   const int b = bh / H, h = bh % H;
   const int qwg = qc * QWG;
-  const int q0 = qwg + 64 * qq;
+  const int q0 = qwg + kQW * qq;
 
   const size_t bih = ((size_t)b * N + i) * H + h;
   const bf16_t* Q = p.q + bih * Jp * D;
@@ -214,7 +221,7 @@ __global__ __launch_bounds__(64 * kRows * QW, 4) void triattn_flash_kernel(Triat
     v_rd[s2] = KSLOTS + vr * 4 + ((2 * lh + s2) ^ key4(vr));
   }
   const int tb_key = (l32 >> 1) & 7;
-  const int tb_row = (2 * qq) * 256 + l32 * 8;
+  const int tb_row = (kRQ * qq) * 256 + l32 * 8;
 
   float m_run[kRQ], l_run[kRQ], l_tot[kRQ];
   f32x16_t oacc[kRQ];
@@ -422,7 +429,7 @@ __global__ __launch_bounds__(64 * kRows * QW, 4) void triattn_flash_kernel(Triat
 
 template <int D, int QW>
 constexpr int lds_bytes() {
-  return (kStages * 64 * QW * 8 + kRows * kStages * (32 * (D / 8) + D * 4)) * 16;
+  return (kStages * kQW * QW * 8 + kRows * kStages * (32 * (D / 8) + D * 4)) * 16;
 }
 
 template <int D, int QW>
@@ -438,7 +445,7 @@ hipError_t launch(const TriattnFlashArgs& a, hipStream_t stream) {
       },
       &configured);
   if (e != hipSuccess) return e;
-  const int n_qc = (a.N + 64 * QW - 1) / (64 * QW), n_rg = (a.N + kRows - 1) / kRows;
+  const int n_qc = (a.N + kQW * QW - 1) / (kQW * QW), n_rg = (a.N + kRows - 1) / kRows;
   const long total = (long)n_qc * n_rg * a.B * a.H;
   const int per_xcd = (int)((total + 7) / 8);
   constexpr int kLds = lds_bytes<D, QW>();
