@@ -71,7 +71,8 @@ def source_digest() -> str:
     """sha256 over everything the library is compiled from: the kernel sources and headers, the public
     header and the compiler flags."""
     h = hashlib.sha256(" ".join(_flags()).encode())
-    files = [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith((".hip", ".h"))]
+    files = [os.path.join(CSRC, f) for f in SOURCES]
+    files += [os.path.join(CSRC, f) for f in sorted(os.listdir(CSRC)) if f.endswith(".h")]
     if os.path.isdir(INCLUDE_DIR):
         files += [os.path.join(INCLUDE_DIR, f) for f in sorted(os.listdir(INCLUDE_DIR)) if f.endswith(".h")]
     for path in files:
