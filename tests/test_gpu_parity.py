@@ -254,3 +254,42 @@ def test_fused_trimul_module(outgoing):
     res = m(zg, mask=mask.to(DEV), inplace_safe=True, _add_with_inplace=True)
     assert res.data_ptr() == zg.data_ptr()
     _check("fused trimul in place", res, z + want, rms_rel=5e-3)
+
+
+def test_config5_four_blocks_against_the_fp32_path():
+    """Config 5's composed output: the four stacked bf16 blocks at N=2048 against the same four blocks on
+    the library's fp32 path (three-term bf16 operands, fp32 accumulation; pinned against the oracle within
+    1e-4 by test_gpu_fp32.py at the sizes the CPU reaches).  A composed fp32 pass on the CPU is about
+    65 TFLOP, so the fp32 kernels stand in for it here.  Every block rounds the pair tensor to bf16 four
+    times (one residual write per module), so the bounds are per stack, not the per-module 2e-2: the
+    error may grow with the square root of the number of modules at most."""
+    lib()
+    n, c, heads, d = 2048, 128, 4, 32
+    seeds = (20, 21, 22, 23)
+    params = [_round_params(orc.make_block_params(s, c, c, d, heads)) for s in seeds]
+    z = orc.round_bf16(orc.make_pair_input(7, (1,), n, c))
+    mask = orc.tail_padding_mask((1,), n, 256).to(DEV)
+    print("config 5: four blocks, bf16 against fp32", flush=True)
+    zb = z.to(DEV).to(torch.bfloat16)
+    for p in params:
+        zb = _load(of3pair.PairStack(c, c, d, heads), p)(zb, mask, inplace_safe=True)
+    got = zb.float().cpu()
+    del zb
+    zf = z.to(DEV)
+    for p in params:
+        m = of3pair.PairStack(c, c, d, heads)
+        m.load_state_dict(p, strict=True)
+        zf = m.to(DEV).float().eval()(zf, mask, inplace_safe=True)
+    want = zf.cpu()
+    del zf
+    of3pair.functional.release_workspaces()
+    valid = slice(0, n - 256)
+    g, w = got[0, valid, valid], want[0, valid, valid]
+    err = (g - w)
+    rms, erms = float(w.pow(2).mean().sqrt()), float(err.pow(2).mean().sqrt())
+    emax, wmax = float(err.abs().max()), float(w.abs().max())
+    print("cfg5 composed: rms %.4g err rms %.4g (%.3g rel) max err %.4g of max %.4g (%.3g rel)"
+          % (rms, erms, erms / rms, emax, wmax, emax / wmax), flush=True)
+    record_parity("cfg5 four blocks bf16 vs fp32 path", g, w, None, "rms_rel <= 1e-2, max|err| <= 2e-2 max|want|")
+    assert erms <= 1e-2 * rms
+    assert emax <= 2e-2 * wmax
