@@ -34,6 +34,23 @@ inline hipError_t cu_count(int dev, int* n) {
   return hipDeviceGetAttribute(n, hipDeviceAttributeMultiprocessorCount, dev);
 }
 
+// 128-position tiles of the N x N positions of one batch element: the whole 128-wide pieces of every row
+// (full_per_row per row), then the remaining N % 128 columns in pieces of 2^tail_shift columns (the
+// smallest power of two >= 8 that covers them) x (128 >> tail_shift) consecutive rows.
+struct RaggedTiles {
+  int full_per_row, tail_shift, per_batch;
+};
+inline RaggedTiles ragged_tiles(int N) {
+  RaggedTiles t;
+  t.full_per_row = N / 128;
+  const int r = N % 128;
+  t.tail_shift = r ? 3 : 7;
+  while ((1 << t.tail_shift) < r) ++t.tail_shift;
+  const int rows = 128 >> t.tail_shift;
+  t.per_batch = N * t.full_per_row + (r ? (N + rows - 1) / rows : 0);
+  return t;
+}
+
 // work-groups of `threads` threads (no dynamic LDS) that fit the device at once
 template <typename Kernel>
 inline hipError_t resident_blocks(Kernel kern, int threads, int dev, int* out) {

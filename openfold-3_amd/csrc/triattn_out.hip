@@ -7,6 +7,9 @@
 //
 // HBM bound: reads o and x once, writes out once.  Two MFMA passes per 128-position tile:
 // gate tile -> multiplied into the o tile in LDS in place -> output projection.
+// A tile is 128 consecutive positions of the flattened [B][N][N] index space of the module frame, so it
+// may run over the end of a row (or of a batch element): a token count off the multiples of 128 costs
+// no partly filled tile per row, only one at the very end.
 #include "of3_device.h"
 #include "of3_kernels.h"
 #include "of3_launch.h"
@@ -15,8 +18,8 @@ namespace of3 {
 
 namespace {
 
-template <int C, int HD>
-__global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int tiles_per_row, int total_tiles) {
+template <int C, int HD, int MODE>
+__global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, uint32_t total_pos, int total_tiles) {
   static_assert(C == HD, "o tile shares the x tile geometry");
   constexpr int NCH = C / 8;
   constexpr int LPP = NCH;
@@ -55,25 +58,57 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int 
   }
 
   const int N = p.N;
-  const int tiles_per_batch = N * tiles_per_row;
+  // A tile starts at position p0 = (b0, i0, j0) (wave-uniform: scalar divisions).  With N >= 128 it holds
+  // positions of at most two rows, whose offsets in the view are the scalars row0 and row1; position d of
+  // the tile then costs a compare and two selects.  Smaller N: the general walk.
+  struct Origin {
+    int b0, i0, j0;
+    int64_t row0, row1;
+  };
+  // MODE 0: N is a multiple of 128, a tile lies inside one row; 1: N >= 128, at most two rows; 2: any N
+  constexpr bool two_rows = MODE == 1, one_row = MODE == 0;
+  auto tile_origin = [&](int tile_id) {
+    Origin t;
+    const uint32_t p0 = (uint32_t)tile_id * TP, nn = (uint32_t)N * (uint32_t)N;
+    t.b0 = (int)(p0 / nn);
+    const uint32_t rem = p0 - (uint32_t)t.b0 * nn;
+    t.i0 = (int)(rem / (uint32_t)N);
+    t.j0 = (int)(rem - (uint32_t)t.i0 * (uint32_t)N);
+    const bool last = t.i0 + 1 == N;
+    t.row0 = t.b0 * p.x_view.stride_b + t.i0 * p.x_view.stride_r;
+    t.row1 = (t.b0 + (last ? 1 : 0)) * p.x_view.stride_b + (last ? 0 : t.i0 + 1) * p.x_view.stride_r;
+    return t;
+  };
+  // element offset of position d of the tile in the x / out view (the position must exist)
+  auto view_offset = [&](const Origin& t, int d) -> int64_t {
+    int j = t.j0 + d;
+    if constexpr (one_row) {
+      return t.row0 + j * p.x_view.stride_k;
+    } else if constexpr (two_rows) {
+      const bool wrapped = j >= N;
+      j -= wrapped ? N : 0;
+      return (wrapped ? t.row1 : t.row0) + j * p.x_view.stride_k;
+    } else {
+      int b = t.b0, i = t.i0;
+      while (j >= N) j -= N, ++i;
+      while (i >= N) i -= N, ++b;
+      return b * p.x_view.stride_b + i * p.x_view.stride_r + j * p.x_view.stride_k;
+    }
+  };
 
   // The loads of a tile are issued one tile ahead (right after the previous tile's values have
   // been consumed by the LayerNorm phase) and travel under that tile's two MFMA phases.
   u32x4_t xraw[LN_ITERS], oraw[LN_ITERS];
   auto load_tile = [&](int tile_id) {
-    const int b = tile_id / tiles_per_batch;
-    const int rem = tile_id - b * tiles_per_batch;
-    const int i = rem / tiles_per_row;
-    const int j0 = (rem - i * tiles_per_row) * TP;
-    const bf16_t* xrow = p.x + b * p.x_view.stride_b + i * p.x_view.stride_r;
-    const bf16_t* orow = p.o + ((size_t)b * N + i) * N * HD;
+    const Origin t = tile_origin(tile_id);
+    const uint32_t p0 = (uint32_t)tile_id * TP;
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
+      const int d = wave * (TP / NW) + it * PPI + ln_pp;
       u32x4_t vx = {0u, 0u, 0u, 0u}, vo = {0u, 0u, 0u, 0u};
-      if (j < N) {
-        vx = *reinterpret_cast<const u32x4_t*>(xrow + j * p.x_view.stride_k + 8 * ln_chunk);
-        vo = *reinterpret_cast<const u32x4_t*>(orow + (size_t)j * HD + 8 * ln_chunk);
+      if (p0 + d < total_pos) {
+        vx = *reinterpret_cast<const u32x4_t*>(p.x + view_offset(t, d) + 8 * ln_chunk);
+        vo = *reinterpret_cast<const u32x4_t*>(p.o + (size_t)(p0 + d) * HD + 8 * ln_chunk);  // o is [B][N][N][HD]
       }
       xraw[it] = vx;
       oraw[it] = vo;
@@ -82,11 +117,8 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int 
   if ((int)blockIdx.x < total_tiles) load_tile(blockIdx.x);
 
   for (int tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
-    const int b = tile_id / tiles_per_batch;
-    const int rem = tile_id - b * tiles_per_batch;
-    const int i = rem / tiles_per_row;
-    const int j0 = (rem - i * tiles_per_row) * TP;
-    bf16_t* outrow = p.out + b * p.x_view.stride_b + i * p.x_view.stride_r;
+    const Origin t = tile_origin(tile_id);
+    const uint32_t p0 = (uint32_t)tile_id * TP;
 
     // ---- LayerNorm of this tile's values, then the next tile's loads
 #pragma unroll
@@ -126,9 +158,9 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int 
       f32x16_t acc = zero16();
 #pragma unroll
       for (int s = 0; s < KS; ++s) acc = mfma_32x32x16(wo[s], otile[tile_slot<NCH, 0>(pos, 2 * s + lh)], acc);
-      const int j = j0 + pos;
-      if (j < N) {
-        const int64_t off = j * p.x_view.stride_k + 32 * ot + 16 * lh;
+      if (p0 + pos < total_pos) {
+        bf16_t* outrow = p.out;
+        const int64_t off = view_offset(t, pos) + 32 * ot + 16 * lh;
         float res[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) res[v] = acc[v];
@@ -157,25 +189,30 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, int 
   }
 }
 
-template <int C, int HD>
+template <int C, int HD, int MODE>
 hipError_t launch(const TriattnOutArgs& a, hipStream_t stream) {
-  auto kern = triattn_out_kernel<C, HD>;
+  auto kern = triattn_out_kernel<C, HD, MODE>;
   static int cache[kMaxDevices];
   int grid_cap = 0;
   hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 512, dev, v); }, &grid_cap);
   if (e != hipSuccess) return e;
-  const int tiles_per_row = (a.N + 127) / 128;
-  const long total = (long)a.B * a.N * tiles_per_row;
+  const long positions = (long)a.B * a.N * a.N;
+  if (positions <= 0 || positions > 0x7fffffffL) return hipErrorInvalidValue;
+  const long total = (positions + 127) / 128;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, tiles_per_row, (int)total);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, (uint32_t)positions, (int)total);
   return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t triattn_out_launch(const TriattnOutArgs& args, int C, int HD, hipStream_t stream) {
-  if (C == 128 && HD == 128) return launch<128, 128>(args, stream);
-  if (C == 64 && HD == 64) return launch<64, 64>(args, stream);
+  // a 128-position tile lies in one row (N a multiple of 128), in at most two (N >= 128), or anywhere
+  const int mode = args.N % 128 == 0 ? 0 : (args.N >= 128 ? 1 : 2);
+  if (C == 128 && HD == 128)
+    return mode == 0 ? launch<128, 128, 0>(args, stream) : (mode == 1 ? launch<128, 128, 1>(args, stream) : launch<128, 128, 2>(args, stream));
+  if (C == 64 && HD == 64)
+    return mode == 0 ? launch<64, 64, 0>(args, stream) : (mode == 1 ? launch<64, 64, 1>(args, stream) : launch<64, 64, 2>(args, stream));
   return hipErrorInvalidValue;
 }
 

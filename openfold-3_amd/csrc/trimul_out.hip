@@ -7,6 +7,11 @@
 // saves one full write and one full read of a z-sized tensor.
 //
 // HBM bound: reads x and z once, writes out once.
+//
+// Tiles are 128 positions: the whole 128-wide pieces of every row first, then, when N is not a multiple
+// of 128, the remaining columns in pieces of 2^s columns x 128 / 2^s consecutive rows (2^s the smallest
+// power of two >= 8 that covers them), so that the ragged end of the rows costs a few tiles per batch
+// element rather than one more tile per row.
 #include "of3_device.h"
 #include "of3_kernels.h"
 #include "of3_launch.h"
@@ -15,8 +20,9 @@ namespace of3 {
 
 namespace {
 
-template <int C, int CH>
-__global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int tiles_per_row, int total_tiles) {
+template <int C, int CH, bool RAGGED>
+__global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int full_per_row, int tail_shift, int tiles_per_batch,
+                                                           int total_tiles) {
   static_assert(C == CH, "position-major x tile shares the z tile geometry");
   constexpr int NCH = C / 8;
   constexpr int LPP = NCH;
@@ -60,7 +66,22 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
   }
 
   const int N = p.N, Np = p.Np;
-  const int tiles_per_batch = N * tiles_per_row;
+  const int main_tiles = N * full_per_row;  // per batch element
+  // tile -> batch element, first row, first column, log2 of its width (all wave-uniform); position pos of
+  // the tile is row i0 + (pos >> shift), column j0 + (pos & (width - 1))
+  auto tile_origin = [&](int tile_id, int& b, int& i0, int& j0, int& shift) {
+    b = tile_id / tiles_per_batch;
+    const int rem = tile_id - b * tiles_per_batch;
+    if (!RAGGED || rem < main_tiles) {  // N a multiple of 128: whole-row pieces only
+      i0 = rem / full_per_row;
+      j0 = (rem - i0 * full_per_row) * TP;
+      shift = 7;
+    } else {
+      i0 = (rem - main_tiles) * (TP >> tail_shift);
+      j0 = full_per_row * TP;
+      shift = tail_shift;
+    }
+  };
   uint32_t* xt32 = reinterpret_cast<uint32_t*>(xtile);
 
   // The loads of a tile (z row-wise for the gate, x channel-major) are issued one tile ahead,
@@ -68,23 +89,27 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
   u32x4_t zraw[LN_ITERS];
   u32x4_t xa[XROUNDS], xb[XROUNDS];
   auto load_tile = [&](int tile_id) {
-    const int b = tile_id / tiles_per_batch;
-    const int rem = tile_id - b * tiles_per_batch;
-    const int i = rem / tiles_per_row;
-    const int j0 = (rem - i * tiles_per_row) * TP;
-    const bf16_t* zrow = p.z + b * p.z_view.stride_b + i * p.z_view.stride_r;
+    int b, i0, j0, shift_rt;
+    tile_origin(tile_id, b, i0, j0, shift_rt);
+    const int shift = RAGGED ? shift_rt : 7;  // a constant without ragged pieces: di below folds to 0
+    const int jmask = (1 << shift) - 1;
+    const bf16_t* zrow = p.z + b * p.z_view.stride_b + i0 * p.z_view.stride_r;  // the tile's first row (scalar)
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
+      const int pos = wave * (TP / NW) + it * PPI + ln_pp;
+      const int di = RAGGED ? pos >> shift : 0, j = j0 + (RAGGED ? pos & jmask : pos);  // di = 0 in the whole-row pieces
       u32x4_t v = {0u, 0u, 0u, 0u};
-      if (j < N) v = *reinterpret_cast<const u32x4_t*>(zrow + j * p.z_view.stride_k + 8 * ln_chunk);
+      if ((!RAGGED || i0 + di < N) && j < N) v = *reinterpret_cast<const u32x4_t*>(zrow + di * p.z_view.stride_r + j * p.z_view.stride_k + 8 * ln_chunk);
       zraw[it] = v;
     }
 #pragma unroll
     for (int rr = 0; rr < XROUNDS; ++rr) {
       const int item = rr * 512 + tid;
-      const int cp = item >> 4, pg = item & 15;  // channels 2cp, 2cp+1; positions 8pg..8pg+7
-      const bf16_t* src = p.x + (((size_t)b * CH + 2 * cp) * Np + i) * Np + j0 + 8 * pg;
+      const int cp = item >> 4, pg = item & 15;  // channels 2cp, 2cp+1; positions 8pg..8pg+7: one row, as the width is >= 8
+      int i = i0 + (RAGGED ? (8 * pg) >> shift : 0);
+      const int j = j0 + (RAGGED ? (8 * pg) & jmask : 8 * pg);  // < Np: the planes are padded to whole 128-wide pieces
+      if (RAGGED) i = i < Np ? i : Np - 1;    // rows of a last piece past the end of the plane: any row, never used
+      const bf16_t* src = p.x + (((size_t)b * CH + 2 * cp) * Np + i) * Np + j;
       xa[rr] = *reinterpret_cast<const u32x4_t*>(src);
       xb[rr] = *reinterpret_cast<const u32x4_t*>(src + (size_t)Np * Np);
     }
@@ -92,11 +117,11 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
   if ((int)blockIdx.x < total_tiles) load_tile(blockIdx.x);
 
   for (int tile_id = blockIdx.x; tile_id < total_tiles; tile_id += gridDim.x) {
-    const int b = tile_id / tiles_per_batch;
-    const int rem = tile_id - b * tiles_per_batch;
-    const int i = rem / tiles_per_row;
-    const int j0 = (rem - i * tiles_per_row) * TP;
-    bf16_t* orow = p.out + b * p.z_view.stride_b + i * p.z_view.stride_r;
+    int b, i0, j0, shift_rt;
+    tile_origin(tile_id, b, i0, j0, shift_rt);
+    const int shift = RAGGED ? shift_rt : 7;
+    const int jmask = (1 << shift) - 1;
+    bf16_t* orow0 = p.out + b * p.z_view.stride_b + i0 * p.z_view.stride_r;  // the tile's first row (scalar)
 
     // x: transpose into xtile[pos][c] with 4-byte (channel pair) writes
 #pragma unroll
@@ -144,9 +169,10 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
         accu = mfma_32x32x16(wz[s], bx, accu);
         accg = mfma_32x32x16(wgt[s], bz, accg);
       }
-      const int j = j0 + pos;
-      if (j < N) {
-        const int64_t off = j * p.z_view.stride_k + 32 * ot + 16 * lh;
+      const int di = RAGGED ? pos >> shift : 0, j = j0 + (RAGGED ? pos & jmask : pos);
+      if ((!RAGGED || i0 + di < N) && j < N) {
+        bf16_t* orow = orow0;
+        const int64_t off = di * p.z_view.stride_r + j * p.z_view.stride_k + 32 * ot + 16 * lh;
         float res[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) res[v] = accu[v] * sigmoidf_fast(accg[v]);
@@ -175,25 +201,27 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int ti
   }
 }
 
-template <int C, int CH>
+template <int C, int CH, bool RAGGED>
 hipError_t launch(const TrimulOutArgs& a, hipStream_t stream) {
-  auto kern = trimul_out_kernel<C, CH>;
+  auto kern = trimul_out_kernel<C, CH, RAGGED>;
   static int cache[kMaxDevices];
   int grid_cap = 0;
   hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 512, dev, v); }, &grid_cap);
   if (e != hipSuccess) return e;
-  const int tiles_per_row = (a.N + 127) / 128;
-  const long total = (long)a.B * a.N * tiles_per_row;
+  const RaggedTiles t = ragged_tiles(a.N);
+  const long total = (long)a.B * t.per_batch;
+  if (total > 0x7fffffffL) return hipErrorInvalidValue;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, tiles_per_row, (int)total);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), 0, stream, a, t.full_per_row, t.tail_shift, t.per_batch, (int)total);
   return hipGetLastError();
 }
 
 }  // namespace
 
 hipError_t trimul_out_launch(const TrimulOutArgs& args, int C, int CH, hipStream_t stream) {
-  if (C == 128 && CH == 128) return launch<128, 128>(args, stream);
-  if (C == 64 && CH == 64) return launch<64, 64>(args, stream);
+  const bool ragged = args.N % 128 != 0;
+  if (C == 128 && CH == 128) return ragged ? launch<128, 128, true>(args, stream) : launch<128, 128, false>(args, stream);
+  if (C == 64 && CH == 64) return ragged ? launch<64, 64, true>(args, stream) : launch<64, 64, false>(args, stream);
   return hipErrorInvalidValue;
 }
 

@@ -126,7 +126,7 @@ def test_trimul_proj(outgoing, C, n, B):
 
 
 @pytest.mark.parametrize("add_residual", [0, 1])
-@pytest.mark.parametrize("C,n,B", [(128, 70, 2), (64, 130, 1)])
+@pytest.mark.parametrize("C,n,B", [(128, 70, 2), (64, 130, 1), (128, 150, 2), (128, 5, 3), (64, 291, 1)])
 def test_trimul_out(add_residual, C, n, B):
     L = lib()
     gen = _gen(29 + n)
@@ -335,7 +335,7 @@ def test_triattn_flash_padding_masks(D, n, B, pads):
 
 
 @pytest.mark.parametrize("transposed,add_residual", [(False, 0), (True, 1)])
-@pytest.mark.parametrize("C,D,n,B", [(128, 32, 70, 2), (64, 16, 130, 1)])
+@pytest.mark.parametrize("C,D,n,B", [(128, 32, 70, 2), (64, 16, 130, 1), (128, 32, 5, 3), (128, 32, 150, 2)])
 def test_triattn_out(transposed, add_residual, C, D, n, B):
     L = lib()
     H = 4
