@@ -164,8 +164,10 @@ int64_t of3_triattn_workspace_bytes(int64_t B, int64_t N, int64_t C, int64_t H, 
 /* The same for either dtype (fp32: q, k, v, o = 4 * B*N*N*H*D floats, triangle bias B*H*N*N floats). */
 int64_t of3_triattn_workspace_bytes_for(int dtype, int64_t B, int64_t N, int64_t C, int64_t H, int64_t D);
 
-/* q is pre-multiplied by log2(e)/sqrt(D); tbias and mbias by log2(e); mbias is -inf for
- * j >= N.  (i, j) are the module's frame as given by x_strides / mask_strides. */
+/* q is pre-multiplied by log2(e)/sqrt(D); tbias and mbias by log2(e).  Columns j >= N are written as far
+ * as of3_triattn_flash reads them, i.e. up to the end of the 32-key panel that holds token N-1 (mbias -inf,
+ * tbias 0, k and vt finite); the rest of the padding up to NP is left as it was.  (i, j) are the module's
+ * frame as given by x_strides / mask_strides. */
 int of3_triattn_proj(const void* x, const int64_t x_strides[3], const float* mask, const int64_t mask_strides[3],
                      const void* ln_w, const void* ln_b, const void* w_q, const void* w_k, const void* w_v,
                      const void* w_bias, void* q, void* k, void* vt, float* tbias, float* mbias, int64_t B,

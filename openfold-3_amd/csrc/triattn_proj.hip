@@ -12,6 +12,13 @@
 // triangle-multiplication input pass: 8 waves per work-group, weights resident in registers
 // as MFMA A operands, 128-position tiles normalised in registers and staged once in a
 // double-buffered LDS tile (one barrier per tile).
+//
+// Tiles: the whole 128-wide pieces of every row; when N is not a multiple of 128 (RAGGED), the remaining
+// columns come in pieces of 32, 64 or 128 columns x 4, 2 or 1 consecutive rows, so that the ragged end
+// of the rows costs a tile per four (two) rows instead of one per row.  The last such piece of a batch
+// element is moved up to end at the last row (rows computed twice are written twice with the same values).
+// Columns are written up to the end of the 32-wide panel that holds the last token, which is as far as
+// the attention core reads.
 #include "of3_device.h"
 #include "of3_kernels.h"
 #include "of3_launch.h"
@@ -37,8 +44,9 @@ __device__ __forceinline__ int proj_slot(int pos, int chunk) {
   return pos * NCH + (chunk ^ key);
 }
 
-template <int C, int D, int NW>
-__global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p, int tiles_per_row, int total_tiles) {
+template <int C, int D, int NW, bool RAGGED>
+__global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p, int full_per_row, int tail_shift,
+                                                               int tiles_per_batch, int total_tiles) {
   constexpr int H = 4;
   constexpr int HD = H * D;
   constexpr int NCH = C / 8;
@@ -84,25 +92,42 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
   const float qscale = kLog2e * __builtin_amdgcn_rsqf((float)D);
 
   const int N = p.N, Jp = p.Jp;
-  const int tiles_per_batch = N * tiles_per_row;
+  // tile -> batch element, first row, first column, log2 of the width (wave-uniform); position pos of the
+  // tile is row i0 + (pos >> shift), column j0 + (pos & (width - 1)); without ragged pieces shift is 7
+  const int main_tiles = N * full_per_row;
+  auto tile_origin = [&](int tile_id, int& b, int& i0, int& j0, int& shift) {
+    b = tile_id / tiles_per_batch;
+    const int rem = tile_id - b * tiles_per_batch;
+    if (!RAGGED || rem < main_tiles) {
+      i0 = rem / full_per_row;
+      j0 = (rem - i0 * full_per_row) * TP;
+      shift = 7;
+    } else {
+      const int rows = TP >> tail_shift;
+      i0 = (rem - main_tiles) * rows;
+      i0 = i0 + rows <= N ? i0 : N - rows;  // the launcher makes sure that N >= rows
+      j0 = full_per_row * TP;
+      shift = tail_shift;
+    }
+  };
 
   u32x4_t raw[LN_ITERS];
   float mraw[LN_ITERS];  // mask of the same positions (used by the lane with ln_chunk == 0)
   auto load_tile = [&](int tile_id) {
-    const int b = tile_id / tiles_per_batch;
-    const int rem = tile_id - b * tiles_per_batch;
-    const int i = rem / tiles_per_row;
-    const int j0 = (rem - i * tiles_per_row) * TP;
-    const bf16_t* xrow = p.x + b * p.x_view.stride_b + i * p.x_view.stride_r;
-    const float* mrow = p.mask ? p.mask + b * p.mask_view.stride_b + i * p.mask_view.stride_r : nullptr;
+    int b, i0, j0, shift_rt;
+    tile_origin(tile_id, b, i0, j0, shift_rt);
+    const int shift = RAGGED ? shift_rt : 7, jmask = (1 << shift) - 1;
+    const bf16_t* xrow = p.x + b * p.x_view.stride_b + i0 * p.x_view.stride_r;  // the tile's first row
+    const float* mrow = p.mask ? p.mask + b * p.mask_view.stride_b + i0 * p.mask_view.stride_r : nullptr;
 #pragma unroll
     for (int it = 0; it < LN_ITERS; ++it) {
-      const int j = j0 + wave * (TP / NW) + it * PPI + ln_pp;
+      const int pos = wave * (TP / NW) + it * PPI + ln_pp;
+      const int di = RAGGED ? pos >> shift : 0, j = j0 + (RAGGED ? pos & jmask : pos);  // every row i0 + di exists
       u32x4_t v = {0u, 0u, 0u, 0u};
       float m = 1.f;
       if (j < N) {
-        v = *reinterpret_cast<const u32x4_t*>(xrow + j * p.x_view.stride_k + 8 * ln_chunk);
-        if (mrow && ln_chunk == 0) m = mrow[j * p.mask_view.stride_k];
+        v = *reinterpret_cast<const u32x4_t*>(xrow + di * p.x_view.stride_r + j * p.x_view.stride_k + 8 * ln_chunk);
+        if (mrow && ln_chunk == 0) m = mrow[di * p.mask_view.stride_r + j * p.mask_view.stride_k];
       }
       raw[it] = v;
       mraw[it] = m;
@@ -141,10 +166,12 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
     }
 
     auto do_tile = [&](int tile_id, int buf) {
-      const int b = tile_id / tiles_per_batch;
-      const int rem = tile_id - b * tiles_per_batch;
-      const int i = rem / tiles_per_row;
-      const int j0 = (rem - i * tiles_per_row) * TP;
+      int b, i0, j0, shift_rt;
+      tile_origin(tile_id, b, i0, j0, shift_rt);
+      const int shift = RAGGED ? shift_rt : 7, jmask = (1 << shift) - 1;
+      // row and first column of the 32-position tile tt (wave-uniform): one row, one 32-key panel
+      auto tile_row = [&](int tt) { return RAGGED ? i0 + ((32 * tt) >> shift) : i0; };
+      auto tile_col = [&](int tt) { return RAGGED ? j0 + ((32 * tt) & jmask) : j0 + 32 * tt; };
 
       // ---- LayerNorm phase (+ mask bias, one lane per position)
 #pragma unroll
@@ -152,7 +179,7 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
         const int pos = wave * (TP / NW) + it * PPI + ln_pp;
         tile[buf][proj_slot<NCH>(pos, ln_chunk)] = layer_norm_chunk<C>(raw[it], lw, lb);
         if (ln_chunk == 0) {
-          const int j = j0 + pos;
+          const int i = RAGGED ? i0 + (pos >> shift) : i0, j = j0 + (RAGGED ? pos & jmask : pos);
           float mb = -__builtin_inff();
           if (j < N) mb = kLog2e * (p.inf * (mraw[it] - 1.f));
           p.mbias[((size_t)b * N + i) * Jp + j] = mb;
@@ -162,9 +189,8 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
       __syncthreads();  // the only barrier per tile (the LDS tile is double buffered)
 
       // ---- projection phase
-      const size_t bi = (size_t)b * N + i;
       auto bias_tile = [&](int tt) {  // triangle bias of position tile tt (wave-uniform, may be a run-time value)
-        const int pos = 32 * tt + l32, j = j0 + pos;
+        const int pos = 32 * tt + l32, i = tile_row(tt), j = tile_col(tt) + l32;
         f32x16_t acc = zero16();
 #pragma unroll
         for (int s = 0; s < KS; ++s)
@@ -186,6 +212,8 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
       }
 #pragma unroll
       for (int tt = 0; tt < TPW; ++tt) {
+        const size_t bi = (size_t)b * N + tile_row(tt);
+        const int jt = tile_col(tt);
 #pragma unroll
         for (int jj = 0; jj < NJ; ++jj) {
           f32x16_t acc = zero16();
@@ -205,7 +233,7 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
               o0[q] = pack_bf16(acc[2 * q], acc[2 * q + 1]);
               o1[q] = pack_bf16(acc[8 + 2 * q], acc[8 + 2 * q + 1]);
             }
-            dst = p.vt + (bi * H + head) * D * Jp + (size_t)((j0 >> 5) + tt) * (D * 32) + d * 32 + 16 * lh;
+            dst = p.vt + (bi * H + head) * D * Jp + (size_t)(jt >> 5) * (D * 32) + d * 32 + 16 * lh;
           } else {
             // the activation operand is re-read from LDS by every job: cheaper than holding it in
             // 32 registers across the jobs
@@ -223,7 +251,7 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
               o0[q] = pack_bf16(acc[2 * q] * sc, acc[2 * q + 1] * sc);
               o1[q] = pack_bf16(acc[8 + 2 * q] * sc, acc[8 + 2 * q + 1] * sc);
             }
-            dst = (is_q ? p.q : p.k) + ((bi * H + head) * Jp + j0 + pos) * D + d0;
+            dst = (is_q ? p.q : p.k) + ((bi * H + head) * Jp + jt + l32) * D + d0;
           }
           *reinterpret_cast<u32x4_t*>(dst) = o0;
           *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
@@ -257,17 +285,19 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
   }
 }
 
-template <int C, int D, int NW>
+template <int C, int D, int NW, bool RAGGED>
 hipError_t launch(const TriattnProjArgs& a, hipStream_t stream) {
-  auto kern = triattn_proj_kernel<C, D, NW>;
+  auto kern = triattn_proj_kernel<C, D, NW, RAGGED>;
   static int cache[kMaxDevices];
   int grid_cap = 0;
   hipError_t e = per_device(cache, [&](int dev, int* v) { return resident_blocks(kern, 64 * NW, dev, v); }, &grid_cap);
   if (e != hipSuccess) return e;
-  const int tiles_per_row = a.Jp / 128;
-  const long total = (long)a.B * a.N * tiles_per_row;
+  RaggedTiles t = {a.Jp / 128, 7, a.N * (a.Jp / 128)};  // whole (padded) rows in 128-wide pieces
+  if (RAGGED) t = ragged_tiles(a.N, 5);                 // pieces of whole 32-key panels
+  const long total = (long)a.B * t.per_batch;
+  if (total > 0x7fffffffL) return hipErrorInvalidValue;
   const int grid = (int)(total < grid_cap ? total : grid_cap);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), 0, stream, a, tiles_per_row, (int)total);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), 0, stream, a, t.full_per_row, t.tail_shift, t.per_batch, (int)total);
   return hipGetLastError();
 }
 
@@ -275,8 +305,10 @@ hipError_t launch(const TriattnProjArgs& a, hipStream_t stream) {
 
 hipError_t triattn_proj_launch(const TriattnProjArgs& args, int C, int D, hipStream_t stream) {
   if (args.H != 4) return hipErrorInvalidValue;
-  if (C == 128 && D == 32) return launch<128, 32, OF3_TP_WAVES>(args, stream);
-  if (C == 64 && D == 16) return launch<64, 16, 8>(args, stream);
+  // ragged pieces hold up to four rows, all of which must exist
+  const bool ragged = args.N % 128 != 0 && args.N >= 4;
+  if (C == 128 && D == 32) return ragged ? launch<128, 32, OF3_TP_WAVES, true>(args, stream) : launch<128, 32, OF3_TP_WAVES, false>(args, stream);
+  if (C == 64 && D == 16) return ragged ? launch<64, 16, 8, true>(args, stream) : launch<64, 16, 8, false>(args, stream);
   return hipErrorInvalidValue;
 }
 

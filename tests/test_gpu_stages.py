@@ -164,7 +164,7 @@ def _triattn_weights(gen, C, H, D):
 
 
 @pytest.mark.parametrize("transposed", [False, True])
-@pytest.mark.parametrize("C,D,n,B", [(128, 32, 70, 2), (64, 16, 130, 1)])
+@pytest.mark.parametrize("C,D,n,B", [(128, 32, 70, 2), (64, 16, 130, 1), (128, 32, 161, 1), (128, 32, 6, 3), (64, 16, 3, 2)])
 def test_triattn_proj(transposed, C, D, n, B):
     L = lib()
     H = 4
@@ -199,8 +199,11 @@ def test_triattn_proj(transposed, C, D, n, B):
     report("vt", vt[..., :n], vr, atol=2e-2, rtol=1e-2)
     report("tbias", tb[..., :n], tbr, atol=2e-2, rtol=1e-2)
     assert torch.equal(mb[..., :n], mbr), "mask bias"
-    assert torch.isinf(mb[..., n:]).all() and (mb[..., n:] < 0).all(), "padded keys must carry -inf"
-    assert torch.isfinite(k[:, :, :, n:].float()).all() and torch.isfinite(vt[..., n:].float()).all()
+    # the padding is written as far as the attention core reads: to the end of the last token's 32-key panel
+    n32 = 32 * ((n + 31) // 32)
+    assert torch.isinf(mb[..., n:n32]).all() and (mb[..., n:n32] < 0).all(), "padded keys must carry -inf"
+    assert torch.isfinite(k[:, :, :, n:n32].float()).all() and torch.isfinite(vt[..., n:n32].float()).all()
+    assert (tb[..., n:n32] == 0).all()
 
 
 # logit_scale > 1 drives the logits far beyond the range in which a softmax without running maxima is
