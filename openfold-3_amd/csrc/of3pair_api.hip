@@ -131,7 +131,7 @@ inline int contract_variant_auto(int64_t planes, int64_t Np) {
   const int64_t cus = current_cu_count();
   const int64_t bm[4] = {256, 256, 256, 384};
   const int64_t bn[4] = {192, 128, 256, 192};
-  const double eff[4] = {0.97, 0.90, 1.00, 1.00};
+  const double eff[4] = {0.93, 0.85, 1.00, 1.00};
   int best = 1;
   double best_cost = 0;
   for (int v = 0; v < 4; ++v) {
