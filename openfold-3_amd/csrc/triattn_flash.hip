@@ -84,6 +84,10 @@ __device__ __forceinline__ int key2(int row) { return (row >> 4) & 1; }  // 2 ch
 #endif
 constexpr int kRows = 4, kRQ = OF3_FLASH_RQ, kStages = 2;
 constexpr int kQW = 32 * kRQ;  // queries per wave
+#ifndef OF3_FLASH_RG_BLOCK
+#define OF3_FLASH_RG_BLOCK 8
+#endif
+constexpr int kRgBlock = OF3_FLASH_RG_BLOCK;  // row groups per block of the work-group order
 constexpr float kRaise = 64.0f;  // the offset of a query is raised only when a logit exceeds it by 2^64 ...
 constexpr float kSnap = 32.0f;   // ... and an offset within +-32 is replaced by 0
 constexpr float kMaskedBelow = -1e8f;  // a mask bias below this sends exp2 of any sane logit to exactly 0
@@ -129,9 +133,18 @@ __global__ __launch_bounds__(64 * kRows * QW, kRQ == 1 ? 6 : 4) void triattn_fla
   const int N = p.N, Jp = p.Jp;
   const int logical = xcd_logical_block(blockIdx.x, per_xcd);
   if (logical >= total) return;  // whole work-group leaves together
-  const int qc = logical % n_qc;
-  const int rg = (logical / n_qc) % n_rg;
-  const int bh = logical / (n_qc * n_rg);
+  // Order of the work-groups of one (batch element, head): blocks of kRgBlock row groups, inside a block
+  // the row group runs fastest, then the query range.  The work-groups resident on an XCD together (about
+  // 64) are then a block of row groups x a run of query ranges, and both streams that miss the L2 are
+  // shared: a row group's K / V^T tiles by its query ranges, a query range's bias slice by the row groups.
+  const int per_bh = n_qc * n_rg;
+  const int bh = logical / per_bh;
+  const int idx = logical - bh * per_bh;
+  const int blk = idx / (kRgBlock * n_qc);
+  const int within = idx - blk * (kRgBlock * n_qc);
+  const int blk_rows = n_rg - blk * kRgBlock < kRgBlock ? n_rg - blk * kRgBlock : kRgBlock;  // the last block may be short
+  const int qc = within / blk_rows;
+  const int rg = blk * kRgBlock + (within - qc * blk_rows);
   const int i_raw = rg * kRows + row;
   const bool row_valid = i_raw < N;  // wave-uniform; idle waves still take part in the loads and barriers
   const int i = row_valid ? i_raw : N - 1;
