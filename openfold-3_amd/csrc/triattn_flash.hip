@@ -87,7 +87,7 @@ constexpr int kQW = 32 * kRQ;  // queries per wave
 #ifndef OF3_FLASH_RG_BLOCK
 #define OF3_FLASH_RG_BLOCK 8
 #endif
-constexpr int kRgBlock = OF3_FLASH_RG_BLOCK;  // row groups per block of the work-group order
+constexpr int kRgBlock = OF3_FLASH_RG_BLOCK, kQcBlock = 8;  // row groups x query ranges per block of the work-group order
 constexpr float kRaise = 64.0f;  // the offset of a query is raised only when a logit exceeds it by 2^64 ...
 constexpr float kSnap = 32.0f;   // ... and an offset within +-32 is replaced by 0
 constexpr float kMaskedBelow = -1e8f;  // a mask bias below this sends exp2 of any sane logit to exactly 0
@@ -133,18 +133,24 @@ __global__ __launch_bounds__(64 * kRows * QW, kRQ == 1 ? 6 : 4) void triattn_fla
   const int N = p.N, Jp = p.Jp;
   const int logical = xcd_logical_block(blockIdx.x, per_xcd);
   if (logical >= total) return;  // whole work-group leaves together
-  // Order of the work-groups of one (batch element, head): blocks of kRgBlock row groups, inside a block
-  // the row group runs fastest, then the query range.  The work-groups resident on an XCD together (about
-  // 64) are then a block of row groups x a run of query ranges, and both streams that miss the L2 are
-  // shared: a row group's K / V^T tiles by its query ranges, a query range's bias slice by the row groups.
+  // Order of the work-groups of one (batch element, head): blocks of kRgBlock row groups x kQcBlock query
+  // ranges; inside a block the query range runs fastest, then the row group.  The work-groups resident on
+  // an XCD together (about 64) are then one such block, and both streams that miss the L2 are shared: a
+  // row group's K / V^T tiles by its query ranges, a query range's bias slice by the row groups.  With
+  // kQcBlock query ranges or fewer (N <= 1024) this is simply: all query ranges of a row group, then the
+  // next row group.
   const int per_bh = n_qc * n_rg;
   const int bh = logical / per_bh;
   const int idx = logical - bh * per_bh;
-  const int blk = idx / (kRgBlock * n_qc);
-  const int within = idx - blk * (kRgBlock * n_qc);
-  const int blk_rows = n_rg - blk * kRgBlock < kRgBlock ? n_rg - blk * kRgBlock : kRgBlock;  // the last block may be short
-  const int qc = within / blk_rows;
-  const int rg = blk * kRgBlock + (within - qc * blk_rows);
+  const int rb = idx / (kRgBlock * n_qc);
+  const int within = idx - rb * (kRgBlock * n_qc);
+  const int rows_here = n_rg - rb * kRgBlock < kRgBlock ? n_rg - rb * kRgBlock : kRgBlock;  // the last block may be short
+  const int qb = within / (rows_here * kQcBlock);
+  const int w2 = within - qb * (rows_here * kQcBlock);
+  const int qw = n_qc - qb * kQcBlock < kQcBlock ? n_qc - qb * kQcBlock : kQcBlock;
+  const int rg_local = w2 / qw;
+  const int qc = qb * kQcBlock + (w2 - rg_local * qw);
+  const int rg = rb * kRgBlock + rg_local;
   const int i_raw = rg * kRows + row;
   const bool row_valid = i_raw < N;  // wave-uniform; idle waves still take part in the loads and barriers
   const int i = row_valid ? i_raw : N - 1;
