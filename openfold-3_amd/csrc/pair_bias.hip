@@ -104,6 +104,18 @@ __global__ __launch_bounds__(512) void pair_bias_kernel(PairBiasArgs p, int tile
         }
         *reinterpret_cast<u32x4_t*>(dst) = o0;
         *reinterpret_cast<u32x4_t*>(dst + 8) = o1;
+      } else if (jl + 16 <= N) {
+        // rows of a length that is no multiple of 8 start at any even byte: pairs of positions from the
+        // first 4-byte boundary on (8 stores, or 1 + 7 + 1) instead of 16 single ones
+        const bool odd = (reinterpret_cast<uintptr_t>(dst) & 2) != 0;
+        if (odd) {
+          dst[0] = to_bf16(acc[0]);
+          dst[15] = to_bf16(acc[15]);
+        }
+        uint32_t* d32 = reinterpret_cast<uint32_t*>(dst + (odd ? 1 : 0));
+#pragma unroll
+        for (int q = 0; q < 7; ++q) d32[q] = odd ? pack_bf16(acc[2 * q + 1], acc[2 * q + 2]) : pack_bf16(acc[2 * q], acc[2 * q + 1]);
+        if (!odd) d32[7] = pack_bf16(acc[14], acc[15]);
       } else {
 #pragma unroll
         for (int v = 0; v < 16; ++v)
