@@ -120,11 +120,11 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
     int plane, tm, tn;
     tile_coords(t_local < my_tiles ? t_local : my_tiles - 1, plane, tm, tn);  // past the end: reload the last tile
     const size_t plane_off = (size_t)plane * Np * Np * 2;
-    const int rows_m_left = Np - tm * BM, rows_n_left = Np - tn * BN;
+    const int rows_m_left = 32 * nk - tm * BM, rows_n_left = 32 * nk - tn * BN;  // rows that hold tokens (>= 32)
 #pragma unroll
     for (int n = 0; n < MI; ++n) {
       const int rb = 16 * (wave * MI + n);
-      const int rbc = rb + 16 <= rows_m_left ? rb : rows_m_left - 16;  // whole blocks stay inside the plane
+      const int rbc = rb + 16 <= rows_m_left ? rb : rows_m_left - 16;  // padding rows: the last rows with tokens again (cache hits)
       dma_base[n] = reinterpret_cast<const char*>(pm) + plane_off + (size_t)(tm * BM + rbc) * (kBK * 2);
     }
 #pragma unroll
@@ -285,10 +285,12 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
         epi[l32 * 16 + ((chunk + 1) ^ (l32 & 7))] = hi;
         acc[mt][nt] = zero16();
       }
-      // Np is a multiple of 128, so a 32-row block and the wave's 128 columns are either
-      // entirely inside the plane or entirely outside: the guard is wave-uniform
+      // Only the rows and columns below Nr = 32 * nk (the tokens, rounded up to whole 32-blocks) are ever
+      // read: a 32-row block is entirely below it or entirely above (wave-uniform), the wave's 128 columns
+      // may straddle it (then the lanes decide, and the stores are not counted)
       const int i0 = tn * BN + wn0 + 32 * nt;
-      if (i0 < Np && jbase < Np) {
+      const int Nr = 32 * nk;
+      if (i0 < Nr && jbase + WM <= Nr) {
 #pragma unroll
         for (int rr = 0; rr < 8; ++rr) {
           const int row = 4 * rr + (lane >> 4), chunk = lane & 15;
@@ -296,6 +298,13 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
           *reinterpret_cast<u32x4_t*>(xo + (size_t)(i0 + row) * Np + jbase + 8 * chunk) = v;
         }
         n_stores += 8;
+      } else if (i0 < Nr && jbase < Nr) {
+#pragma unroll
+        for (int rr = 0; rr < 8; ++rr) {
+          const int row = 4 * rr + (lane >> 4), chunk = lane & 15;
+          const u32x4_t v = epi[row * 16 + (chunk ^ (row & 7))];
+          if (jbase + 8 * chunk < Nr) *reinterpret_cast<u32x4_t*>(xo + (size_t)(i0 + row) * Np + jbase + 8 * chunk) = v;
+        }
       }
       __builtin_amdgcn_sched_barrier(0);  // one block at a time keeps the live registers low
     }
@@ -404,12 +413,12 @@ __global__ __launch_bounds__(512, 1) void contract8_kernel(const bf16_t* __restr
     int plane, tm, tn;
     tile_coords(t_local < my_tiles ? t_local : my_tiles - 1, plane, tm, tn);  // past the end: reload the last tile
     const size_t plane_off = (size_t)plane * Np * Np * 2;
-    const int rows_m_left = Np - tm * BM, rows_n_left = Np - tn * BN;
+    const int rows_m_left = 32 * nk - tm * BM, rows_n_left = 32 * nk - tn * BN;  // rows that hold tokens (>= 32)
 #pragma unroll
     for (int n = 0; n < IPW_LO; ++n) {
       const int rb = block_row(n);
       const int left = n < MI ? rows_m_left : rows_n_left;
-      const int rbc = rb + 16 <= left ? rb : left - 16;  // whole blocks stay inside the plane
+      const int rbc = rb + 16 <= left ? rb : left - 16;  // padding rows: the last rows with tokens again (cache hits)
       const bf16_t* side = n < MI ? pm : pn;
       const int first = n < MI ? tm * BM : tn * BN;
       dma_base[n] = reinterpret_cast<const char*>(side) + plane_off + (size_t)(first + rbc) * (kBK * 2);
@@ -543,12 +552,13 @@ __global__ __launch_bounds__(512, 1) void contract8_kernel(const bf16_t* __restr
         acc[mt][nt] = zero16();
       }
       const int i0 = tn * BN + wn0 + 32 * nt;
-      const bool whole = i0 + 32 <= Np && jbase + WM <= Np;  // wave-uniform
+      const int Nr = 32 * nk;  // the tokens, rounded up to whole 32-blocks: nothing beyond is ever read
+      const bool whole = i0 + 32 <= Nr && jbase + WM <= Nr;  // wave-uniform
 #pragma unroll
       for (int rr = 0; rr < 6; ++rr) {
         const int idx = 64 * rr + lane, row = idx / 12, chunk = idx - 12 * row;
         const u32x4_t v = epi4[row * EPI_ROW + (chunk ^ ((row >> 2) & 3))];
-        if (whole || (i0 + row < Np && jbase + 8 * chunk < Np))
+        if (whole || (i0 + row < Nr && jbase + 8 * chunk < Nr))
           *reinterpret_cast<u32x4_t*>(xo + (size_t)(i0 + row) * Np + jbase + 8 * chunk) = v;
       }
       if (whole) n_stores += 6;
