@@ -204,6 +204,37 @@ def test_config5_n2048_modules_at_sampled_positions():
     _check("cfg5 tri_att_end", got, want, rms_rel=6e-3)
 
 
+@pytest.mark.parametrize("n,pad", [(1000, 0), (929, 37)])
+def test_ragged_large_n_modules_at_sampled_positions(n, pad):
+    """Token counts far from the multiples of 128 (ragged tiles in every pass, contraction tiles that hang
+    over the edge of the plane, a last key tile with few keys), at a size the CPU oracle only reaches at
+    sampled rows / fibres: first and last rows, the rows around the last whole 128-wide piece and around the
+    padded tail."""
+    lib()
+    c, heads, d = 128, 4, 32
+    p = _round_params(orc.make_block_params(31, c, c, d, heads))
+    stack = _load(of3pair.PairStack(c, c, d, heads), p)
+    z = orc.round_bf16(orc.make_pair_input(32, (), n, c))
+    mask = orc.tail_padding_mask((), n, pad)
+    zg = z.to(DEV).to(torch.bfloat16)[None]
+    mg = mask.to(DEV)[None]
+    last_full = 128 * (n // 128)
+    rows = sorted({0, 1, last_full - 1, last_full, n - pad - 1, n - 2, n - 1})
+    cols = sorted({0, 511, last_full - 1, last_full, last_full + 1, n - pad - 1, n - 1})
+    print("ragged n", n, "pad", pad, "rows", rows, flush=True)
+    for name, mod, outgoing in (("tri_mul_out", stack.tri_mul_out, True), ("tri_mul_in", stack.tri_mul_in, False)):
+        got = mod(zg, mask=mg)[0][rows][:, cols].float().cpu()
+        want = orc.trimul_update_at(z, mask, orc._sub(p, name + "."), outgoing, rows, cols)
+        _check("n=%d %s" % (n, name), got, want, rms_rel=6e-3)
+    got = stack.tri_att_start(zg, mask=mg)[0][rows].float().cpu()
+    want = orc.triattn_update_rows(z, mask, orc._sub(p, "tri_att_start."), heads, rows, starting=True)
+    _check("n=%d tri_att_start" % n, got, want, rms_rel=6e-3)
+    got = stack.tri_att_end(zg.transpose(-2, -3), mask=mg.transpose(-1, -2))[0][rows].float().cpu()
+    want = orc.triattn_update_rows(z.transpose(0, 1), mask.transpose(0, 1), orc._sub(p, "tri_att_end."), heads, rows,
+                                   starting=True)
+    _check("n=%d tri_att_end" % n, got, want, rms_rel=6e-3)
+
+
 def test_config5_four_blocks_run_in_place():
     """Config 5 end to end: 4 stacked blocks at N=2048 in place (1 GiB pair tensor).  Checked
     through size-independent properties: finite output, bitwise identical on a second run,
