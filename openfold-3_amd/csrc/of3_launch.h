@@ -3,6 +3,7 @@
 // with hipFuncSetAttribute and occupancy figures belong to the device that was current when
 // they were set or asked for.
 #pragma once
+#include "of3_tiles.h"
 
 #include <hip/hip_runtime.h>
 
@@ -32,23 +33,6 @@ inline hipError_t per_device(int (&cache)[kMaxDevices], Setup&& setup, int* out)
 
 inline hipError_t cu_count(int dev, int* n) {
   return hipDeviceGetAttribute(n, hipDeviceAttributeMultiprocessorCount, dev);
-}
-
-// 128-position tiles of the N x N positions of one batch element: the whole 128-wide pieces of every row
-// (full_per_row per row), then the remaining N % 128 columns in pieces of 2^tail_shift columns (the
-// smallest power of two >= 2^min_shift that covers them) x (128 >> tail_shift) consecutive rows.
-struct RaggedTiles {
-  int full_per_row, tail_shift, per_batch;
-};
-inline RaggedTiles ragged_tiles(int N, int min_shift = 3) {
-  RaggedTiles t;
-  t.full_per_row = N / 128;
-  const int r = N % 128;
-  t.tail_shift = r ? min_shift : 7;
-  while ((1 << t.tail_shift) < r) ++t.tail_shift;
-  const int rows = 128 >> t.tail_shift;
-  t.per_batch = N * t.full_per_row + (r ? (N + rows - 1) / rows : 0);
-  return t;
 }
 
 // work-groups of `threads` threads (no dynamic LDS) that fit the device at once

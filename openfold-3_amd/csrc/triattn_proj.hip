@@ -92,23 +92,11 @@ __global__ __launch_bounds__(64 * NW) void triattn_proj_kernel(TriattnProjArgs p
   const float qscale = kLog2e * __builtin_amdgcn_rsqf((float)D);
 
   const int N = p.N, Jp = p.Jp;
-  // tile -> batch element, first row, first column, log2 of the width (wave-uniform); position pos of the
-  // tile is row i0 + (pos >> shift), column j0 + (pos & (width - 1)); without ragged pieces shift is 7
-  const int main_tiles = N * full_per_row;
+  // tile -> batch element, first row, first column, log2 of the width (wave-uniform); the last ragged piece
+  // is moved up to end at the last row, so every row of a tile exists (the launcher makes sure that N >= 4)
   auto tile_origin = [&](int tile_id, int& b, int& i0, int& j0, int& shift) {
-    b = tile_id / tiles_per_batch;
-    const int rem = tile_id - b * tiles_per_batch;
-    if (!RAGGED || rem < main_tiles) {
-      i0 = rem / full_per_row;
-      j0 = (rem - i0 * full_per_row) * TP;
-      shift = 7;
-    } else {
-      const int rows = TP >> tail_shift;
-      i0 = (rem - main_tiles) * rows;
-      i0 = i0 + rows <= N ? i0 : N - rows;  // the launcher makes sure that N >= rows
-      j0 = full_per_row * TP;
-      shift = tail_shift;
-    }
+    const TilePlace t = tile_place<RAGGED>(tile_id, N, full_per_row, tail_shift, tiles_per_batch, true);
+    b = t.b, i0 = t.i0, j0 = t.j0, shift = t.shift;
   };
 
   u32x4_t raw[LN_ITERS];

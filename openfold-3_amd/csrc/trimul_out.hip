@@ -66,21 +66,11 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int fu
   }
 
   const int N = p.N, Np = p.Np;
-  const int main_tiles = N * full_per_row;  // per batch element
-  // tile -> batch element, first row, first column, log2 of its width (all wave-uniform); position pos of
-  // the tile is row i0 + (pos >> shift), column j0 + (pos & (width - 1))
+  // tile -> batch element, first row, first column, log2 of its width (all wave-uniform); the last ragged
+  // piece may run past the last row: those positions are left out below
   auto tile_origin = [&](int tile_id, int& b, int& i0, int& j0, int& shift) {
-    b = tile_id / tiles_per_batch;
-    const int rem = tile_id - b * tiles_per_batch;
-    if (!RAGGED || rem < main_tiles) {  // N a multiple of 128: whole-row pieces only
-      i0 = rem / full_per_row;
-      j0 = (rem - i0 * full_per_row) * TP;
-      shift = 7;
-    } else {
-      i0 = (rem - main_tiles) * (TP >> tail_shift);
-      j0 = full_per_row * TP;
-      shift = tail_shift;
-    }
+    const TilePlace t = tile_place<RAGGED>(tile_id, N, full_per_row, tail_shift, tiles_per_batch, false);
+    b = t.b, i0 = t.i0, j0 = t.j0, shift = t.shift;
   };
   uint32_t* xt32 = reinterpret_cast<uint32_t*>(xtile);
 
