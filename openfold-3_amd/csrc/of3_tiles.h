@@ -57,4 +57,66 @@ OF3_HD inline TilePlace tile_place(int tile_id, int N, int full_per_row, int tai
   return t;
 }
 
+// ---- tiles of 128 consecutive positions of the flattened [B][N][N] index space (triattn_out) -----------
+// A tile starts at position p0 = 128 * tile_id = (b0, i0, j0).  MODE 0: N is a multiple of 128, a tile lies
+// inside one row; 1: N >= 128, at most two rows, whose element offsets in the strided view are row0 and row1;
+// 2: any N, the general walk.
+struct FlatTile {
+  int b0, i0, j0;
+  long long row0, row1;
+};
+OF3_HD inline FlatTile flat_tile(int tile_id, int N, long long stride_b, long long stride_r) {
+  FlatTile t;
+  const unsigned p0 = (unsigned)tile_id * 128u, nn = (unsigned)N * (unsigned)N;
+  t.b0 = (int)(p0 / nn);
+  const unsigned rem = p0 - (unsigned)t.b0 * nn;
+  t.i0 = (int)(rem / (unsigned)N);
+  t.j0 = (int)(rem - (unsigned)t.i0 * (unsigned)N);
+  const bool last = t.i0 + 1 == N;
+  t.row0 = t.b0 * stride_b + t.i0 * stride_r;
+  t.row1 = (t.b0 + (last ? 1 : 0)) * stride_b + (last ? 0 : t.i0 + 1) * stride_r;
+  return t;
+}
+// element offset of position d (0..127) of the tile in the view; the position must exist
+template <int MODE>
+OF3_HD inline long long flat_offset(const FlatTile& t, int d, int N, long long stride_b, long long stride_r,
+                                    long long stride_k) {
+  int j = t.j0 + d;
+  if (MODE == 0) {
+    return t.row0 + j * stride_k;
+  } else if (MODE == 1) {
+    const bool wrapped = j >= N;
+    j -= wrapped ? N : 0;
+    return (wrapped ? t.row1 : t.row0) + j * stride_k;
+  } else {
+    int b = t.b0, i = t.i0;
+    while (j >= N) j -= N, ++i;  // at most once when N >= 128
+    while (i >= N) i -= N, ++b;
+    return b * stride_b + i * stride_r + j * stride_k;
+  }
+}
+
+// ---- order of the attention core's work-groups -----------------------------------------------------------
+// Work items of one (batch element, head) are (query range qc < n_qc, row group rg < n_rg).  They are taken in
+// blocks of RB row groups x QB query ranges; inside a block the query range runs fastest, then the row group.
+struct FlashItem {
+  int bh, qc, rg;
+};
+OF3_HD inline FlashItem flash_item(int logical, int n_qc, int n_rg, int RB, int QB) {
+  FlashItem w;
+  const int per_bh = n_qc * n_rg;
+  w.bh = logical / per_bh;
+  const int idx = logical - w.bh * per_bh;
+  const int rb = idx / (RB * n_qc);
+  const int within = idx - rb * (RB * n_qc);
+  const int rows_here = n_rg - rb * RB < RB ? n_rg - rb * RB : RB;  // the last block of row groups may be short
+  const int qb = within / (rows_here * QB);
+  const int w2 = within - qb * (rows_here * QB);
+  const int qw = n_qc - qb * QB < QB ? n_qc - qb * QB : QB;        // and so may the last block of query ranges
+  const int rg_local = w2 / qw;
+  w.qc = qb * QB + (w2 - rg_local * qw);
+  w.rg = rb * RB + rg_local;
+  return w;
+}
+
 }  // namespace of3

@@ -139,18 +139,8 @@ __global__ __launch_bounds__(64 * kRows * QW, kRQ == 1 ? 6 : 4) void triattn_fla
   // row group's K / V^T tiles by its query ranges, a query range's bias slice by the row groups.  With
   // kQcBlock query ranges or fewer (N <= 1024) this is simply: all query ranges of a row group, then the
   // next row group.
-  const int per_bh = n_qc * n_rg;
-  const int bh = logical / per_bh;
-  const int idx = logical - bh * per_bh;
-  const int rb = idx / (kRgBlock * n_qc);
-  const int within = idx - rb * (kRgBlock * n_qc);
-  const int rows_here = n_rg - rb * kRgBlock < kRgBlock ? n_rg - rb * kRgBlock : kRgBlock;  // the last block may be short
-  const int qb = within / (rows_here * kQcBlock);
-  const int w2 = within - qb * (rows_here * kQcBlock);
-  const int qw = n_qc - qb * kQcBlock < kQcBlock ? n_qc - qb * kQcBlock : kQcBlock;
-  const int rg_local = w2 / qw;
-  const int qc = qb * kQcBlock + (w2 - rg_local * qw);
-  const int rg = rb * kRgBlock + rg_local;
+  const FlashItem item = flash_item(logical, n_qc, n_rg, kRgBlock, kQcBlock);  // of3_tiles.h
+  const int bh = item.bh, qc = item.qc, rg = item.rg;
   const int i_raw = rg * kRows + row;
   const bool row_valid = i_raw < N;  // wave-uniform; idle waves still take part in the loads and barriers
   const int i = row_valid ? i_raw : N - 1;

@@ -58,42 +58,13 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, uint
   }
 
   const int N = p.N;
-  // A tile starts at position p0 = (b0, i0, j0) (wave-uniform: scalar divisions).  With N >= 128 it holds
-  // positions of at most two rows, whose offsets in the view are the scalars row0 and row1; position d of
-  // the tile then costs a compare and two selects.  Smaller N: the general walk.
-  struct Origin {
-    int b0, i0, j0;
-    int64_t row0, row1;
-  };
-  // MODE 0: N is a multiple of 128, a tile lies inside one row; 1: N >= 128, at most two rows; 2: any N
-  constexpr bool two_rows = MODE == 1, one_row = MODE == 0;
-  auto tile_origin = [&](int tile_id) {
-    Origin t;
-    const uint32_t p0 = (uint32_t)tile_id * TP, nn = (uint32_t)N * (uint32_t)N;
-    t.b0 = (int)(p0 / nn);
-    const uint32_t rem = p0 - (uint32_t)t.b0 * nn;
-    t.i0 = (int)(rem / (uint32_t)N);
-    t.j0 = (int)(rem - (uint32_t)t.i0 * (uint32_t)N);
-    const bool last = t.i0 + 1 == N;
-    t.row0 = t.b0 * p.x_view.stride_b + t.i0 * p.x_view.stride_r;
-    t.row1 = (t.b0 + (last ? 1 : 0)) * p.x_view.stride_b + (last ? 0 : t.i0 + 1) * p.x_view.stride_r;
-    return t;
-  };
-  // element offset of position d of the tile in the x / out view (the position must exist)
+  // A tile starts at position p0 = (b0, i0, j0) (wave-uniform: scalar divisions); with N >= 128 it holds
+  // positions of at most two rows, whose offsets in the view are scalars, and position d of the tile costs a
+  // compare and two selects (of3_tiles.h).
+  typedef FlatTile Origin;
+  auto tile_origin = [&](int tile_id) { return flat_tile(tile_id, N, p.x_view.stride_b, p.x_view.stride_r); };
   auto view_offset = [&](const Origin& t, int d) -> int64_t {
-    int j = t.j0 + d;
-    if constexpr (one_row) {
-      return t.row0 + j * p.x_view.stride_k;
-    } else if constexpr (two_rows) {
-      const bool wrapped = j >= N;
-      j -= wrapped ? N : 0;
-      return (wrapped ? t.row1 : t.row0) + j * p.x_view.stride_k;
-    } else {
-      int b = t.b0, i = t.i0;
-      while (j >= N) j -= N, ++i;
-      while (i >= N) i -= N, ++b;
-      return b * p.x_view.stride_b + i * p.x_view.stride_r + j * p.x_view.stride_k;
-    }
+    return flat_offset<MODE>(t, d, N, p.x_view.stride_b, p.x_view.stride_r, p.x_view.stride_k);
   };
 
   // The loads of a tile are issued one tile ahead (right after the previous tile's values have

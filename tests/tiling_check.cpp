@@ -77,11 +77,55 @@ static int check_input_pass(int N, int B) {
   return 0;
 }
 
+// triattn_out: tiles of 128 consecutive positions of the flattened [B][N][N] index space; the offset of a
+// position in a strided view (plain and transposed) must be that of its (b, i, j)
+static int check_flat_pass(int N, int B) {
+  const long long C = 128;
+  for (int transposed = 0; transposed < 2; ++transposed) {
+    const long long sb = (long long)N * N * C, sr = transposed ? C : N * C, sk = transposed ? N * C : C;
+    const long long total = (long long)B * N * N;
+    const int tiles = (int)((total + 127) / 128);
+    std::vector<char> seen((size_t)total, 0);
+    for (int tile = 0; tile < tiles; ++tile) {
+      const FlatTile t = flat_tile(tile, N, sb, sr);
+      for (int d = 0; d < 128; ++d) {
+        const long long p = (long long)tile * 128 + d;
+        if (p >= total) continue;
+        const int b = (int)(p / ((long long)N * N)), i = (int)(p / N % N), j = (int)(p % N);
+        const long long want = b * sb + i * sr + j * sk;
+        const long long got = N % 128 == 0 ? flat_offset<0>(t, d, N, sb, sr, sk)
+                              : (N >= 128 ? flat_offset<1>(t, d, N, sb, sr, sk) : flat_offset<2>(t, d, N, sb, sr, sk));
+        if (got != want || got < 0 || got + C > B * sb) return fail("flat offset", N, tile, d);
+        seen[(size_t)p] = 1;
+      }
+    }
+    for (long long p = 0; p < total; ++p)
+      if (!seen[(size_t)p]) return fail("flat position not visited", N, (int)p, 0);
+  }
+  return 0;
+}
+
+// attention core: the order of the work-groups is a one-to-one map onto (head, query range, row group)
+static int check_flash_order(int N) {
+  const int n_qc = (N + 127) / 128, n_rg = (N + 3) / 4, BH = 3;
+  std::vector<char> seen((size_t)BH * n_qc * n_rg, 0);
+  for (int logical = 0; logical < BH * n_qc * n_rg; ++logical) {
+    const FlashItem w = flash_item(logical, n_qc, n_rg, 8, 8);
+    if (w.bh < 0 || w.bh >= BH || w.qc < 0 || w.qc >= n_qc || w.rg < 0 || w.rg >= n_rg) return fail("flash item", N, logical, 0);
+    char& s = seen[((size_t)w.bh * n_qc + w.qc) * n_rg + w.rg];
+    if (s) return fail("flash item taken twice", N, logical, 0);
+    s = 1;
+    // with eight query ranges or fewer the order is the plain one
+    if (n_qc <= 8 && (w.qc != logical % n_qc || w.rg != logical / n_qc % n_rg)) return fail("flash plain order", N, logical, 0);
+  }
+  return 0;
+}
+
 int main(int argc, char** argv) {
   for (int a = 1; a < argc; ++a) {
     const int N = std::atoi(argv[a]);
     if (N < 1) return 2;
-    if (check_output_pass(N, 2) || check_input_pass(N, 2)) return 1;
+    if (check_output_pass(N, 2) || check_input_pass(N, 2) || check_flat_pass(N, 2) || check_flash_order(N)) return 1;
     std::printf("ok %d\n", N);
   }
   return 0;
