@@ -119,4 +119,13 @@ OF3_HD inline FlashItem flash_item(int logical, int n_qc, int n_rg, int RB, int 
   return w;
 }
 
+// ---- contraction: rows a direct-to-LDS instruction brings in -------------------------------------------
+// A tile's operand rows start at tile_first; an instruction covers the 16 rows from tile_first + rb on.  Rows
+// from `token_rows` (the tokens, rounded up to whole 32-blocks) on are padding: such a block takes the last 16
+// rows with tokens instead (lines the caches already hold), wherever the tile lies.  Returns the first row.
+OF3_HD inline int contract_rows_first(int tile_first, int rb, int token_rows) {
+  const int left = token_rows - tile_first;  // may be zero or less for a tile that lies in the padding
+  return tile_first + (rb + 16 <= left ? rb : left - 16);
+}
+
 }  // namespace of3

@@ -120,18 +120,16 @@ __global__ __launch_bounds__(256, 1) void contract_kernel(const bf16_t* __restri
     int plane, tm, tn;
     tile_coords(t_local < my_tiles ? t_local : my_tiles - 1, plane, tm, tn);  // past the end: reload the last tile
     const size_t plane_off = (size_t)plane * Np * Np * 2;
-    const int rows_m_left = 32 * nk - tm * BM, rows_n_left = 32 * nk - tn * BN;  // rows that hold tokens (>= 32)
+    // blocks of padding rows take the last rows with tokens again (of3_tiles.h)
 #pragma unroll
     for (int n = 0; n < MI; ++n) {
-      const int rb = 16 * (wave * MI + n);
-      const int rbc = rb + 16 <= rows_m_left ? rb : rows_m_left - 16;  // padding rows: the last rows with tokens again (cache hits)
-      dma_base[n] = reinterpret_cast<const char*>(pm) + plane_off + (size_t)(tm * BM + rbc) * (kBK * 2);
+      const int row = contract_rows_first(tm * BM, 16 * (wave * MI + n), 32 * nk);
+      dma_base[n] = reinterpret_cast<const char*>(pm) + plane_off + (size_t)row * (kBK * 2);
     }
 #pragma unroll
     for (int n = 0; n < NI; ++n) {
-      const int rb = 16 * (wave * NI + n);
-      const int rbc = rb + 16 <= rows_n_left ? rb : rows_n_left - 16;
-      dma_base[MI + n] = reinterpret_cast<const char*>(pn) + plane_off + (size_t)(tn * BN + rbc) * (kBK * 2);
+      const int row = contract_rows_first(tn * BN, 16 * (wave * NI + n), 32 * nk);
+      dma_base[MI + n] = reinterpret_cast<const char*>(pn) + plane_off + (size_t)row * (kBK * 2);
     }
     issue_kb = ((tm + tn) & 3) % nk;  // rotated start (a small spread keeps the sharers' lines in L2)
     issue_left = nk;
@@ -413,15 +411,12 @@ __global__ __launch_bounds__(512, 1) void contract8_kernel(const bf16_t* __restr
     int plane, tm, tn;
     tile_coords(t_local < my_tiles ? t_local : my_tiles - 1, plane, tm, tn);  // past the end: reload the last tile
     const size_t plane_off = (size_t)plane * Np * Np * 2;
-    const int rows_m_left = 32 * nk - tm * BM, rows_n_left = 32 * nk - tn * BN;  // rows that hold tokens (>= 32)
+    // blocks of padding rows take the last rows with tokens again (of3_tiles.h)
 #pragma unroll
     for (int n = 0; n < IPW_LO; ++n) {
-      const int rb = block_row(n);
-      const int left = n < MI ? rows_m_left : rows_n_left;
-      const int rbc = rb + 16 <= left ? rb : left - 16;  // padding rows: the last rows with tokens again (cache hits)
       const bf16_t* side = n < MI ? pm : pn;
-      const int first = n < MI ? tm * BM : tn * BN;
-      dma_base[n] = reinterpret_cast<const char*>(side) + plane_off + (size_t)(first + rbc) * (kBK * 2);
+      const int row = contract_rows_first(n < MI ? tm * BM : tn * BN, block_row(n), 32 * nk);
+      dma_base[n] = reinterpret_cast<const char*>(side) + plane_off + (size_t)row * (kBK * 2);
     }
     issue_kb = ((tm + tn) & 3) % nk;
     issue_left = nk;

@@ -121,11 +121,28 @@ static int check_flash_order(int N) {
   return 0;
 }
 
+// contraction: whatever the tile shape, every load instruction's 16 rows lie below the last row with tokens
+static int check_contract_rows(int N) {
+  const int Np = (N + 127) / 128 * 128, token_rows = (N + 31) / 32 * 32;
+  const int shapes[4][2] = {{256, 192}, {256, 128}, {256, 256}, {384, 192}};
+  for (const auto& sh : shapes)
+    for (int side = 0; side < 2; ++side) {
+      const int T = sh[side];
+      for (int first = 0; first < Np; first += T)
+        for (int rb = 0; rb < T; rb += 16) {
+          const int row = contract_rows_first(first, rb, token_rows);
+          if (row < 0 || row + 16 > token_rows || token_rows > Np) return fail("contraction rows", N, first, rb);
+          if (first + rb + 16 <= token_rows && row != first + rb) return fail("contraction rows moved", N, first, rb);
+        }
+    }
+  return 0;
+}
+
 int main(int argc, char** argv) {
   for (int a = 1; a < argc; ++a) {
     const int N = std::atoi(argv[a]);
     if (N < 1) return 2;
-    if (check_output_pass(N, 2) || check_input_pass(N, 2) || check_flat_pass(N, 2) || check_flash_order(N)) return 1;
+    if (check_output_pass(N, 2) || check_input_pass(N, 2) || check_flat_pass(N, 2) || check_flash_order(N) || check_contract_rows(N)) return 1;
     std::printf("ok %d\n", N);
   }
   return 0;
