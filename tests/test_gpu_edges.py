@@ -32,6 +32,31 @@ def test_block_small_and_ragged_sizes(n):
     _check("block n=%d" % n, got, want, rms_rel=1.2e-2)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_block_random_ragged_shapes(seed):
+    """Seeded random token counts (every width of the ragged row ends: 8, 16, 32, 64 and 128 columns),
+    batch sizes, both channel widths, random and tail-padding masks; out of place and in place."""
+    lib()
+    gen = torch.Generator().manual_seed(9000 + seed)
+    wide = seed % 2 == 0
+    c, d = (128, 32) if wide else (64, 16)
+    n = int(torch.randint(3, 190, (1,), generator=gen)) if seed < 6 else (int(torch.randint(129, 140, (1,), generator=gen)) if seed == 6 else 161)
+    b = int(torch.randint(1, 4, (1,), generator=gen))
+    m, p = _block(c, d, seed=9100 + seed)
+    z = orc.round_bf16(torch.randn(b, n, n, c, generator=gen))
+    if seed % 3 == 0:
+        mask = orc.tail_padding_mask((b,), n, torch.randint(0, max(1, n // 4), (b,), generator=gen))
+    else:
+        mask = (torch.rand(b, n, n, generator=gen) > 0.2).float()
+    print("random ragged block: seed", seed, "c", c, "n", n, "batch", b, flush=True)
+    zg = z.to(DEV).to(torch.bfloat16)
+    want = orc.pair_stack_block(z, mask, p, 4)
+    got = m(zg, mask.to(DEV))
+    _check("random block seed %d n=%d" % (seed, n), got, want, rms_rel=1.2e-2)
+    res = m(zg, mask.to(DEV), inplace_safe=True)
+    assert res.data_ptr() == zg.data_ptr() and torch.equal(res, got), "in place and out of place differ"
+
+
 def test_fully_masked_input():
     """mask == 0 everywhere: trimul contributes (LN_out.bias Wz^T)*gate, attention averages v uniformly."""
     lib()
