@@ -235,6 +235,40 @@ def test_ragged_large_n_modules_at_sampled_positions(n, pad):
     _check("n=%d tri_att_end" % n, got, want, rms_rel=6e-3)
 
 
+def test_n4096_modules_at_sampled_positions():
+    """Twice the token count of the largest benchmark configuration (a 4.3 GB pair tensor, 64-bit offsets in
+    every intermediate): each module against the oracle at sampled rows / fibres, then one block in place."""
+    lib()
+    n, pad, c, heads, d = 4096, 100, 128, 4, 32
+    p = _round_params(orc.make_block_params(5, c, c, d, heads))
+    stack = _load(of3pair.PairStack(c, c, d, heads), p)
+    z = orc.round_bf16(orc.make_pair_input(6, (), n, c))
+    mask = orc.tail_padding_mask((), n, pad)
+    zg = z.to(DEV).to(torch.bfloat16)[None]
+    mg = mask.to(DEV)[None]
+    rows = [0, 1, n // 2 - 1, n - pad - 1, n - 1]
+    cols = [0, 511, n // 2, n - pad - 1, n - 2, n - 1]
+    print("n = 4096: trimul", flush=True)
+    for name, mod, outgoing in (("tri_mul_out", stack.tri_mul_out, True), ("tri_mul_in", stack.tri_mul_in, False)):
+        got = mod(zg, mask=mg)[0][rows][:, cols].float().cpu()
+        want = orc.trimul_update_at(z, mask, orc._sub(p, name + "."), outgoing, rows, cols)
+        _check("n=4096 " + name, got, want, rms_rel=6e-3)
+    print("n = 4096: triangle attention", flush=True)
+    got = stack.tri_att_start(zg, mask=mg)[0][rows].float().cpu()
+    want = orc.triattn_update_rows(z, mask, orc._sub(p, "tri_att_start."), heads, rows, starting=True)
+    _check("n=4096 tri_att_start", got, want, rms_rel=6e-3)
+    got = stack.tri_att_end(zg.transpose(-2, -3), mask=mg.transpose(-1, -2))[0][rows].float().cpu()
+    want = orc.triattn_update_rows(z.transpose(0, 1), mask.transpose(0, 1), orc._sub(p, "tri_att_end."), heads, rows,
+                                   starting=True)
+    _check("n=4096 tri_att_end", got, want, rms_rel=6e-3)
+    del got, want, z
+    res = stack(zg, mg, inplace_safe=True)
+    assert res.data_ptr() == zg.data_ptr() and torch.isfinite(res.float()).all()
+    del res, zg
+    of3pair.functional.release_workspaces()
+    torch.cuda.empty_cache()
+
+
 def test_config5_four_blocks_run_in_place():
     """Config 5 end to end: 4 stacked blocks at N=2048 in place (1 GiB pair tensor).  Checked
     through size-independent properties: finite output, bitwise identical on a second run,
