@@ -91,6 +91,9 @@ __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcp
 __device__ __forceinline__ float sigmoidf_fast(float x) {
   return fast_rcp(1.f + fast_exp2(-kLog2e * x));
 }
+// sigmoid(x) from t = -log2(e) * x, for the passes whose normalised activations feed nothing but a gate:
+// they fold the factor into the LayerNorm's weight and bias, and the gate's matrix product delivers t
+__device__ __forceinline__ float sigmoid_from_scaled(float t) { return fast_rcp(1.f + fast_exp2(t)); }
 
 // all-reduce (sum) over the LPP (8 or 16) consecutive lanes that share one position, with
 // DPP lane permutations (no LDS round trips): xor 1 and xor 2 inside each quad, then

@@ -41,9 +41,13 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, uint
   const int lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
   const int ln_chunk = lane % LPP, ln_pp = lane / LPP;
 
+  // LayerNorm(x) feeds the gate only: its weight and bias carry the factor -log2(e) of the gate's
+  // base-2 exponential, one multiplication per gate value less
   float lw[8], lb[8];
   load_affine8(p.ln_w, ln_chunk, lw);
   load_affine8(p.ln_b, ln_chunk, lb);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) lw[e] *= -kLog2e, lb[e] *= -kLog2e;
 
   const int ot = wave % NOT;
   const int t0 = (wave / NOT) * TPW;
@@ -116,7 +120,7 @@ __global__ __launch_bounds__(512) void triattn_out_kernel(TriattnOutArgs p, uint
         float ov[8];
         unpack8(otile[slot], ov);
 #pragma unroll
-        for (int v = 0; v < 8; ++v) ov[v] *= sigmoidf_fast(acc[8 * half + v]);
+        for (int v = 0; v < 8; ++v) ov[v] *= sigmoid_from_scaled(acc[8 * half + v]);
         otile[slot] = pack8(ov);
       }
     }

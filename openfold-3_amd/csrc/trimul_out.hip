@@ -50,6 +50,10 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int fu
   load_affine8(p.ln_in_b, ln_chunk, ib);
   load_affine8(p.ln_out_w, ln_chunk, ow);
   load_affine8(p.ln_out_b, ln_chunk, ob);
+  // LayerNorm_in(z) feeds the gate only: its weight and bias carry the factor -log2(e) of the gate's
+  // base-2 exponential, one multiplication per gate value less
+#pragma unroll
+  for (int e = 0; e < 8; ++e) iw[e] *= -kLog2e, ib[e] *= -kLog2e;
 
   // A operands: logical output channel of A-row r is 32*ot + rowperm16(r), so that a lane
   // ends up with the 16 consecutive channels 32*ot + 16*lh + v
@@ -165,7 +169,7 @@ __global__ __launch_bounds__(512) void trimul_out_kernel(TrimulOutArgs p, int fu
         const int64_t off = di * p.z_view.stride_r + j * p.z_view.stride_k + 32 * ot + 16 * lh;
         float res[16];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) res[v] = accu[v] * sigmoidf_fast(accg[v]);
+        for (int v = 0; v < 16; ++v) res[v] = accu[v] * sigmoid_from_scaled(accg[v]);
         if (p.add_residual) {
           const u32x4_t r0 = rtile[tile_slot<NCH, 0>(pos, 4 * ot + 2 * lh)];
           const u32x4_t r1 = rtile[tile_slot<NCH, 0>(pos, 4 * ot + 2 * lh + 1)];
