@@ -168,6 +168,17 @@ def test_shapes_beyond_32_bit_position_counts_are_refused(lib):
     assert lib.of3_trimul_contract_variant(1, 768, 96) == _lib.OF3_EINVAL
 
 
+def test_contract_variant_choice_follows_the_measured_table(lib):
+    """Tile variant per token count on 256 compute units (the count the library assumes without a device):
+    at each of these sizes the choice is the variant that was fastest inside the block on an MI355X
+    (1: 256 x 192, 2: 256 x 128, 3: 256 x 256, 4: 384 x 192 tiles)."""
+    measured_best = {256: 2, 320: 4, 448: 3, 512: 3, 576: 4, 640: 4, 700: 4, 768: 4, 769: 3, 800: 3, 850: 3,
+                     900: 3, 960: 3, 1000: 3, 1100: 4, 1280: 3, 2048: 3}
+    got = {n: lib.of3_trimul_contract_variant(1, n, 128) for n in measured_best}
+    assert got == measured_best
+    assert lib.of3_trimul_contract_variant(4, 512, 64) == 3  # the template stack: 256 planes of 512 x 512
+
+
 def test_check_maps_status_to_exceptions(lib):
     from of3pair import _lib
 
